@@ -1,0 +1,398 @@
+// Row-wise and element-wise kernels for gfx950: embedding gather, RMSNorm,
+// SwiGLU, the fused QK-norm + rotary + cache write, dtype casts, and the
+// sampling kernels (argmax, temperature). All arithmetic is float32; only
+// loads and stores convert. One C entry point per operation.
+#include "common.h"
+
+#include <math.h>
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = float(table[ids[t], :]). Reference: src/backend/cpu/cpu_backend.cpp:51-76.
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                             int D) {
+  const int t = blockIdx.x;
+  const TW* row = table + static_cast<size_t>(ids[t]) * D;
+  float* o = out + static_cast<size_t>(t) * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) o[d] = load_as_float(row + d);
+}
+
+extern "C" int tie_embed(const void* table, int table_dtype, const int* ids, float* out, int T, int D,
+                         hipStream_t stream) {
+  if (T <= 0 || D <= 0) return TIE_BAD_ARGUMENT;
+  const int threads = D >= 1024 ? 256 : 64;
+  if (table_dtype == TIE_F32) {
+    embed_kernel<float><<<T, threads, 0, stream>>>(static_cast<const float*>(table), ids, out, D);
+  } else if (table_dtype == TIE_BF16) {
+    embed_kernel<bf16_t><<<T, threads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, D);
+  } else {
+    return TIE_BAD_ARGUMENT;
+  }
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// out[r, i] = (x[src(r), i] * inv) * w[i], inv = 1 / sqrt(mean(x^2) + eps), src(r) = rows ? rows[r] : r.
+// Reference: src/backend/cpu/cpu_backend.cpp:141-159 (weight multiplies after normalisation).
+template <typename TX, typename TO>
+__global__ void rms_norm_kernel(const TX* __restrict__ x, const float* __restrict__ w, float eps,
+                                TO* __restrict__ out, const int* __restrict__ rows, int n) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const TX* xr = x + static_cast<size_t>(rows ? rows[r] : r) * n;
+  TO* o = out + static_cast<size_t>(r) * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = load_as_float(xr + i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    store_from_float(o + i, (load_as_float(xr + i) * inv) * w[i]);
+  }
+}
+
+extern "C" int tie_rms_norm(const void* x, int x_dtype, const float* w, float eps, void* out, int out_dtype,
+                            const int* rows, int R, int n, hipStream_t stream) {
+  if (R <= 0 || n <= 0) return TIE_BAD_ARGUMENT;
+  const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
+#define LAUNCH(TX, TO)                                                                                   \
+  rms_norm_kernel<TX, TO><<<R, threads, 0, stream>>>(static_cast<const TX*>(x), w, eps, static_cast<TO*>(out), \
+                                                     rows, n)
+  if (x_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float);
+  else if (x_dtype == TIE_F32 && out_dtype == TIE_BF16) LAUNCH(float, bf16_t);
+  else if (x_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(bf16_t, float);
+  else if (x_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t);
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------- SwiGLU
+// gate_up is [T, 2I] with the gate in columns [0, I) and up in [I, 2I).
+// out[t, i] = gate / (1 + exp(-gate)) * up, left to right. Reference: cpu_backend.cpp:195-207.
+template <typename TX, typename TO>
+__global__ void swiglu_kernel(const TX* __restrict__ gate_up, TO* __restrict__ out, int I) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const TX* row = gate_up + static_cast<size_t>(t) * 2 * I;
+  const float g = load_as_float(row + i);
+  const float u = load_as_float(row + I + i);
+  store_from_float(out + static_cast<size_t>(t) * I + i, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int T, int I,
+                          hipStream_t stream) {
+  if (T <= 0 || I <= 0 || T > 65535 * 64) return TIE_BAD_ARGUMENT;
+  const dim3 grid((I + 255) / 256, T);
+#define LAUNCH(TX, TO) \
+  swiglu_kernel<TX, TO><<<grid, 256, 0, stream>>>(static_cast<const TX*>(gate_up), static_cast<TO*>(out), I)
+  if (in_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float);
+  else if (in_dtype == TIE_F32 && out_dtype == TIE_BF16) LAUNCH(float, bf16_t);
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(bf16_t, float);
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// --------------------------------------------------------------------- cast
+template <typename TX, typename TO>
+__global__ void cast_kernel(const TX* __restrict__ x, TO* __restrict__ out, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) store_from_float(out + i, load_as_float(x + i));
+}
+
+extern "C" int tie_cast(const void* x, int in_dtype, void* out, int out_dtype, long long n, hipStream_t stream) {
+  if (n <= 0) return TIE_BAD_ARGUMENT;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  if (in_dtype == TIE_F32 && out_dtype == TIE_BF16)
+    cast_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const float*>(x), static_cast<bf16_t*>(out), n);
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32)
+    cast_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<float*>(out), n);
+  else
+    return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}
+
+// ------------------------------------------ QK-norm + rotary + cache write
+// One wave per (token, head slot). Head slots 0..H-1 are query heads, then KVH
+// key heads, then KVH value heads of the fused projection row
+// qkv[t] = [q (H*Dh) | k (KVH*Dh) | v (KVH*Dh)], in_row elements apart from the next token's.
+//   q, k: per-head RMSNorm over Dh with one weight vector shared by all heads,
+//         THEN rotate-half rotary: pairs (i, i + Dh/2), angle = float(pos) * inv_freq[i]
+//         (reference: src/model/qwen3.cpp:222-225, cpu_backend.cpp:161-193, backend/rope.h:9-13).
+//   q goes to q_out[t * q_row + h*Dh + d]; k (after norm and rotation) and raw v go to the
+//   paged cache at ((page*KVH + h)*block_size + offset)*Dh + d with page = slot / block_size,
+//   offset = slot % block_size (cpu_backend.cpp:235-259).
+// Norm weights or inv_freq may be null: that step is then skipped. With k_dense set, keys are
+// written there (row stride k_row) instead of into the cache; without write_kv and k_dense only
+// the query heads are processed. q_out and k_dense may alias qkv (each wave holds its head in
+// registers before it writes).
+#define TIE_MAX_PAIRS 4  // head_dim <= 512
+
+template <typename TX, typename TQ, typename TC>
+__global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
+                                             const float* __restrict__ k_w, float eps,
+                                             const float* __restrict__ inv_freq,
+                                             const int* __restrict__ positions, const int* __restrict__ slots,
+                                             TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
+                                             int KVH, int Dh, int block_size, int in_row, int q_row, int k_row) {
+  const int t = blockIdx.y;
+  const int slot_index = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int half = Dh / 2;
+  const TX* in = qkv + static_cast<size_t>(t) * in_row + static_cast<size_t>(slot_index) * Dh;
+
+  const bool is_q = slot_index < H;
+  const bool is_k = !is_q && slot_index < H + KVH;
+
+  if (!is_q && !is_k) {  // value head: straight copy into the cache
+    const int h = slot_index - H - KVH;
+    const int slot = slots[t];
+    TC* dst = v_cache + ((static_cast<size_t>(slot / block_size) * KVH + h) * block_size + slot % block_size) * Dh;
+    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + d, load_as_float(in + d));
+    return;
+  }
+
+  float x1[TIE_MAX_PAIRS], x2[TIE_MAX_PAIRS];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < TIE_MAX_PAIRS; ++i) {
+    const int p = lane + i * TIE_WAVE;
+    x1[i] = 0.f;
+    x2[i] = 0.f;
+    if (p < half) {
+      x1[i] = load_as_float(in + p);
+      x2[i] = load_as_float(in + p + half);
+      ss += x1[i] * x1[i] + x2[i] * x2[i];
+    }
+  }
+  const float* w = is_q ? q_w : k_w;
+  float inv = 1.0f;
+  if (w != nullptr) {
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / static_cast<float>(Dh) + eps);
+  }
+  const float pos = static_cast<float>(positions[t]);
+
+  TQ* dense_dst = nullptr;
+  TC* cache_dst = nullptr;
+  if (is_q) {
+    dense_dst = q_out + static_cast<size_t>(t) * q_row + static_cast<size_t>(slot_index) * Dh;
+  } else if (k_dense != nullptr) {
+    dense_dst = k_dense + static_cast<size_t>(t) * k_row + static_cast<size_t>(slot_index - H) * Dh;
+  } else {
+    const int h = slot_index - H;
+    const int slot = slots[t];
+    cache_dst = k_cache + ((static_cast<size_t>(slot / block_size) * KVH + h) * block_size + slot % block_size) * Dh;
+  }
+#pragma unroll
+  for (int i = 0; i < TIE_MAX_PAIRS; ++i) {
+    const int p = lane + i * TIE_WAVE;
+    if (p >= half) continue;
+    float a = x1[i], b = x2[i];
+    if (w != nullptr) {
+      a = (a * inv) * w[p];
+      b = (b * inv) * w[p + half];
+    }
+    float o1 = a, o2 = b;
+    if (inv_freq != nullptr) {
+      const float angle = pos * inv_freq[p];
+      float sn, cs;
+      sincosf(angle, &sn, &cs);
+      o1 = a * cs - b * sn;
+      o2 = b * cs + a * sn;
+    }
+    if (dense_dst != nullptr) {
+      store_from_float(dense_dst + p, o1);
+      store_from_float(dense_dst + p + half, o2);
+    } else {
+      store_from_float(cache_dst + p, o1);
+      store_from_float(cache_dst + p + half, o2);
+    }
+  }
+}
+
+extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int q_dtype,
+                                         const float* q_w, const float* k_w, float eps, const float* inv_freq,
+                                         const int* positions, const int* slots, void* k_cache, void* v_cache,
+                                         int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
+                                         int Dh, int block_size, int in_row, int q_row, int k_row,
+                                         hipStream_t stream) {
+  if (T <= 0 || H <= 0 || KVH <= 0 || Dh <= 0 || Dh % 2 != 0 || Dh > 2 * TIE_MAX_PAIRS * TIE_WAVE ||
+      block_size <= 0 || T > 65535 || q_row < H * Dh)
+    return TIE_BAD_ARGUMENT;
+  if (write_kv && (slots == nullptr || k_cache == nullptr || v_cache == nullptr || k_dense != nullptr))
+    return TIE_BAD_ARGUMENT;
+  const int heads = H + ((write_kv || k_dense != nullptr) ? KVH : 0) + (write_kv ? KVH : 0);
+  if (in_row < heads * Dh || (k_dense != nullptr && k_row < KVH * Dh)) return TIE_BAD_ARGUMENT;
+  const dim3 grid(heads, T);
+#define LAUNCH(TX, TQ, TC)                                                                                   \
+  qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
+      static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, positions, slots,       \
+      static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
+      block_size, in_row, q_row, k_row)
+  if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
+  else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
+  else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_BF16) LAUNCH(float, float, bf16_t);
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------------------ argmax
+// out[r] = index of the first maximum of logits[r, :] (ties go to the lowest id,
+// as std::max_element in src/sampling/sampler.cpp:24); -1 if the row holds a NaN.
+__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+  __shared__ float best_v[16];
+  __shared__ int best_i[16];
+  __shared__ int saw_nan;
+  const int r = blockIdx.x;
+  const float* row = logits + static_cast<size_t>(r) * V;
+  if (threadIdx.x == 0) saw_nan = 0;
+  __syncthreads();
+  float bv = -INFINITY;
+  int bi = V;  // sentinel: larger than any index
+  bool nan = false;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    const float v = row[i];
+    nan |= (v != v);
+    if (v > bv || (v == bv && i < bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+  if (nan) saw_nan = 1;
+#pragma unroll
+  for (int off = TIE_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, TIE_WAVE);
+    const int oi = __shfl_xor(bi, off, TIE_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  const int lane = threadIdx.x & (TIE_WAVE - 1);
+  const int wave = threadIdx.x / TIE_WAVE;
+  if (lane == 0) {
+    best_v[wave] = bv;
+    best_i[wave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int waves = blockDim.x / TIE_WAVE;
+    for (int w = 1; w < waves; ++w) {
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+        bv = best_v[w];
+        bi = best_i[w];
+      }
+    }
+    out[r] = saw_nan ? -1 : bi;
+  }
+}
+
+extern "C" int tie_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
+  if (R <= 0 || V <= 0) return TIE_BAD_ARGUMENT;
+  argmax_kernel<<<R, 1024, 0, stream>>>(logits, out, V);
+  return tie_launch_status();
+}
+
+// ------------------------------------------------------ temperature sampling
+// Draws out[r] from softmax(logits[r] * inv_temperature[r]) by inverting the
+// cumulative sum in index order with the uniform number uniform[r] in [0, 1):
+// weights exp((l - max) * inv_t) in float, sums in double, r = uniform * total,
+// first index at which the running remainder turns negative
+// (src/sampling/sampler.cpp:35-39,56-60,75-80 without top-k / top-p).
+// out[r] = -1 for a row with a NaN, -2 for a row that is all -inf; a +inf logit wins outright.
+#define SAMPLE_THREADS 1024
+__global__ void sample_kernel(const float* __restrict__ logits, const float* __restrict__ inv_temperature,
+                              const double* __restrict__ uniform, int* __restrict__ out, int V) {
+  __shared__ float fscratch[16];
+  __shared__ double sums[SAMPLE_THREADS];
+  __shared__ int flag_nan;
+  __shared__ int chosen;
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* row = logits + static_cast<size_t>(r) * V;
+  if (tid == 0) {
+    flag_nan = 0;
+    chosen = V;
+  }
+  __syncthreads();
+  float mx = -INFINITY;
+  bool nan = false;
+  for (int i = tid; i < V; i += SAMPLE_THREADS) {
+    const float v = row[i];
+    nan |= (v != v);
+    mx = fmaxf(mx, v);
+  }
+  if (nan) flag_nan = 1;
+  mx = block_max(mx, fscratch);
+  __syncthreads();
+  if (flag_nan) {
+    if (tid == 0) out[r] = -1;
+    return;
+  }
+  if (mx == -INFINITY) {
+    if (tid == 0) out[r] = -2;
+    return;
+  }
+  const float inv_t = inv_temperature[r];
+  // Each thread owns one contiguous segment so that the walk is in index order.
+  const int seg = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int begin = min(tid * seg, V);
+  const int end = min(begin + seg, V);
+  if (mx == INFINITY) {  // the lowest +inf index wins without a draw
+    int first = V;
+    for (int i = begin; i < end; ++i) {
+      if (row[i] == INFINITY) {
+        first = i;
+        break;
+      }
+    }
+    if (first < V) atomicMin(&chosen, first);
+    __syncthreads();
+    if (tid == 0) out[r] = chosen;
+    return;
+  }
+  double local = 0.0;
+  for (int i = begin; i < end; ++i) local += static_cast<double>(expf((row[i] - mx) * inv_t));
+  sums[tid] = local;
+  __syncthreads();
+  if (tid == 0) {
+    double total = 0.0;
+    for (int i = 0; i < SAMPLE_THREADS; ++i) total += sums[i];
+    double rem = uniform[r] * total;
+    int owner = SAMPLE_THREADS - 1;
+    for (int i = 0; i < SAMPLE_THREADS; ++i) {
+      if (rem - sums[i] < 0.0) {
+        owner = i;
+        break;
+      }
+      rem -= sums[i];
+    }
+    // Walk the owner's segment; fall back to the last index with weight if rounding leaves a remainder.
+    const int b = min(owner * seg, V), e = min(b + seg, V);
+    int pick = -1;
+    for (int i = b; i < e; ++i) {
+      rem -= static_cast<double>(expf((row[i] - mx) * inv_t));
+      if (rem < 0.0) {
+        pick = i;
+        break;
+      }
+    }
+    if (pick < 0) pick = V - 1;
+    out[r] = pick;
+  }
+}
+
+extern "C" int tie_sample(const float* logits, const float* inv_temperature, const double* uniform, int* out,
+                          int R, int V, hipStream_t stream) {
+  if (R <= 0 || V <= 0) return TIE_BAD_ARGUMENT;
+  sample_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, inv_temperature, uniform, out, V);
+  return tie_launch_status();
+}

@@ -1,0 +1,198 @@
+"""One step's batch: flat, unpadded runs of tokens, one run per request.
+
+An entry is (a request's cache holdings, how many of its tokens are already
+cached, its next tokens, the rows among them whose logits are wanted). The runs
+may be whole prompts, portions of prompts cut anywhere, or single decoded
+tokens, freely mixed. ``build`` lays out the arrays the kernels read, as the
+reference's engine does (``src/engine/engine.cpp:104-135``):
+
+    tokens[T] positions[T] seq_of_row[T] query_start[S+1] context_lens[S]
+    state_slots[S] logit_rows[R]   and per paged cache group:
+    slot_mapping[T] block_tables[S, max_blocks_per_seq]
+
+``context_lens`` counts the cached tokens AFTER this step; the query at row t of
+sequence s sits at position ``context_lens[s] - n_new[s] + (t - query_start[s])``.
+All arrays travel to the device in one copy from one pinned staging buffer.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import FREED, CacheManager, RequestCache
+from ..errors import CapacityError, InvalidArgument
+
+
+@dataclasses.dataclass
+class StepEntry:
+    cache: RequestCache
+    start: int                       # tokens of the request already in the cache
+    tokens: Sequence[int]            # its next tokens, run in this step
+    want: Sequence[int] = ()         # places among ``tokens`` whose logits are wanted
+
+
+class GroupStep:
+    """This step's view of one paged cache group."""
+
+    def __init__(self, slot_mapping, block_tables):
+        self.slot_mapping = slot_mapping     # int32 [T]
+        self.block_tables = block_tables     # int32 [S, max_blocks_per_seq]
+        self.extra: Dict[str, torch.Tensor] = {}
+
+
+class StepBatch:
+    """The arrays of one step, on the device, plus the host-side numbers parts plan with."""
+
+    def __init__(self):
+        self.num_tokens = 0
+        self.num_seqs = 0
+        self.num_logit_rows = 0
+        self.tokens = self.positions = self.seq_of_row = None
+        self.query_start = self.context_lens = self.state_slots = self.logit_rows = None
+        self.groups: Dict[int, GroupStep] = {}
+        # host copies for planning
+        self.host_new_tokens: List[int] = []
+        self.host_context_lens: List[int] = []
+        self.max_context = 0
+        self.max_new_tokens = 0
+        self.all_decode = False
+
+
+def _align(n: int, to: int = 4) -> int:
+    return (n + to - 1) // to * to
+
+
+class BatchBuilder:
+    """Builds StepBatches into reusable staging memory."""
+
+    def __init__(self, cache: CacheManager, vocab_size: int, max_blocks_per_seq: int, device):
+        if max_blocks_per_seq <= 0:
+            raise InvalidArgument(f"max_blocks_per_seq must be positive, got {max_blocks_per_seq}")
+        self.cache = cache
+        self.vocab_size = vocab_size
+        self.max_blocks_per_seq = max_blocks_per_seq
+        self.device = torch.device(device)
+        self._host: Optional[torch.Tensor] = None
+        self._dev: Optional[torch.Tensor] = None
+        self._copied = None  # event: the last copy out of the staging buffer has finished
+
+    def _buffers(self, count: int):
+        if self._host is None or self._host.numel() < count:
+            size = max(count * 2, 4096)
+            pin = self.device.type == "cuda"
+            self._host = torch.empty(size, dtype=torch.int32, pin_memory=pin)
+            self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
+            self._copied = None
+        elif self._copied is not None:
+            self._copied.synchronize()
+        return self._host, self._dev
+
+    def build(self, entries: Sequence[StepEntry]) -> StepBatch:
+        if not entries:
+            raise InvalidArgument("a step needs at least one entry")
+        bs = self.cache.block_size
+        MB = self.max_blocks_per_seq
+        S = len(entries)
+        seen = set()
+        T = 0
+        R = 0
+        for e in entries:
+            n = len(e.tokens)
+            if n < 1:
+                raise InvalidArgument("an entry of a step needs at least one token")
+            if id(e.cache) in seen:
+                raise InvalidArgument("a request appears twice in one step")
+            seen.add(id(e.cache))
+            if e.start < 0:
+                raise InvalidArgument(f"an entry starts at position {e.start}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise InvalidArgument(f"wanted place {w} lies outside the entry's {n} tokens")
+            need = self.cache.blocks_for(e.start + n)
+            if need > MB:
+                raise CapacityError(
+                    f"{e.start + n} tokens need {need} KV blocks but a block-table row holds {MB}")
+            for g in self.cache.plan.paged_groups:
+                if len(e.cache.tables[g]) < need:
+                    raise InvalidArgument(
+                        f"a request has {len(e.cache.tables[g])} KV blocks reserved; {e.start + n} tokens need {need}")
+            if self.cache.plan.state_groups and e.cache.state_slot < 0:
+                raise InvalidArgument("a request of a model with per-request state has no state slot")
+            T += n
+            R += len(e.want)
+
+        groups = self.cache.plan.paged_groups
+        layout = {}
+        offset = 0
+        for name, count in (("tokens", T), ("positions", T), ("seq_of_row", T), ("query_start", S + 1),
+                            ("context_lens", S), ("state_slots", S), ("logit_rows", R)):
+            layout[name] = (offset, count)
+            offset += _align(count)
+        for g in groups:
+            layout[("slots", g)] = (offset, T)
+            offset += _align(T)
+            layout[("tables", g)] = (offset, S * MB)
+            offset += _align(S * MB)
+        host_t, dev_t = self._buffers(offset)
+        host = host_t.numpy()
+
+        def view(key):
+            o, c = layout[key]
+            return host[o:o + c]
+
+        tokens, positions, seq_of_row = view("tokens"), view("positions"), view("seq_of_row")
+        query_start, context_lens = view("query_start"), view("context_lens")
+        state_slots, logit_rows = view("state_slots"), view("logit_rows")
+        batch = StepBatch()
+        row = 0
+        r = 0
+        query_start[0] = 0
+        for s, e in enumerate(entries):
+            n = len(e.tokens)
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if ids.min() < 0 or ids.max() >= self.vocab_size:
+                bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
+                raise InvalidArgument(f"token id {bad} outside vocabulary of {self.vocab_size}")
+            tokens[row:row + n] = ids
+            positions[row:row + n] = np.arange(e.start, e.start + n, dtype=np.int32)
+            seq_of_row[row:row + n] = s
+            context_lens[s] = e.start + n
+            state_slots[s] = max(e.cache.state_slot, 0)
+            for w in e.want:
+                logit_rows[r] = row + w
+                r += 1
+            for g in groups:
+                table = e.cache.tables[g]
+                view(("slots", g))[row:row + n] = self.cache.slots(e.cache, g, e.start, e.start + n)
+                trow = view(("tables", g))[s * MB:(s + 1) * MB]
+                trow[:len(table)] = [0 if b == FREED else b for b in table][:MB]
+                trow[len(table):] = 0
+            row += n
+            query_start[s + 1] = row
+            batch.host_new_tokens.append(n)
+            batch.host_context_lens.append(e.start + n)
+
+        dev_t[:offset].copy_(host_t[:offset], non_blocking=True)
+        if self.device.type == "cuda":
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
+        def dev(key, shape=None):
+            o, c = layout[key]
+            t = dev_t[o:o + c]
+            return t.view(*shape) if shape else t
+
+        batch.num_tokens, batch.num_seqs, batch.num_logit_rows = T, S, R
+        batch.tokens, batch.positions, batch.seq_of_row = dev("tokens"), dev("positions"), dev("seq_of_row")
+        batch.query_start, batch.context_lens = dev("query_start"), dev("context_lens")
+        batch.state_slots, batch.logit_rows = dev("state_slots"), dev("logit_rows")
+        for g in groups:
+            batch.groups[g] = GroupStep(dev(("slots", g)), dev(("tables", g), (S, MB)))
+        batch.max_context = max(batch.host_context_lens)
+        batch.max_new_tokens = max(batch.host_new_tokens)
+        batch.all_decode = batch.max_new_tokens == 1
+        return batch

@@ -1,0 +1,246 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+Five kinds of part exist, each with a registry from a kind name to a class:
+
+* norm          ``forward(ctx, x, rows=None) -> h``
+* position      describes or applies a position encoding to queries and keys
+* mixer         ``forward(ctx, h, cache, residual)``; declares a cache need
+* feed_forward  ``forward(ctx, h, residual)``
+* block         ``forward(ctx, x, layer, cache)``: the arrangement of the above
+
+plus the two ends of a model, ``embedding`` and ``head``. A part is built from
+the parameters of its PartSpec (sizes, constants, tensor names) and never looks
+at the model around it. It declares the tensors it expects (``tensors()``),
+takes them at load time (``load``) and runs on a StepContext.
+
+The residual stream is float32 in both compute modes; ``h`` (a norm's output,
+a matrix product's input) has the activation dtype of the mode. Mixers and
+feed-forwards ADD their result to the ``residual`` tensor they are given, which
+lets the last matrix product of a part fold the addition into its epilogue.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Callable, Dict, List, Mapping, Optional
+
+import torch
+
+import dataclasses
+
+from ..errors import InvalidArgument
+from ..weights.binder import BFLOAT16, FLOAT32, TensorSpec
+
+@dataclasses.dataclass(frozen=True)
+class PartSpec:
+    """A registered part kind plus the parameters (sizes, constants, tensor names) it is built with."""
+
+    kind: str
+    params: Mapping[str, Any] = dataclasses.field(default_factory=dict)
+
+
+_KINDS = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+_REGISTRIES: Dict[str, Dict[str, type]] = {k: {} for k in _KINDS}
+
+
+def register_part(family: str, kind: str, cls: type = None):
+    """Registers ``cls`` as the part ``kind`` of ``family``; usable as a decorator."""
+    if family not in _REGISTRIES:
+        raise InvalidArgument(f"unknown part family '{family}' (families: {', '.join(_KINDS)})")
+
+    def apply(c):
+        _REGISTRIES[family][kind] = c
+        return c
+
+    return apply(cls) if cls is not None else apply
+
+
+def unregister_part(family: str, kind: str) -> None:
+    _REGISTRIES.get(family, {}).pop(kind, None)
+
+
+def registered_parts(family: str):
+    return tuple(sorted(_REGISTRIES[family]))
+
+
+def build_part(family: str, spec: PartSpec, **extra):
+    """Instantiates the part ``spec`` names from the registry of ``family``."""
+    try:
+        cls = _REGISTRIES[family][spec.kind]
+    except KeyError:
+        raise InvalidArgument(
+            f"no {family} part is registered as '{spec.kind}' (registered: {', '.join(registered_parts(family)) or 'none'})"
+        ) from None
+    return cls(dict(spec.params), **extra)
+
+
+class Part:
+    """Base of every part: declared tensors, loading, and nothing else."""
+
+    def __init__(self, params: Mapping[str, Any]):
+        self.params = dict(params)
+
+    def tensors(self) -> List[TensorSpec]:
+        return []
+
+    def load(self, fetch: Callable[[str, str], torch.Tensor], mode: str, device) -> None:
+        """Takes the part's tensors: ``fetch(name, role)`` returns the placed device tensor."""
+
+    def children(self) -> List["Part"]:
+        return []
+
+    def all_tensors(self) -> List[TensorSpec]:
+        out = list(self.tensors())
+        for child in self.children():
+            out.extend(child.all_tensors())
+        return out
+
+    def load_all(self, fetch, mode: str, device) -> None:
+        self.load(fetch, mode, device)
+        for child in self.children():
+            child.load_all(fetch, mode, device)
+
+
+class Workspace:
+    """Named scratch tensors that live across steps and only ever grow.
+
+    A part asks for ``get(name, shape, dtype)`` each step and receives a view of
+    the buffer kept under that name; steady-state steps allocate nothing, and
+    the addresses stay put, which replaying a recorded step relies on.
+    """
+
+    def __init__(self, device):
+        self.device = device
+        self._buffers: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        numel = 1
+        for d in shape:
+            numel *= int(d)
+        key = f"{name}:{dtype}"
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < numel:
+            buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:numel].view(*shape)
+
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+
+
+class StepContext:
+    """What a part sees of one step: the batch, the mode, scratch memory and the caches."""
+
+    def __init__(self, batch, mode: str, device, workspace: Workspace, cache_manager, cache_plan):
+        self.batch = batch
+        self.mode = mode
+        self.device = device
+        self.workspace = workspace
+        self.cache_manager = cache_manager
+        self.cache_plan = cache_plan
+        self.act_dtype = torch.float32 if mode == FLOAT32 else torch.bfloat16
+        self.notes: Dict[Any, Any] = {}   # per-step memo shared by parts (e.g. one plan for all layers)
+
+    @property
+    def num_tokens(self) -> int:
+        return self.batch.num_tokens
+
+    def scratch(self, name: str, shape, dtype: torch.dtype = None) -> torch.Tensor:
+        return self.workspace.get(name, shape, dtype or self.act_dtype)
+
+    def cache_of(self, call_index: int):
+        """The cache binding of run-order entry ``call_index`` (None if its mixer has no cache)."""
+        from ..cache.spec import PagedKV
+
+        entry = self.cache_plan.calls[call_index]
+        if entry is None:
+            return None
+        need = self.cache_plan.groups[entry.group].need
+        if isinstance(need, PagedKV):
+            k, v = self.cache_manager.kv_planes(entry.group, entry.plane)
+            return PagedBinding(need, entry.writes, k, v, self.batch.groups[entry.group],
+                                self.cache_manager.block_size)
+        return StateBinding(need, entry.writes, self.cache_manager.state_plane(entry.group, entry.plane),
+                            self.batch.state_slots)
+
+
+class PagedBinding:
+    """Keys and values of one plane plus this step's slots and block tables of its group."""
+
+    def __init__(self, need, writes, k_cache, v_cache, step, block_size):
+        self.need = need
+        self.writes = writes
+        self.k_cache = k_cache      # [num_blocks, kv_heads, block_size, head_dim]
+        self.v_cache = v_cache
+        self.step = step            # GroupStep: slot_mapping [T], block_tables [S, MB], ...
+        self.block_size = block_size
+
+
+class StateBinding:
+    """The fixed-size states of one plane plus the slot of each sequence of this step."""
+
+    def __init__(self, need, writes, state, state_slots):
+        self.need = need
+        self.writes = writes
+        self.state = state          # [max_state_slots, *shape]
+        self.state_slots = state_slots  # int32 [S] on the device
+
+
+class Norm(Part):
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Position(Part):
+    """A position encoding applied to queries and keys inside an attention mixer.
+
+    ``rotary_table()`` returns ``(inv_freq float32 [rotary_dim/2], rotary_dim,
+    pairing)`` when the encoding is a rotation of pairs by position * inv_freq,
+    which the fused kernel applies itself; otherwise it returns None and the
+    mixer calls ``apply(ctx, q, k, positions)`` on float32 tensors
+    ``[T, heads, head_dim]`` instead.
+    """
+
+    def rotary_table(self):
+        return None
+
+    def apply(self, ctx: StepContext, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        """What this mixer needs from the cache: a PagedKV, a FixedState, or None."""
+        return None
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """The arrangement of one layer's parts. ``layer`` carries .mixer, .feed_forward and .norms."""
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+__all__ = [
+    "BFLOAT16", "FLOAT32", "Block", "Embedding", "FeedForward", "Head", "Mixer", "Norm", "PagedBinding",
+    "Part", "PartSpec", "Position", "StateBinding", "StepContext", "TensorSpec", "Workspace", "build_part",
+    "register_part", "registered_parts", "unregister_part",
+]

@@ -1,0 +1,31 @@
+"""Arrangements of a layer's parts.
+
+``pre_norm`` is the reference's block (``src/model/qwen3.cpp:216-239``):
+``x += mixer(norm(x)); x += feed_forward(norm(x))`` with the norms named
+``pre_mixer`` and ``pre_feed_forward`` in the layer's spec and nothing applied
+to the sub-layer outputs.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..errors import InvalidArgument
+from .base import Block, StepContext, register_part
+
+
+@register_part("block", "pre_norm")
+class PreNormBlock(Block):
+    NORMS = ("pre_mixer", "pre_feed_forward")
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
+        h = layer.norms["pre_mixer"].forward(ctx, x)
+        layer.mixer.forward(ctx, h, cache, x)
+        h = layer.norms["pre_feed_forward"].forward(ctx, x)
+        layer.feed_forward.forward(ctx, h, x)
+
+    @classmethod
+    def check(cls, norms) -> None:
+        missing = [n for n in cls.NORMS if n not in norms]
+        if missing:
+            raise InvalidArgument(f"a pre_norm block needs the norms {', '.join(cls.NORMS)}; missing {', '.join(missing)}")

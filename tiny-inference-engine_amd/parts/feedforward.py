@@ -1,0 +1,44 @@
+"""The dense SwiGLU feed-forward.
+
+``g = h @ Wg^T``, ``u = h @ Wu^T``, ``a = g / (1 + exp(-g)) * u`` evaluated left
+to right, ``out = a @ Wd^T``, added to the residual; no bias, no experts
+(``src/model/qwen3.cpp:235-239``, ``src/backend/cpu/cpu_backend.cpp:195-207``).
+Gate and up run as one product over the two matrices side by side.
+Parameters: ``hidden``, ``intermediate``, ``names`` (``gate``, ``up``, ``down``).
+"""
+
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from .. import kernels
+from .base import FeedForward, StepContext, TensorSpec, register_part
+from .linear import Linear
+
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, params):
+        super().__init__(params)
+        self.hidden = int(params["hidden"])
+        self.intermediate = int(params["intermediate"])
+        names = params["names"]
+        self.gate_up = Linear([names["gate"], names["up"]], [self.intermediate, self.intermediate], self.hidden)
+        self.down = Linear([names["down"]], [self.hidden], self.intermediate)
+
+    def tensors(self) -> List[TensorSpec]:
+        return self.gate_up.tensors() + self.down.tensors()
+
+    def load(self, fetch, mode, device) -> None:
+        self.gate_up.load(fetch)
+        self.down.load(fetch)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, residual: torch.Tensor) -> None:
+        T = h.shape[0]
+        gate_up = ctx.scratch("swiglu.gate_up", (T, 2 * self.intermediate))
+        self.gate_up(h, gate_up)
+        act = ctx.scratch("swiglu.act", (T, self.intermediate))
+        kernels.swiglu(gate_up, act)
+        self.down(act, residual, accumulate=True)

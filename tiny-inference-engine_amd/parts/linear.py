@@ -1,0 +1,51 @@
+"""A projection ``out = x @ W^T`` whose weight may be several stored matrices side by side.
+
+Weights keep their stored ``[out, in]`` layout (``src/model/qwen3.cpp:81-90``).
+Listing several names concatenates them along the output dimension at load
+time (q, k, v or gate, up in one product): the arithmetic of each output
+column is unchanged, the activation is read once instead of several times.
+No bias: the reference has none.
+"""
+
+from __future__ import annotations
+
+from typing import List, Sequence, Tuple
+
+import torch
+
+from .. import kernels
+from ..errors import InvalidArgument
+from ..weights.binder import TensorSpec
+
+
+class Linear:
+    def __init__(self, names: Sequence[str], out_features: Sequence[int], in_features: int, init_std: float = 0.02):
+        if len(names) != len(out_features) or not names:
+            raise InvalidArgument("a projection needs one output size per weight name")
+        self.names = list(names)
+        self.out_features = list(out_features)
+        self.in_features = in_features
+        self.init_std = init_std
+        self.weight: torch.Tensor = None
+
+    @property
+    def total_out(self) -> int:
+        return sum(self.out_features)
+
+    def tensors(self) -> List[TensorSpec]:
+        return [TensorSpec(n, (o, self.in_features), "matrix", ("normal", self.init_std))
+                for n, o in zip(self.names, self.out_features)]
+
+    def load(self, fetch) -> None:
+        parts = [fetch(n, "matrix") for n in self.names]
+        if len(parts) == 1:
+            self.weight = parts[0]
+            return
+        dtypes = {p.dtype for p in parts}
+        if len(dtypes) > 1:  # stored in different widths: the wider one decides
+            parts = [p.to(torch.float32) for p in parts]
+        self.weight = torch.cat(parts, dim=0).contiguous()
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+        kernels.linear(x, self.weight, out, accumulate)
+        return out

@@ -1,0 +1,39 @@
+"""RMSNorm: ``out = (x * inv) * w`` with ``inv = 1 / sqrt(mean(x^2) + eps)``.
+
+The weight multiplies after normalisation and is the plain ``w`` (not ``1 + w``);
+no bias, no mean subtraction; statistics in float32
+(``src/backend/cpu/cpu_backend.cpp:141-159``). Parameters: ``dim``, ``eps``,
+``weight`` (tensor name).
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import kernels
+from .base import Norm, StepContext, TensorSpec, register_part
+
+
+@register_part("norm", "rms_norm")
+class RMSNorm(Norm):
+    def __init__(self, params):
+        super().__init__(params)
+        self.dim = int(params["dim"])
+        self.eps = float(params["eps"])
+        self.weight_name = params["weight"]
+        self.weight: torch.Tensor = None
+
+    def tensors(self) -> List[TensorSpec]:
+        return [TensorSpec(self.weight_name, (self.dim,), "vector", ("one_plus_uniform", 0.1))]
+
+    def load(self, fetch, mode, device) -> None:
+        self.weight = fetch(self.weight_name, "vector")
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
+        count = x.shape[0] if rows is None else rows.numel()
+        out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
+        kernels.rms_norm(x, self.weight, self.eps, out, rows)
+        return out
