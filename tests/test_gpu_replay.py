@@ -1,0 +1,126 @@
+"""The engine against the plain implementation under every way of cutting the work.
+
+Each request alone and whole; most of it in one step and the last 32 tokens one by one; in
+portions of changing size down to two tokens; and mixed, up to four live requests, portions
+of some beside decoded tokens of others, in a pool so small that pages are used again -
+in float32 and in bfloat16, for two tiny configurations that differ in every size.
+"""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import trace_helpers as th
+from conftest import BLOCK_SIZE, ROOT, TINY, load_plain_weights
+
+pytestmark = pytest.mark.gpu
+
+# max |engine - plain| / max |plain| over a request's logits
+TOLERANCE = {"float32": 1e-4, "bfloat16": 3e-2}
+LENGTHS = {"A": [5, 11, 17, 40, 64, 33], "B": [1, 23, 40, 64, 90, 37]}
+
+
+def reference_logits(folder, cfg, requests):
+    weights = load_plain_weights(folder)
+    return {rid: plain.forward(weights, cfg, toks).float() for rid, toks in requests.items()}
+
+
+def check(got, want, dtype, label):
+    worst = 0.0
+    for rid, ref in want.items():
+        rows = got[rid]
+        assert sorted(rows) == list(range(ref.shape[0])), f"{label}: request {rid} misses positions"
+        mine = torch.stack([rows[p] for p in range(ref.shape[0])])
+        assert torch.isfinite(mine).all(), f"{label}: request {rid} has non-finite logits"
+        err = (mine - ref).abs().amax(dim=1) / ref.abs().max()
+        bad = int(torch.argmax((err > TOLERANCE[dtype]).float())) if bool((err > TOLERANCE[dtype]).any()) else -1
+        assert bad < 0, (f"{label}: request {rid} first differs at position {bad} "
+                         f"(relative error {float(err[bad]):.3e}, allowed {TOLERANCE[dtype]:.0e})")
+        worst = max(worst, float(err.max()))
+    return worst
+
+
+@pytest.fixture(scope="module")
+def folders(model_folders, model_folders_bf16):
+    return {"float32": model_folders, "bfloat16": model_folders_bf16}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_all_ways_of_cutting(folders, name, dtype):
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders[dtype][name]
+    requests = th.make_requests(cfg["vocab_size"], LENGTHS[name], seed=5)
+    want = reference_logits(folder, cfg, requests)
+    bs = BLOCK_SIZE[name]
+    biggest = max(th.round64(len(t)) for t in requests.values())
+
+    def replayer(max_tokens):
+        return TraceReplayer.from_folder(folder, dtype, max_tokens, block_size=bs)
+
+    results = {}
+    results["whole"] = th.collect(replayer(biggest), th.whole(requests))
+    results["prefill+decode"] = th.collect(replayer(biggest), th.prefill_then_decode(requests))
+    results["portions"] = th.collect(replayer(biggest), th.portions(requests))
+    steps, peak = th.mixed(requests, max_live=4, seed=3)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    rep = replayer(peak)
+    results["mixed"] = th.collect(rep, steps)
+    assert rep.cache.num_free() == rep.cache.num_blocks          # every page came back
+    for label, got in results.items():
+        check(got, want, dtype, f"{name}/{dtype}/{label}")
+    # the ways of cutting agree with each other far more closely than with the reference in bf16
+    if dtype == "float32":
+        for label in ("prefill+decode", "portions", "mixed"):
+            for rid in requests:
+                a = torch.stack([results["whole"][rid][p] for p in range(len(requests[rid]))])
+                b = torch.stack([results[label][rid][p] for p in range(len(requests[rid]))])
+                assert float((a - b).abs().max() / a.abs().max()) < 1e-5, f"{name}: whole vs {label}, request {rid}"
+
+
+def test_pages_are_used_again(folders):
+    """A pool of exactly one request's pages serves request after request."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["float32"]["A"]
+    requests = th.make_requests(cfg["vocab_size"], [60, 64, 50, 61], seed=9)
+    want = reference_logits(folder, cfg, requests)
+    rep = TraceReplayer.from_folder(folder, "float32", 64, block_size=4)
+    got = th.collect(rep, th.portions(requests, sizes=(9, 2, 30, 5)))
+    check(got, want, "float32", "A/reuse")
+
+
+def test_trace_run_program(folders, tmp_path):
+    """The program itself: JSON lines in, .f32 files and 'done' lines out."""
+    folder, cfg = folders["float32"]["B"]
+    requests = th.make_requests(cfg["vocab_size"], [23, 40], seed=2)
+    steps, peak = th.mixed(requests, max_live=2, seed=1)
+    steps.append({"step": len(steps), "entries": [{"id": "late", "tokens": [1, 2, 3], "want": []}], "end": ["late"]})
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", folder, "--dtype", "float32",
+         "--out", str(out), "--max-tokens", str(peak + 64)],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    assert not (out / f"{steps[-1]['step']}.f32").exists()        # nothing was wanted in the last step
+    want = reference_logits(folder, cfg, requests)
+    position = {}
+    for s in steps[:-1]:
+        data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+        r = 0
+        for e in s["entries"]:
+            start = position.get(e["id"], 0)
+            for w in e["want"]:
+                ref = want[e["id"]][start + w]
+                assert float(np.abs(data[r] - ref.numpy()).max() / ref.abs().max()) < 1e-4
+                r += 1
+            position[e["id"]] = start + len(e["tokens"])
+        assert r == data.shape[0]

@@ -53,9 +53,8 @@ def _build_dir() -> pathlib.Path:
     preferred = CSRC / "_build"
     try:
         preferred.mkdir(parents=True, exist_ok=True)
-        probe = preferred / f".write-test-{os.getpid()}"
-        probe.write_bytes(b"")
-        probe.unlink()
+        if not os.access(preferred, os.W_OK | os.X_OK):
+            raise PermissionError(str(preferred))
         return preferred
     except OSError:
         fallback = pathlib.Path(tempfile.gettempdir()) / f"tie_amd_build_{os.getuid()}"
@@ -95,7 +94,8 @@ def compile_library(name: str, source: str, defines: Optional[Mapping[str, objec
     _log(f"compiling {source} -> {target.name} (hipcc, {ARCH})")
     started = time.time()
     env = dict(os.environ)
-    env.setdefault("HOME", tempfile.gettempdir())  # hipcc may want a home for its caches
+    if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+        env["HOME"] = tempfile.gettempdir()  # hipcc may want a writable home for its caches
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     output = []
     reader = threading.Thread(target=lambda: output.append(proc.stdout.read()), daemon=True)
