@@ -1,0 +1,238 @@
+"""Generation through the engine on the GPU: the entry points, chunked prefill, batching, preemption.
+
+Scenarios of the reference's tests/engine/test_engine.cpp and test_engine_batching.cpp, with the plain
+implementation in place of the fixtures the reference downloads.
+"""
+
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from conftest import BLOCK_SIZE, ROOT, load_plain_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def prompt_of(n, vocab, salt=0):
+    return [(i * 5 + 1 + salt * 13) % vocab for i in range(n)]
+
+
+def make_engine(folder, block_size, **kw):
+    import tie_amd
+
+    kw.setdefault("kv_blocks", 256)
+    kw.setdefault("dtype", "float32")
+    return tie_amd.create_engine(folder, block_size=block_size, **kw)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point_matches_the_plain_implementation(model_folders, name):
+    import tie_amd
+
+    folder, cfg = model_folders[name]
+    weights = load_plain_weights(folder)
+    for n in (1, 9, 30):
+        prompt = prompt_of(n, cfg["vocab_size"], n)
+        want = plain.greedy(weights, cfg, prompt, 12)
+        got = tie_amd.generate(folder, prompt, tie_amd.SamplingParams(max_tokens=12), dtype="float32",
+                               block_size=BLOCK_SIZE[name], kv_blocks=64)
+        assert got == want
+
+
+def test_bfloat16_greedy_generation_starts_like_the_plain_implementation(model_folders_bf16):
+    import tie_amd
+
+    folder, cfg = model_folders_bf16["B"]
+    weights = load_plain_weights(folder)
+    prompt = prompt_of(23, cfg["vocab_size"])
+    want = plain.greedy(weights, cfg, prompt, 8)
+    got = tie_amd.generate(folder, prompt, tie_amd.SamplingParams(max_tokens=8), dtype="bfloat16", kv_blocks=64)
+    assert got[:3] == want[:3]
+
+
+def test_the_command_line_generates_the_same_tokens(model_folders):
+    folder, cfg = model_folders["B"]
+    prompt = prompt_of(11, cfg["vocab_size"])
+    want = plain.greedy(load_plain_weights(folder), cfg, prompt, 6)
+    proc = subprocess.run([sys.executable, str(ROOT / "bin" / "tie"), "generate", "-m", folder, "-p",
+                           ",".join(map(str, prompt)), "--temp", "0", "--max-tokens", "6", "--dtype", "float32",
+                           "--kv-mem", "16M"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == want
+    assert "[tie] hip | load" in proc.stderr and "6 tok generated" in proc.stderr
+    proc = subprocess.run([sys.executable, str(ROOT / "bin" / "tie"), "generate", "-m", folder + "/missing", "-p", "1"],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 1 and "tie: error:" in proc.stderr
+
+
+def test_stop_token_max_tokens_and_pages_returned(model_folders):
+    import tie_amd
+
+    folder, cfg = model_folders["A"]
+    engine = make_engine(folder, 4)
+    prompt = prompt_of(7, cfg["vocab_size"])
+    free = engine.cache.num_free()
+    out = engine.generate(prompt, tie_amd.SamplingParams(max_tokens=9))
+    assert len(out) == 9 and engine.cache.num_free() == free and not engine.has_work()
+    stopper = make_engine(folder, 4, stop_tokens=[out[3]])
+    first = out.index(out[3])
+    assert stopper.generate(prompt, tie_amd.SamplingParams(max_tokens=9)) == out[:first + 1]   # the stop token is kept
+    assert stopper.cache.num_free() == free
+
+
+def test_chunked_prefill_generates_the_unchunked_tokens(model_folders):
+    import tie_amd
+
+    folder, cfg = model_folders["B"]
+    prompt = prompt_of(40, cfg["vocab_size"])
+    params = tie_amd.SamplingParams(max_tokens=10)
+    whole = make_engine(folder, 16, max_seqs=1, max_tokens_per_step=64).generate(prompt, params)
+    for kw in (dict(max_tokens_per_step=5), dict(max_tokens_per_step=64, prefill_chunk=13)):
+        engine = make_engine(folder, 16, max_seqs=1, **kw)
+        assert engine.generate(prompt, params) == whole
+        assert engine.stats().steps > 10 and engine.stats().prefill_tokens == 40 and engine.stats().decode_tokens == 9
+
+
+def test_capacity_rejections_and_clamping(model_folders):
+    import tie_amd
+    from tie_amd.errors import CapacityError, InvalidArgument
+
+    folder, cfg = model_folders["A"]                      # context 128
+    engine = make_engine(folder, 4, kv_blocks=10)         # the pool holds 40 tokens
+    with pytest.raises(InvalidArgument, match="empty"):
+        engine.add_request([])
+    with pytest.raises(InvalidArgument, match="outside vocabulary"):
+        engine.add_request([1, cfg["vocab_size"]])
+    with pytest.raises(CapacityError, match="KV blocks"):
+        engine.add_request([1] * 40)
+    sid = engine.add_request([1] * 30, tie_amd.SamplingParams(max_tokens=100))
+    assert engine.sequence(sid).params.max_tokens == 10   # clamped to the room the pool leaves
+    while engine.has_work():
+        engine.step()
+    assert engine.sequence(sid).num_generated == 10 and engine.sequence(sid).finish_reason.value == "length"
+    big = make_engine(folder, 4, kv_blocks=64)
+    with pytest.raises(CapacityError, match="context"):
+        big.add_request([1] * 128)
+
+
+def mixed_requests(vocab, sampled):
+    import tie_amd
+
+    lens, outs = [3, 17, 9, 30, 1, 12, 25, 6], [10, 4, 12, 8, 6, 9, 5, 11]     # test_engine_batching.cpp:26-41
+    reqs = []
+    for i, (n, m) in enumerate(zip(lens, outs)):
+        prompt = [(t * 7 + i * 13 + 1) % vocab for t in range(n)]
+        p = tie_amd.SamplingParams(max_tokens=m)
+        if sampled:
+            p = tie_amd.SamplingParams(max_tokens=m, temperature=0.8, top_k=10 if i % 2 else 0, seed=100 + i)
+        reqs.append((prompt, p))
+    return reqs
+
+
+@pytest.mark.parametrize("sampled", [False, True])
+@pytest.mark.parametrize("kv_blocks", [256, 12])          # 12 pages of 4 tokens force preemption
+def test_requests_batched_together_generate_what_each_generates_alone(model_folders, sampled, kv_blocks):
+    folder, cfg = model_folders["A"]
+    reqs = mixed_requests(cfg["vocab_size"], sampled)
+    together = make_engine(folder, 4, kv_blocks=kv_blocks, max_seqs=8, max_tokens_per_step=16, policy="fcfs")
+    ids = [together.add_request(p, s) for p, s in reqs]
+    while together.has_work():
+        together.step()
+    stats = together.stats()
+    if kv_blocks == 12:
+        assert stats.preemptions > 0
+    assert stats.seqs_scheduled > stats.steps                 # really batched
+    assert together.cache.num_free() == kv_blocks
+    for sid, (prompt, params) in zip(ids, reqs):
+        alone = make_engine(folder, 4, max_seqs=1, max_tokens_per_step=16)
+        assert alone.generate(prompt, params) == together.sequence(sid).generated, f"request {sid}"
+
+
+def test_a_failing_step_is_rolled_back_and_offered_again(model_folders):
+    import tie_amd
+
+    folder, cfg = model_folders["A"]
+    reqs = mixed_requests(cfg["vocab_size"], False)
+    engine = make_engine(folder, 4, max_seqs=8, max_tokens_per_step=16, policy="fcfs")
+    calls = {"n": 0}
+
+    def hook(index, x):
+        if index == 1:
+            calls["n"] += 1
+            if calls["n"] == 3:
+                raise RuntimeError("injected failure")
+
+    engine.model.layer_hook = hook
+    ids = [engine.add_request(p, s) for p, s in reqs]
+    failures = 0
+    while engine.has_work():
+        try:
+            engine.step()
+        except RuntimeError:
+            failures += 1
+    assert failures == 1
+    engine.model.layer_hook = None
+    for sid, (prompt, params) in zip(ids, reqs):
+        alone = make_engine(folder, 4, max_seqs=1, max_tokens_per_step=16)
+        assert alone.generate(prompt, params) == engine.sequence(sid).generated
+
+
+def test_cancel_release_and_callbacks(model_folders):
+    import tie_amd
+    from tie_amd.errors import InvalidArgument
+
+    folder, cfg = model_folders["A"]
+    engine = make_engine(folder, 4, max_seqs=4, max_tokens_per_step=32)
+    seen = []
+    a = engine.add_request(prompt_of(5, 256), tie_amd.SamplingParams(max_tokens=20))
+    b = engine.add_request(prompt_of(6, 256, 1), tie_amd.SamplingParams(max_tokens=5))
+
+    def on_token(seq_id, token):
+        seen.append((seq_id, token))
+        if seq_id == a and len([s for s in seen if s[0] == a]) == 3:
+            engine.cancel(a)                                  # safe from a token callback
+        with pytest.raises(InvalidArgument):
+            engine.step()                                     # but stepping inside a step is refused
+
+    engine.on_token = on_token
+    with pytest.raises(InvalidArgument, match="still running"):
+        engine.release(a)
+    while engine.has_work():
+        engine.step()
+    assert engine.sequence(a).finish_reason.value == "cancelled" and engine.sequence(a).num_generated == 3
+    assert engine.sequence(b).num_generated == 5
+    engine.release(a)
+    with pytest.raises(InvalidArgument, match="no sequence"):
+        engine.sequence(a)
+    assert engine.cache.num_free() == engine.cache.num_blocks
+
+
+def test_device_sampling_matches_the_host_sampler():
+    import numpy as np
+    from tie_amd.sampling import DeviceSampler, RandomStream, SamplingParams, sample
+
+    g = torch.Generator().manual_seed(4)
+    logits = (torch.randn(6, 1000, generator=g) * 3).cuda()
+    logits[0, 17] = logits[0].max() + 1
+    logits[0, 400] = logits[0, 17]                            # a tie: the lowest id wins
+    logits[5, 3] = float("inf")
+    params = [SamplingParams(), SamplingParams(temperature=0.8, seed=1), SamplingParams(temperature=1.5, seed=2),
+              SamplingParams(temperature=0.7, top_k=20, top_p=0.8, seed=3), SamplingParams(temperature=1e-40),
+              SamplingParams(temperature=1.0, seed=5)]
+    sampler = DeviceSampler("cuda:0")
+    dev_rngs = [RandomStream(p.seed) for p in params]
+    host_rngs = [RandomStream(p.seed) for p in params]
+    host = logits.cpu().numpy()
+    for _ in range(50):
+        got = sampler.sample_rows(logits, params, dev_rngs)
+        want = [sample(host[i], params[i], host_rngs[i]) for i in range(6)]
+        assert got == want
+    assert got[0] == 17 and got[5] == 3
+    bad = logits.clone()
+    bad[2, 9] = float("nan")
+    from tie_amd.errors import InvalidArgument
+    with pytest.raises(InvalidArgument, match="NaN"):
+        sampler.sample_rows(bad, params, dev_rngs)

@@ -1,0 +1,275 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine's.
+
+Head sizes in steps of 16, head counts and groupings that are no powers of two, widths and
+vocabularies with tails, scattered and unordered block tables, windows. Where random data would
+hide a fault (a far key among hundreds, a window's edge, a page of the cache) the inputs are made
+so that it shows.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale).to(dtype)
+
+
+def close(got, want, rel, what=""):
+    got, want = got.detach().cpu().to(F64), want.detach().cpu().to(F64)
+    err = float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+    assert err <= rel, f"{what}: relative error {err:.3e} > {rel:.0e}"
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    from tie_amd import kernels
+
+    table = rnd(37, 100, seed=1, dtype=dtype).cuda()
+    ids = i32([3, 0, 36, 3, 17])
+    out = torch.empty(5, 100, dtype=torch.float32, device="cuda")
+    kernels.embed(table, ids, out)
+    assert torch.equal(out.cpu(), table.cpu().float()[ids.cpu().long()])
+
+
+@pytest.mark.parametrize("n", [16, 100, 1000, 4096, 5120])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rms_norm(n, out_dtype):
+    from tie_amd import kernels
+
+    x = rnd(7, n, seed=2, scale=3.0).cuda()
+    w = (1 + 0.1 * rnd(n, seed=3)).cuda()
+    out = torch.empty(7, n, dtype=out_dtype, device="cuda")
+    kernels.rms_norm(x, w, 1e-5, out)
+    want = plain.rms_norm(x.cpu(), w.cpu(), 1e-5)
+    close(out, want, 1e-5 if out_dtype == torch.float32 else 5e-3, f"rms_norm n={n}")
+    rows = i32([6, 0, 3])
+    picked = torch.empty(3, n, dtype=out_dtype, device="cuda")
+    kernels.rms_norm(x, w, 1e-5, picked, rows)
+    assert torch.equal(picked, out[rows.long()])
+
+
+def test_swiglu():
+    from tie_amd import kernels
+
+    gu = rnd(5, 2 * 200, seed=4, scale=2.0).cuda()
+    out = torch.empty(5, 200, dtype=torch.float32, device="cuda")
+    kernels.swiglu(gu, out)
+    g, u = gu.cpu().to(F64)[:, :200], gu.cpu().to(F64)[:, 200:]
+    close(out, g / (1 + torch.exp(-g)) * u, 1e-6, "swiglu")
+    zero = torch.zeros(1, 8, device="cuda")
+    z = torch.empty(1, 4, device="cuda")
+    kernels.swiglu(zero, z)
+    assert float(z.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("T,N,K", [(1, 64, 64), (5, 70, 100), (64, 64, 16), (130, 200, 96), (3, 384, 200)])
+@pytest.mark.parametrize("dtypes", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                    (torch.bfloat16, torch.float32)])
+def test_gemm_generic(T, N, K, dtypes):
+    from tie_amd import kernels
+
+    x = rnd(T, K, seed=5, dtype=dtypes[0]).cuda()
+    w = rnd(N, K, seed=6, scale=0.1, dtype=dtypes[1]).cuda()
+    out = torch.empty(T, N, dtype=torch.float32, device="cuda")
+    kernels.gemm_generic(x, w, out)
+    want = plain.linear(x.cpu(), w.cpu())
+    close(out, want, 2e-6, f"gemm {T}x{N}x{K}")
+    base = rnd(T, N, seed=7).cuda()
+    acc = base.clone()
+    kernels.gemm_generic(x, w, acc, accumulate=True)
+    close(acc, want + base.cpu().to(F64), 2e-6, "gemm accumulate")
+    # a row's result does not depend on the other rows of the call
+    one = torch.empty(1, N, dtype=torch.float32, device="cuda")
+    kernels.gemm_generic(x[T - 1:T].contiguous(), w, one)
+    assert torch.equal(one[0], out[T - 1])
+
+
+def paged_cache(k, v, block_size, table, num_blocks, dtype):
+    """Scatters k, v [T, KVH, Dh] of one sequence into caches [NB, KVH, bs, Dh] through ``table``."""
+    T, KVH, Dh = k.shape
+    kc = torch.full((num_blocks, KVH, block_size, Dh), float("nan"), dtype=dtype)
+    vc = torch.full((num_blocks, KVH, block_size, Dh), float("nan"), dtype=dtype)
+    for j in range(T):
+        kc[table[j // block_size], :, j % block_size] = k[j].to(dtype)
+        vc[table[j // block_size], :, j % block_size] = v[j].to(dtype)
+    return kc, vc
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
+                                         (2, 1, 256, 4), (2, 2, 512, 2)])
+def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
+    from tie_amd import kernels
+
+    T, eps, theta = 6, 1e-5, 1e4
+    qkv = rnd(T, (H + 2 * KVH) * Dh, seed=8, scale=2.0).cuda()
+    qw, kw = (1 + 0.1 * rnd(Dh, seed=9)).cuda(), (1 + 0.1 * rnd(Dh, seed=10)).cuda()
+    positions = [0, 1, 5, 77, 300, 4095]
+    slots = [9, 2, 31, 4, 17, 0]
+    inv_freq = torch.from_numpy(plain.rope_inv_freq(theta, Dh)).cuda()
+    NB = 32 // bs + 1
+    kc = torch.zeros(NB, KVH, bs, Dh, device="cuda")
+    vc = torch.zeros_like(kc)
+    q = torch.empty(T, H * Dh, device="cuda")
+    kernels.qk_norm_rope_kv_write(qkv, q, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc, vc, H, KVH, Dh, bs)
+    x = qkv.cpu()
+    q_in = x[:, :H * Dh].view(T, H, Dh)
+    k_in = x[:, H * Dh:(H + KVH) * Dh].view(T, KVH, Dh)
+    v_in = x[:, (H + KVH) * Dh:].view(T, KVH, Dh)
+    q_want = plain.rope_neox(plain.rms_norm(q_in, qw.cpu(), eps), positions, theta)
+    k_want = plain.rope_neox(plain.rms_norm(k_in, kw.cpu(), eps), positions, theta)
+    close(q.view(T, H, Dh), q_want, 2e-6, "q")
+    for t, slot in enumerate(slots):                          # ((page*KVH + h)*bs + offset)*Dh
+        close(kc[slot // bs, :, slot % bs], k_want[t], 2e-6, f"k of token {t}")
+        assert torch.equal(vc[slot // bs, :, slot % bs].cpu(), v_in[t])
+    written = torch.zeros(NB * bs, dtype=torch.bool)
+    written[slots] = True
+    assert float(kc.cpu().view(NB, KVH, bs, Dh).permute(0, 2, 1, 3).reshape(NB * bs, -1)[~written].abs().max()) == 0.0
+    # without norm weights and frequencies it is a plain copy; position 0 is the identity of the rotation
+    q2 = torch.empty_like(q)
+    kernels.qk_norm_rope_kv_write(qkv, q2, None, None, 0.0, None, i32(positions), i32(slots), kc, vc, H, KVH, Dh, bs)
+    assert torch.equal(q2, qkv[:, :H * Dh])
+    kernels.qk_norm_rope_kv_write(qkv, q2, None, None, 0.0, inv_freq, i32([0] * T), i32(slots), kc, vc, H, KVH, Dh, bs)
+    assert torch.equal(q2, qkv[:, :H * Dh])
+
+
+def attention_case(H, KVH, Dh, bs, lens_new, lens_ctx, seed, dtype=torch.float32, window=None, spike=None):
+    """Builds a batch of sequences with scattered, unordered block tables; returns kernel inputs and the plain result."""
+    rng = np.random.RandomState(seed)
+    S = len(lens_ctx)
+    MB = max(math.ceil(c / bs) for c in lens_ctx) + 1
+    NB = sum(math.ceil(c / bs) for c in lens_ctx) + 3
+    pages = list(rng.permutation(NB))
+    kc = torch.full((NB, KVH, bs, Dh), float("nan"), dtype=dtype)
+    vc = torch.full((NB, KVH, bs, Dh), float("nan"), dtype=dtype)
+    tables = np.zeros((S, MB), dtype=np.int32)
+    q_rows, want_rows, seq_of_row, query_start = [], [], [], [0]
+    for s in range(S):
+        ctx, n_new = lens_ctx[s], lens_new[s]
+        q = rnd(ctx, H, Dh, seed=seed * 100 + s)
+        k = rnd(ctx, KVH, Dh, seed=seed * 100 + s + 50)
+        v = rnd(ctx, KVH, Dh, seed=seed * 100 + s + 70)
+        if spike is not None:                               # one far key stands out for the last query
+            j = spike(ctx)
+            k[j] = 0
+            k[j, :, 0] = 30.0
+            q[ctx - 1] = 0
+            q[ctx - 1, :, 0] = 30.0
+            v[j] = 5.0
+        q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+        table = [int(pages.pop()) for _ in range(math.ceil(ctx / bs))]
+        tables[s, :len(table)] = table
+        for j in range(ctx):
+            kc[table[j // bs], :, j % bs] = k[j]
+            vc[table[j // bs], :, j % bs] = v[j]
+        full = plain.causal_attention(q, k, v, Dh ** -0.5, window)
+        q_rows.append(q[ctx - n_new:].reshape(n_new, H * Dh))
+        want_rows.append(full[ctx - n_new:].reshape(n_new, H * Dh))
+        seq_of_row += [s] * n_new
+        query_start.append(query_start[-1] + n_new)
+    kc, vc = torch.nan_to_num(kc, nan=1e30), torch.nan_to_num(vc, nan=1e30)   # unused slots hold garbage
+    return dict(q=torch.cat(q_rows).cuda().contiguous(), kc=kc.cuda(), vc=vc.cuda(), tables=torch.from_numpy(tables).cuda(),
+                query_start=i32(query_start), context_lens=i32(lens_ctx), seq_of_row=i32(seq_of_row),
+                want=torch.cat(want_rows)), S
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
+                                         (2, 1, 256, 4), (1, 1, 512, 2)])
+def test_paged_attention_generic_mixed_batch(H, KVH, Dh, bs):
+    from tie_amd import kernels
+
+    # a whole prompt, a portion that continues a cached prefix, single decoded tokens, a one-token prompt
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=[13, 5, 1, 1, 1], lens_ctx=[13, 29, 40, 300, 1], seed=3)
+    out = torch.empty_like(case["q"])
+    kernels.paged_attention_generic(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                    case["tables"], case["seq_of_row"], H, Dh ** -0.5)
+    close(out, case["want"], 1e-5, f"attention H={H} KVH={KVH} Dh={Dh}")
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "far"])
+def test_paged_attention_generic_finds_one_far_key(where):
+    from tie_amd import kernels
+
+    spike = {"first": lambda ctx: 0, "page_edge": lambda ctx: 16 * 3 - 1, "far": lambda ctx: ctx - 259}[where]
+    case, S = attention_case(4, 2, 32, 16, lens_new=[1, 7], lens_ctx=[700, 523], seed=5, spike=spike)
+    out = torch.empty_like(case["q"])
+    kernels.paged_attention_generic(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                    case["tables"], case["seq_of_row"], 4, 32 ** -0.5)
+    close(out, case["want"], 1e-5, f"spike at {where}")
+    assert float(out[0].min()) > 4.9                          # the last query really reads the marked value
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 100])
+def test_paged_attention_generic_window_edges(window):
+    from tie_amd import kernels
+
+    case, S = attention_case(4, 2, 16, 4, lens_new=[9, 1, 20], lens_ctx=[30, 41, 20], seed=7, window=window)
+    out = torch.empty_like(case["q"])
+    kernels.paged_attention_generic(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                    case["tables"], case["seq_of_row"], 4, 16 ** -0.5, window=window)
+    close(out, case["want"], 1e-5, f"window {window}")
+
+
+def test_paged_attention_generic_bfloat16_cache():
+    from tie_amd import kernels
+
+    case, S = attention_case(6, 2, 32, 16, lens_new=[11, 1], lens_ctx=[27, 90], seed=9, dtype=torch.bfloat16)
+    out = torch.empty_like(case["q"])
+    kernels.paged_attention_generic(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                    case["tables"], case["seq_of_row"], 6, 32 ** -0.5)
+    close(out, case["want"], 1e-2, "bfloat16 attention")
+
+
+def test_argmax_and_sample_kernels():
+    from tie_amd import kernels
+
+    logits = rnd(4, 1537, seed=11, scale=2.0)
+    logits[1, 900] = logits[1, 30] = 50.0                      # a tie: the lowest id
+    logits[2, 5] = float("nan")
+    logits = logits.cuda()
+    out = torch.empty(4, dtype=torch.int32, device="cuda")
+    kernels.argmax_rows(logits, out)
+    assert out.tolist() == [int(torch.argmax(logits[0])), 30, -1, int(torch.argmax(logits[3]))]
+    # frequencies of log {0.7, 0.2, 0.1} at temperature 1 (the reference's sampler test), many rows at once
+    R = 4000
+    rows = torch.log(torch.tensor([0.7, 0.2, 0.1])).repeat(R, 1).cuda()
+    g = torch.Generator().manual_seed(1)
+    uniform = torch.rand(R, generator=g, dtype=torch.float64).cuda()
+    drawn = torch.empty(R, dtype=torch.int32, device="cuda")
+    kernels.sample_rows(rows, torch.ones(R, device="cuda"), uniform, drawn)
+    freq = torch.bincount(drawn.cpu().long(), minlength=3).double() / R
+    assert freq[0] == pytest.approx(0.7, abs=0.03) and freq[1] == pytest.approx(0.2, abs=0.03)
+    # the draw inverts the cumulative sum in index order
+    want = torch.searchsorted(torch.cumsum(torch.tensor([0.7, 0.2, 0.1], dtype=torch.float64), 0) / 1.0, uniform.cpu() * 1.0,
+                              right=True).clamp(max=2)
+    assert (drawn.cpu().long() == want).float().mean() > 0.999
+
+
+def test_kernels_refuse_what_they_cannot_take():
+    from tie_amd import kernels
+    from tie_amd.errors import InvalidArgument, KernelUnavailable
+
+    with pytest.raises(KernelUnavailable, match="no CPU fallback"):
+        kernels.rms_norm(torch.zeros(2, 8), torch.ones(8), 1e-6, torch.zeros(2, 8))
+    with pytest.raises(InvalidArgument):
+        kernels.rms_norm(torch.zeros(2, 8).cuda(), torch.ones(4).cuda(), 1e-6, torch.zeros(2, 8).cuda())
+    with pytest.raises(InvalidArgument):
+        kernels.gemm_generic(torch.zeros(2, 8).cuda(), torch.zeros(4, 6).cuda(), torch.zeros(2, 4).cuda())
+    with pytest.raises(InvalidArgument, match="head_dim"):
+        kernels.qk_norm_rope_kv_write(torch.zeros(1, 3 * 1024).cuda(), torch.zeros(1, 1024).cuda(), None, None, 0.0, None,
+                                      i32([0]), i32([0]), torch.zeros(1, 1, 4, 1024).cuda(),
+                                      torch.zeros(1, 1, 4, 1024).cuda(), 1, 1, 1024, 4)
+    with pytest.raises(InvalidArgument):
+        kernels.embed(torch.zeros(4, 8, dtype=torch.float16).cuda(), i32([0]), torch.zeros(1, 8).cuda())

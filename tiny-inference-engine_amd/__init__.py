@@ -11,3 +11,11 @@ from .errors import (CapacityError, InvalidArgument, KernelUnavailable, LoadErro
                      UnsupportedError)
 
 __all__ = ["CapacityError", "InvalidArgument", "KernelUnavailable", "LoadError", "TieError", "UnsupportedError"]
+
+from .sampling.params import SamplingParams  # noqa: E402
+from .api import create_engine, generate  # noqa: E402
+from .engine.engine import Engine  # noqa: E402
+from .models.builder import load_model  # noqa: E402
+from .weights.random_init import write_random_model  # noqa: E402
+
+__all__ += ["Engine", "SamplingParams", "create_engine", "generate", "load_model", "write_random_model"]
