@@ -97,17 +97,6 @@ def test_gemm_generic(T, N, K, dtypes):
     assert torch.equal(one[0], out[T - 1])
 
 
-def paged_cache(k, v, block_size, table, num_blocks, dtype):
-    """Scatters k, v [T, KVH, Dh] of one sequence into caches [NB, KVH, bs, Dh] through ``table``."""
-    T, KVH, Dh = k.shape
-    kc = torch.full((num_blocks, KVH, block_size, Dh), float("nan"), dtype=dtype)
-    vc = torch.full((num_blocks, KVH, block_size, Dh), float("nan"), dtype=dtype)
-    for j in range(T):
-        kc[table[j // block_size], :, j % block_size] = k[j].to(dtype)
-        vc[table[j // block_size], :, j % block_size] = v[j].to(dtype)
-    return kc, vc
-
-
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
                                          (2, 1, 256, 4), (2, 2, 512, 2)])
 def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
@@ -121,7 +110,7 @@ def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
     inv_freq = torch.from_numpy(plain.rope_inv_freq(theta, Dh)).cuda()
     NB = 32 // bs + 1
     kc = torch.zeros(NB, KVH, bs, Dh, device="cuda")
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(NB, KVH, Dh, bs, device="cuda")           # values lie transposed inside a page
     q = torch.empty(T, H * Dh, device="cuda")
     kernels.qk_norm_rope_kv_write(qkv, q, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc, vc, H, KVH, Dh, bs)
     x = qkv.cpu()
@@ -133,7 +122,7 @@ def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
     close(q.view(T, H, Dh), q_want, 2e-6, "q")
     for t, slot in enumerate(slots):                          # ((page*KVH + h)*bs + offset)*Dh
         close(kc[slot // bs, :, slot % bs], k_want[t], 2e-6, f"k of token {t}")
-        assert torch.equal(vc[slot // bs, :, slot % bs].cpu(), v_in[t])
+        assert torch.equal(vc[slot // bs, :, :, slot % bs].cpu(), v_in[t])
     written = torch.zeros(NB * bs, dtype=torch.bool)
     written[slots] = True
     assert float(kc.cpu().view(NB, KVH, bs, Dh).permute(0, 2, 1, 3).reshape(NB * bs, -1)[~written].abs().max()) == 0.0
@@ -153,7 +142,7 @@ def attention_case(H, KVH, Dh, bs, lens_new, lens_ctx, seed, dtype=torch.float32
     NB = sum(math.ceil(c / bs) for c in lens_ctx) + 3
     pages = list(rng.permutation(NB))
     kc = torch.full((NB, KVH, bs, Dh), float("nan"), dtype=dtype)
-    vc = torch.full((NB, KVH, bs, Dh), float("nan"), dtype=dtype)
+    vc = torch.full((NB, KVH, Dh, bs), float("nan"), dtype=dtype)
     tables = np.zeros((S, MB), dtype=np.int32)
     q_rows, want_rows, seq_of_row, query_start = [], [], [], [0]
     for s in range(S):
@@ -173,7 +162,7 @@ def attention_case(H, KVH, Dh, bs, lens_new, lens_ctx, seed, dtype=torch.float32
         tables[s, :len(table)] = table
         for j in range(ctx):
             kc[table[j // bs], :, j % bs] = k[j]
-            vc[table[j // bs], :, j % bs] = v[j]
+            vc[table[j // bs], :, :, j % bs] = v[j]
         full = plain.causal_attention(q, k, v, Dh ** -0.5, window)
         q_rows.append(q[ctx - n_new:].reshape(n_new, H * Dh))
         want_rows.append(full[ctx - n_new:].reshape(n_new, H * Dh))
@@ -232,6 +221,74 @@ def test_paged_attention_generic_bfloat16_cache():
     close(out, case["want"], 1e-2, "bfloat16 attention")
 
 
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(16, 8), (70, 96), (384, 200), (100, 4096), (33, 1000)])
+def test_skinny_gemm_bf16(M, N, K):
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=21, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=22, scale=0.1, dtype=torch.bfloat16).cuda()
+    want = plain.linear(x.cpu(), w.cpu())
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    kernels.skinny_gemm_bf16(x, w, out)
+    close(out, want, 1e-5, f"skinny gemm {M}x{N}x{K}")
+    base = rnd(M, N, seed=23).cuda()
+    acc = base.clone()
+    kernels.skinny_gemm_bf16(x, w, acc, accumulate=True)
+    close(acc, want + base.cpu().to(F64), 1e-5, "skinny gemm accumulate")
+    half = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    kernels.skinny_gemm_bf16(x, w, half)
+    close(half, want, 5e-3, "skinny gemm bfloat16 output")
+    # a row's result does not depend on how many rows the call holds
+    one = torch.empty(1, N, dtype=torch.float32, device="cuda")
+    kernels.skinny_gemm_bf16(x[M - 1:M].contiguous(), w, one)
+    assert torch.equal(one[0], out[M - 1])
+
+
+def run_decode(case, S, H, Dh, nsplit, window=None):
+    from tie_amd import kernels
+
+    q = case["q"]
+    out = torch.full_like(q, float("nan"))
+    part_o = torch.empty(S * H * nsplit * Dh, dtype=torch.float32, device="cuda")
+    part_ml = torch.empty(S * H * nsplit * 2, dtype=torch.float32, device="cuda")
+    kernels.attention_decode_bf16(q, case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                  case["tables"], S, H, Dh ** -0.5, window, nsplit, part_o, part_ml)
+    return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
+                                         (16, 1, 64, 4), (2, 1, 256, 32)])
+@pytest.mark.parametrize("nsplit", [1, 3, 8])
+def test_attention_decode_bf16(H, KVH, Dh, bs, nsplit):
+    lens = [1, 31, 32, 33, 300, 700, 64]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=[1] * len(lens), lens_ctx=lens, seed=13, dtype=torch.bfloat16)
+    out = run_decode(case, S, H, Dh, nsplit)
+    close(out, case["want"], 1e-2, f"decode attention H={H} KVH={KVH} Dh={Dh} bs={bs} splits={nsplit}")
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "far", "last"])
+@pytest.mark.parametrize("nsplit", [1, 5])
+def test_attention_decode_bf16_finds_one_far_key(where, nsplit):
+    spike = {"first": lambda ctx: 0, "page_edge": lambda ctx: 16 * 3 - 1, "tile_edge": lambda ctx: 32 * 7,
+             "far": lambda ctx: ctx - 259, "last": lambda ctx: ctx - 2}[where]
+    case, S = attention_case(8, 2, 64, 16, lens_new=[1, 1], lens_ctx=[700, 523], seed=15, dtype=torch.bfloat16,
+                             spike=spike)
+    out = run_decode(case, S, 8, 64, nsplit)
+    close(out, case["want"], 1e-2, f"spike at {where}")
+    assert float(out.float().min()) > 4.9
+
+
+@pytest.mark.parametrize("window", [1, 5, 32, 33, 100])
+def test_attention_decode_bf16_window_edges(window):
+    lens = [30, 41, 20, 200]
+    case, S = attention_case(4, 2, 32, 4, lens_new=[1] * 4, lens_ctx=lens, seed=17, dtype=torch.bfloat16, window=window)
+    for nsplit in (1, 4):
+        out = run_decode(case, S, 4, 32, nsplit, window=window)
+        close(out, case["want"], 1e-2, f"decode window {window} splits {nsplit}")
+
+
 def test_argmax_and_sample_kernels():
     from tie_amd import kernels
 
@@ -270,6 +327,6 @@ def test_kernels_refuse_what_they_cannot_take():
     with pytest.raises(InvalidArgument, match="head_dim"):
         kernels.qk_norm_rope_kv_write(torch.zeros(1, 3 * 1024).cuda(), torch.zeros(1, 1024).cuda(), None, None, 0.0, None,
                                       i32([0]), i32([0]), torch.zeros(1, 1, 4, 1024).cuda(),
-                                      torch.zeros(1, 1, 4, 1024).cuda(), 1, 1, 1024, 4)
+                                      torch.zeros(1, 1, 1024, 4).cuda(), 1, 1, 1024, 4)
     with pytest.raises(InvalidArgument):
         kernels.embed(torch.zeros(4, 8, dtype=torch.float16).cuda(), i32([0]), torch.zeros(1, 8).cuda())

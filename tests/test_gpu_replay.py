@@ -124,3 +124,23 @@ def test_trace_run_program(folders, tmp_path):
                 r += 1
             position[e["id"]] = start + len(e["tokens"])
         assert r == data.shape[0]
+
+
+def test_recorded_decode_steps_replay_to_the_eager_result(folders):
+    """Decode steps replayed from a HIP graph give bit for bit what eager launches give, replay after
+    replay, with other steps (prompt portions, other batch shapes) and synchronisations in between."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["bfloat16"]["B"]
+    requests = th.make_requests(cfg["vocab_size"], [70, 45, 52], seed=12)
+    steps, peak = th.mixed(requests, max_live=3, seed=4, tail=24)
+    eager = TraceReplayer.from_folder(folder, "bfloat16", peak, block_size=16, use_graphs=False)
+    graphs = TraceReplayer.from_folder(folder, "bfloat16", peak, block_size=16, use_graphs=True)
+    for step in steps:
+        a = eager.run_step(step)
+        b = graphs.run_step(step)
+        torch.cuda.synchronize()
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert torch.equal(a, b), f"step {step['step']} differs between eager launches and the replayed graph"
+    assert graphs.runner.graph_replays >= 10 and eager.runner.graph_replays == 0

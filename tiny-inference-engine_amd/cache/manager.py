@@ -6,7 +6,12 @@ same slots in all planes of the group - the reference's layout
 (``src/kv/paged_kv_cache.h:27-30``, ``paged_kv_cache.cpp:91-99``) with a group
 dimension added. Per group the device tensor is
 
-    [planes][2 (K, V)][num_blocks][num_kv_heads][block_size][head_dim]
+    [planes][2 (K, V)][num_blocks][num_kv_heads][block_size * head_dim]
+
+where a key page holds one row per position (``[block_size][head_dim]``) and a
+value page is transposed (``[head_dim][block_size]``, one row per dimension):
+the matrix cores consume keys along head_dim and values along positions, and
+each gets its operand in contiguous 16-byte pieces this way.
 
 A request holds one block table per paged group: position j lives in page
 ``table[j // block_size]`` at offset ``j % block_size``. Tables grow
@@ -250,9 +255,11 @@ class CacheManager:
 
     # --------------------------------------------------------------- storage
     def kv_planes(self, group: int, plane: int):
-        """K and V of one plane: two ``[num_blocks, num_kv_heads, block_size, head_dim]`` views."""
+        """K and V of one plane: ``[num_blocks, num_kv_heads, block_size, head_dim]`` and, transposed
+        inside the page, ``[num_blocks, num_kv_heads, head_dim, block_size]``."""
         tensor = self.kv[group]
-        return tensor[plane, 0], tensor[plane, 1]
+        nb, kvh, bs, dh = tensor.shape[2:]
+        return tensor[plane, 0], tensor[plane, 1].view(nb, kvh, dh, bs)
 
     def state_plane(self, group: int, plane: int) -> torch.Tensor:
         """The states of one plane: ``[max_state_slots, *shape]``."""

@@ -80,11 +80,12 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     if (active) {
       for (int jj = g; jj < nkeys; jj += groups) {
         const int j2 = base + jj;
-        const TC* vr = v_cache +
-            ((static_cast<size_t>(table[j2 / block_size]) * KVH + kvh) * block_size + j2 % block_size) * Dh;
+        // values lie transposed inside a page: [page][kv head][dim][offset]
+        const TC* vr = v_cache + (static_cast<size_t>(table[j2 / block_size]) * KVH + kvh) * Dh * block_size +
+                       j2 % block_size;
         const float pj = p_s[jj];
-        acc0 = fmaf(pj, load_as_float(vr + d0), acc0);
-        if (wide && d0 + AT < Dh) acc1 = fmaf(pj, load_as_float(vr + d0 + AT), acc1);
+        acc0 = fmaf(pj, load_as_float(vr + static_cast<size_t>(d0) * block_size), acc0);
+        if (wide && d0 + AT < Dh) acc1 = fmaf(pj, load_as_float(vr + static_cast<size_t>(d0 + AT) * block_size), acc1);
       }
     }
     __syncthreads();                                  // p_s is rewritten by the next chunk

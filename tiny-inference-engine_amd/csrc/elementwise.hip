@@ -124,9 +124,11 @@ extern "C" int tie_cast(const void* x, int in_dtype, void* out, int out_dtype, l
 //   q, k: per-head RMSNorm over Dh with one weight vector shared by all heads,
 //         THEN rotate-half rotary: pairs (i, i + Dh/2), angle = float(pos) * inv_freq[i]
 //         (reference: src/model/qwen3.cpp:222-225, cpu_backend.cpp:161-193, backend/rope.h:9-13).
-//   q goes to q_out[t * q_row + h*Dh + d]; k (after norm and rotation) and raw v go to the
-//   paged cache at ((page*KVH + h)*block_size + offset)*Dh + d with page = slot / block_size,
-//   offset = slot % block_size (cpu_backend.cpp:235-259).
+//   q goes to q_out[t * q_row + h*Dh + d]; k (after norm and rotation) and raw v go to the paged
+//   cache with page = slot / block_size, offset = slot % block_size (cpu_backend.cpp:235-259):
+//   keys at ((page*KVH + h)*block_size + offset)*Dh + d, one row per position; values transposed
+//   inside the page, at ((page*KVH + h)*Dh + d)*block_size + offset, one row per dimension, which
+//   is the order in which the attention kernels' matrix cores consume them.
 // Norm weights or inv_freq may be null: that step is then skipped. With k_dense set, keys are
 // written there (row stride k_row) instead of into the cache; without write_kv and k_dense only
 // the query heads are processed. q_out and k_dense may alias qkv (each wave holds its head in
@@ -152,8 +154,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   if (!is_q && !is_k) {  // value head: straight copy into the cache
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
-    TC* dst = v_cache + ((static_cast<size_t>(slot / block_size) * KVH + h) * block_size + slot % block_size) * Dh;
-    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + d, load_as_float(in + d));
+    TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
+    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + static_cast<size_t>(d) * block_size, load_as_float(in + d));
     return;
   }
 

@@ -58,6 +58,7 @@ class StepBatch:
         self.host_new_tokens: List[int] = []
         self.host_context_lens: List[int] = []
         self.max_context = 0
+        self.plan_context = 0      # the context length kernels size their grids for (>= max_context)
         self.max_new_tokens = 0
         self.all_decode = False
 
@@ -90,6 +91,11 @@ class BatchBuilder:
         elif self._copied is not None:
             self._copied.synchronize()
         return self._host, self._dev
+
+    @property
+    def staging_ptr(self) -> int:
+        """Address of the device-side staging buffer; a recorded step is bound to it."""
+        return 0 if self._dev is None else self._dev.data_ptr()
 
     def build(self, entries: Sequence[StepEntry]) -> StepBatch:
         if not entries:
@@ -193,6 +199,9 @@ class BatchBuilder:
         for g in groups:
             batch.groups[g] = GroupStep(dev(("slots", g)), dev(("tables", g), (S, MB)))
         batch.max_context = max(batch.host_context_lens)
+        batch.plan_context = 1024                 # contexts are planned for in buckets: 1024, 2048, 4096, ...
+        while batch.plan_context < batch.max_context:
+            batch.plan_context *= 2
         batch.max_new_tokens = max(batch.host_new_tokens)
         batch.all_decode = batch.max_new_tokens == 1
         return batch

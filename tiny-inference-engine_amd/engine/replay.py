@@ -32,7 +32,7 @@ from .runner import ModelRunner
 
 
 class TraceReplayer:
-    def __init__(self, model: Model, max_tokens: int, block_size: int = 16):
+    def __init__(self, model: Model, max_tokens: int, block_size: int = 16, use_graphs=None):
         """``max_tokens``: the most tokens live requests hold at any time, each request's
         count rounded up to a multiple of 64 (of the block size if that is larger); the page pool
         is made for exactly this many, so pages are used again."""
@@ -43,14 +43,15 @@ class TraceReplayer:
         num_blocks = math.ceil(max_tokens / block_size)
         self.cache = CacheManager(model.cache_plan, block_size=block_size, num_blocks=num_blocks,
                                   dtype=cache_dtype, device=model.device, max_state_slots=8)
-        self.runner = ModelRunner(model, self.cache, max_seq_len=num_blocks * block_size)
+        self.runner = ModelRunner(model, self.cache, max_seq_len=num_blocks * block_size, use_graphs=use_graphs)
         self.requests: Dict[str, RequestCache] = {}
         self.lengths: Dict[str, int] = {}
 
     @classmethod
-    def from_folder(cls, folder, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0"):
+    def from_folder(cls, folder, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
+                    use_graphs=None):
         model = load_model(folder, normalize_mode(dtype), device)
-        return cls(model, max_tokens, block_size)
+        return cls(model, max_tokens, block_size, use_graphs)
 
     def run_step(self, step: dict) -> Optional[torch.Tensor]:
         """Runs one step of a trace; returns float32 logits ``[wanted, vocab]`` (on the device) or None."""

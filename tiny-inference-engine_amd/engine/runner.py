@@ -6,11 +6,19 @@ step's arrays, runs embedding, the run order and the head on the wanted rows,
 and leaves the keys and values of the new tokens in the cache
 (``src/model/qwen3.cpp:160-263`` is the reference's step). Pages must have been
 reserved by the caller; nothing is sampled here.
+
+Steps that hold only decoded tokens (one new row per sequence) are launch-bound:
+a few hundred small kernels. In bfloat16 mode such a step is recorded once per
+shape (sequences, wanted rows, context bucket) into a HIP graph and replayed
+afterwards; the step's arrays live at fixed addresses in the staging buffer,
+so a replay reads the new step's tokens, positions, slots and block tables.
+The reference gets the same effect by recording every op of a step into one
+command buffer (``src/backend/metal/metal_backend.mm:95-109``).
 """
 
 from __future__ import annotations
 
-from typing import Optional, Sequence
+from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
@@ -18,30 +26,71 @@ from ..cache.manager import CacheManager
 from ..errors import InvalidArgument
 from ..models.builder import Model
 from ..parts.base import StepContext, Workspace
-from .batch import BatchBuilder, StepEntry
+from ..weights.binder import BFLOAT16
+from .batch import BatchBuilder, StepBatch, StepEntry
+
+
+class _RecordedStep:
+    def __init__(self, graph, logits, staging_ptr, generation):
+        self.graph = graph
+        self.logits = logits
+        self.staging_ptr = staging_ptr
+        self.generation = generation
 
 
 class ModelRunner:
-    def __init__(self, model: Model, cache: CacheManager, max_seq_len: Optional[int] = None):
+    def __init__(self, model: Model, cache: CacheManager, max_seq_len: Optional[int] = None,
+                 use_graphs: Optional[bool] = None):
         if model.mode is None:
             raise InvalidArgument("the model has no weights loaded")
         if cache.plan is not model.cache_plan and cache.plan != model.cache_plan:
             raise InvalidArgument("the cache was not planned for this model")
         self.model = model
         self.cache = cache
-        self.device = model.device
+        self.device = torch.device(model.device)
         limit = model.spec.max_positions
         self.max_seq_len = min(limit, max_seq_len) if max_seq_len else limit
         self.max_blocks_per_seq = cache.blocks_for(self.max_seq_len)
         self.builder = BatchBuilder(cache, model.spec.vocab_size, self.max_blocks_per_seq, self.device)
         self.workspace = Workspace(self.device)
+        if use_graphs is None:
+            use_graphs = model.mode == BFLOAT16 and self.device.type == "cuda"
+        self.use_graphs = use_graphs
+        self._recorded: Dict[Tuple[int, int, int], _RecordedStep] = {}
+        self.graph_replays = 0
+
+    def _forward(self, batch: StepBatch) -> Optional[torch.Tensor]:
+        ctx = StepContext(batch, self.model.mode, self.device, self.workspace, self.cache, self.model.cache_plan)
+        return self.model.forward(ctx)
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """Runs one batch; returns float32 logits ``[wanted rows, vocab]`` on the device, or None."""
+        """Runs one batch; returns float32 logits ``[wanted rows, vocab]`` on the device, or None.
+
+        The returned tensor is scratch memory of the runner: it is valid until the next step.
+        """
         for e in entries:
             if e.start + len(e.tokens) > self.max_seq_len:
                 raise InvalidArgument(
                     f"a request would reach {e.start + len(e.tokens)} tokens; the limit is {self.max_seq_len}")
         batch = self.builder.build(entries)
-        ctx = StepContext(batch, self.model.mode, self.device, self.workspace, self.cache, self.model.cache_plan)
-        return self.model.forward(ctx)
+        if not (self.use_graphs and batch.all_decode and self.model.layer_hook is None):
+            return self._forward(batch)
+
+        # A decode-only step: replay its recording, or run it eagerly once and record it for next time.
+        key = (batch.num_seqs, batch.num_logit_rows, batch.plan_context)
+        staging_ptr = self.builder.staging_ptr
+        recorded = self._recorded.get(key)
+        if recorded is not None and recorded.staging_ptr == staging_ptr and \
+                recorded.generation == self.workspace.generation:
+            recorded.graph.replay()
+            self.graph_replays += 1
+            return recorded.logits
+        logits = self._forward(batch)                    # eager: does the step and settles the workspace
+        generation = self.workspace.generation
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):                    # records the same launches; nothing runs here
+            recorded_logits = self._forward(batch)
+        if self.workspace.generation == generation and self.builder.staging_ptr == staging_ptr:
+            self._recorded[key] = _RecordedStep(graph, recorded_logits, staging_ptr, generation)
+        return logits

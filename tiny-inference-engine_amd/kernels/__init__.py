@@ -27,7 +27,13 @@ _SOURCES = {
     "elementwise": ("tie_elementwise", "elementwise.hip"),
     "gemm_generic": ("tie_gemm_generic", "gemm_generic.hip"),
     "attention_generic": ("tie_attention_generic", "attention_generic.hip"),
+    "skinny_gemm_bf16": ("tie_skinny_gemm_bf16", "skinny_gemm_bf16.hip"),
 }
+# libraries compiled once per head size: key -> (file stem prefix, source)
+_PER_HEAD_DIM = {
+    "attention_decode_bf16": ("tie_attention_decode_bf16", "attention_decode_bf16.hip"),
+}
+MFMA_HEAD_DIMS = tuple(range(16, 257, 16))   # head sizes the matrix-core attention kernels are built for
 
 _SIGNATURES = {
     "elementwise": {
@@ -50,26 +56,48 @@ _SIGNATURES = {
                                         _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                                         _c_int, _c_void],
     },
+    "skinny_gemm_bf16": {
+        "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    },
+    "attention_decode_bf16": {
+        "tie_attention_decode_head_dim": [],
+        "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                      _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                      _c_void],
+    },
 }
 
 _libs = {}
 
 
-def library_list(extra_defines=None):
-    """``(name, source, defines)`` of every library, for building them all."""
-    return [(stem, source, {}) for stem, source in _SOURCES.values()]
+def library_list(head_dims=(16, 32, 64, 128)):
+    """``(name, source, defines)`` of every library, for building them all up front.
+
+    The per-head-size libraries are listed for ``head_dims``; any other head size is compiled the
+    first time a model with it runs.
+    """
+    libs = [(stem, source, {}) for stem, source in _SOURCES.values()]
+    for stem, source in _PER_HEAD_DIM.values():
+        for d in head_dims:
+            libs.append((f"{stem}_hd{d}", source, {"HEAD_DIM": d}))
+    return libs
 
 
-def _lib(key: str):
-    lib = _libs.get(key)
+def _lib(key: str, head_dim: int = 0):
+    cache_key = (key, head_dim)
+    lib = _libs.get(cache_key)
     if lib is None:
-        stem, source = _SOURCES[key]
-        lib = build.load_library(stem, source)
+        if head_dim:
+            stem, source = _PER_HEAD_DIM[key]
+            lib = build.load_library(f"{stem}_hd{head_dim}", source, {"HEAD_DIM": head_dim})
+        else:
+            stem, source = _SOURCES[key]
+            lib = build.load_library(stem, source)
         for fn, argtypes in _SIGNATURES[key].items():
             f = getattr(lib, fn)
             f.argtypes = argtypes
             f.restype = _c_int
-        _libs[key] = lib
+        _libs[cache_key] = lib
     return lib
 
 
@@ -106,6 +134,16 @@ def _gpu_strided(t: torch.Tensor, name: str) -> torch.Tensor:
     if t.stride(1) != 1 or t.stride(0) < t.shape[1]:
         raise InvalidArgument(f"{name} must have contiguous rows")
     return t
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, KVH: int, block_size: int, Dh: int) -> None:
+    """Keys ``[pages, kv heads, block_size, head_dim]``; values transposed in the page ``[pages, kv heads, head_dim, block_size]``."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.dtype != v_cache.dtype or \
+            tuple(k_cache.shape[1:]) != (KVH, block_size, Dh) or \
+            tuple(v_cache.shape) != (k_cache.shape[0], KVH, Dh, block_size):
+        raise InvalidArgument(f"KV cache planes {list(k_cache.shape)} / {list(v_cache.shape)} do not fit "
+                              f"{KVH} kv heads, block size {block_size}, head_dim {Dh} "
+                              f"(keys [pages, heads, block, dim], values [pages, heads, dim, block])")
 
 
 def _code(t: torch.Tensor, name: str) -> int:
@@ -203,9 +241,30 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate
         _code(out, "matmul output"), int(accumulate), T, N, K, _stream()), "gemm_generic")
 
 
+def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores."""
+    _gpu(x, "matmul input")
+    _gpu(w, "matmul weight")
+    _gpu(out, "matmul output")
+    M, K = x.shape
+    N, K2 = w.shape
+    if K != K2 or tuple(out.shape) != (M, N):
+        raise InvalidArgument(f"matmul: input {list(x.shape)}, weight {list(w.shape)}, output {list(out.shape)}")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise InvalidArgument("skinny_gemm_bf16 takes bfloat16 operands")
+    if M > 64 or K % 8:
+        raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows and K % 8 == 0, got M={M}, K={K}")
+    _check(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16(
+        x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), M, N, K,
+        _stream()), "skinny_gemm_bf16")
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     """out (+)= x @ w.T, on the fastest kernel that takes these operands."""
-    gemm_generic(x, w, out, accumulate)
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= 64 and x.shape[1] % 8 == 0:
+        skinny_gemm_bf16(x, w, out, accumulate)
+    else:
+        gemm_generic(x, w, out, accumulate)
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
@@ -253,10 +312,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _i32(slots, "slot mapping", T)
         _gpu(k_cache, "k cache")
         _gpu(v_cache, "v cache")
-        if k_cache.shape != v_cache.shape or k_cache.dtype != v_cache.dtype or k_cache.dim() != 4 or \
-                k_cache.shape[1] != KVH or k_cache.shape[2] != block_size or k_cache.shape[3] != Dh:
-            raise InvalidArgument(f"KV cache planes {list(k_cache.shape)} / {list(v_cache.shape)} do not fit "
-                                  f"{KVH} kv heads, block size {block_size}, head_dim {Dh}")
+        _check_cache(k_cache, v_cache, KVH, block_size, Dh)
         cache_code = _code(k_cache, "k cache")
     _check(_lib("elementwise").tie_qk_norm_rope_kv_write(
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
@@ -276,6 +332,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _gpu(k_cache, "k cache")
     _gpu(v_cache, "v cache")
     NB, KVH, bs, Dh = k_cache.shape
+    _check_cache(k_cache, v_cache, KVH, bs, Dh)
     T = q.shape[0]
     H = num_heads
     if tuple(q.shape) != (T, H * Dh) or tuple(out.shape) != (T, H * Dh):
@@ -322,12 +379,71 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
                                           out.data_ptr(), R, V, _stream()), "sample")
 
 
+def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
+    """How many ways the keys of each sequence are split so that a decode step fills the GPU."""
+    target_waves = 1024
+    by_occupancy = -(-target_waves // max(1, num_seqs * num_kv_heads))
+    by_length = max(1, max_context // 128)          # at least four 32-key tiles a split
+    return max(1, min(by_occupancy, by_length))
+
+
+def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                          query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
+                          num_seqs: int, num_heads: int, scale: float, window: Optional[int], nsplit: int,
+                          part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                          seq_ids: Optional[torch.Tensor] = None) -> None:
+    """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all)."""
+    _gpu(q, "queries")
+    _gpu(out, "attention output")
+    _gpu(k_cache, "k cache")
+    _gpu(v_cache, "v cache")
+    NB, KVH, bs, Dh = k_cache.shape
+    _check_cache(k_cache, v_cache, KVH, bs, Dh)
+    H = num_heads
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise InvalidArgument("attention_decode_bf16 takes bfloat16 queries, cache and output")
+    if q.shape[1] != H * Dh or out.shape != q.shape:
+        raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
+    if Dh not in MFMA_HEAD_DIMS or H % KVH or H // KVH > 16 or bs % 4:
+        raise InvalidArgument(f"attention_decode_bf16 takes head sizes in steps of 16 up to 256, at most 16 query heads "
+                              f"a KV head and block sizes in steps of 4; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+    _i32(query_start, "query_start")
+    _i32(context_lens, "context_lens")
+    _i32(block_tables, "block tables")
+    if seq_ids is not None:
+        _i32(seq_ids, "sequence ids", num_seqs)
+    if nsplit > 1:
+        _f32(part_o, "split accumulators")
+        _f32(part_ml, "split maxima and sums")
+        if part_o.numel() < num_seqs * H * nsplit * Dh or part_ml.numel() < num_seqs * H * nsplit * 2:
+            raise InvalidArgument("the buffers for the splits are too small")
+    lib = _lib("attention_decode_bf16", Dh)
+    _check(lib.tie_attention_decode_bf16(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
+        query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
+        block_tables.shape[1], float(scale), int(window or 0), nsplit, _stream()), "attention_decode_bf16")
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
-                    num_heads: int, scale: float, window: Optional[int] = None) -> None:
+                    num_heads: int, scale: float, window: Optional[int] = None, scratch=None) -> None:
     """Causal attention over the paged cache for one step's batch, on the fastest kernel that takes it.
 
     ``step`` is the cache group's view of the step (block tables), ``batch`` the step's arrays
-    (query_start, context_lens, seq_of_row).
+    (query_start, context_lens, seq_of_row) and host-side numbers; ``scratch(name, shape, dtype)``
+    hands out workspace for the partial results of split keys.
     """
+    NB, KVH, bs, Dh = k_cache.shape
+    fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
+            and num_heads % KVH == 0 and num_heads // KVH <= 16 and bs % 4 == 0)
+    if fast and batch.all_decode and scratch is not None:
+        S = batch.num_seqs
+        nsplit = decode_splits(S, KVH, batch.plan_context)
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = scratch("attention.split_o", (S * num_heads * nsplit * Dh,), torch.float32)
+            part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
+        attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
+                              S, num_heads, scale, window, nsplit, part_o, part_ml)
+        return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window)

@@ -103,5 +103,6 @@ class PagedAttention(Mixer):
                 cache.v_cache, H, KVH, Dh, cache.block_size, write_kv=cache.writes)
 
         attn = ctx.scratch("attention.out", (T, self.q_dim))
-        kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window)
+        kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window,
+                                scratch=ctx.scratch)
         self.out(attn, residual, accumulate=True)

@@ -111,6 +111,7 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
+        self.generation = 0   # grows whenever a buffer is replaced: recorded steps are then stale
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         numel = 1
@@ -121,6 +122,7 @@ class Workspace:
         if buf is None or buf.numel() < numel:
             buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
+            self.generation += 1
         return buf[:numel].view(*shape)
 
     def nbytes(self) -> int:
