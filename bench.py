@@ -1,0 +1,222 @@
+"""Decode and prefill throughput of the engine on one MI355X, Qwen3-8B shape, random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line. A "step" is one decode step of the engine (schedule, build the batch, run
+the model, sample greedily) at the default batch of 8 with every sequence near the benchmark
+context length; ``value`` is decoded tokens a second. The same line carries
+
+* ``prefill``: tokens a second of one 2048-token prompt run as one step, and the fraction of the
+  bf16 MFMA peak its flops reach;
+* ``roofline``: the bytes a decode step has to read (every weight it uses once, and the cache of
+  the live requests) divided by its time, against the HBM peak;
+* ``points``: decoded tokens a second at batch 1 and at batch 64.
+
+The sizes are those of a Qwen3-8B config.json; weights are random (N(0, 0.02), norm weights
+1 + U(-0.1, 0.1)) and token ids are uniform, since neither checkpoints nor datasets exist here.
+"""
+
+import argparse
+import json
+import sys
+import time
+
+QWEN3_8B = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 36, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 128, "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 40960,
+}
+BLOCK_SIZE = 16
+PREFILL_TOKENS = 2048
+PEAK_HBM_GBS = 8000.0          # MI355X: 8 TB/s
+PEAK_FLOPS = {"bf16": 2.5e15}  # dense MFMA
+
+
+def log(message):
+    print(f"[bench] {message}", file=sys.stderr, flush=True)
+
+
+def build_model(cfg, seed=0):
+    import torch
+    from tie_amd.models import expected_tensors_for_config, load_model_from_tensors
+    from tie_amd.weights.random_init import random_tensors
+
+    specs = [s for s in expected_tensors_for_config(cfg) if not s.optional]
+    tensors = dict(random_tensors(specs, seed, torch.bfloat16, device="cuda"))
+    model = load_model_from_tensors(cfg, tensors, "bfloat16", "cuda:0")
+    del tensors
+    torch.cuda.empty_cache()
+    return model
+
+
+def weight_bytes_per_step(cfg, batch):
+    """Bytes of weights one decode step reads: every matrix once, the embedding rows of the batch, the norms."""
+    D, I, V, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    Q = cfg["num_attention_heads"] * cfg["head_dim"]
+    KV = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = (Q + 2 * KV) * D + D * Q + 2 * I * D + D * I
+    matrices = (L * per_layer + V * D) * 2
+    norms = (L * (2 * D + 2 * cfg["head_dim"]) + D) * 4
+    return matrices + norms + batch * D * 2
+
+
+def kv_bytes_per_token(cfg):
+    return 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * 2
+
+
+def prefill_flops(cfg, T, R=1):
+    D, I, V, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    Q = cfg["num_attention_heads"] * cfg["head_dim"]
+    KV = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = (Q + 2 * KV) * D + D * Q + 2 * I * D + D * I
+    gemm = 2 * T * L * per_layer + 2 * R * V * D
+    attention = 2 * T * T * cfg["head_dim"] * cfg["num_attention_heads"] * L   # causal: QK^T and PV over T^2 / 2 pairs
+    return gemm + attention
+
+
+def make_engine(model, batch, context, max_tokens_per_step):
+    from tie_amd.api import create_engine
+
+    blocks = batch * (-(-context // BLOCK_SIZE) + 1) + 8
+    return create_engine(model, kv_blocks=blocks, block_size=BLOCK_SIZE, max_seqs=max(batch, 1),
+                         max_tokens_per_step=max(max_tokens_per_step, batch), policy="fcfs", watermark_blocks=0,
+                         max_seq_len=context)
+
+
+def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
+    """Decode ``steps`` timed steps at ``batch`` sequences whose context ends at ``context`` tokens."""
+    import random
+
+    import torch
+    from tie_amd.engine.sequence import SeqState
+    from tie_amd.sampling.params import SamplingParams
+
+    engine = make_engine(model, batch, context, chunk)
+    rng = random.Random(batch)
+    prompt_len = context - (steps + warmup) - 1
+    ids = [engine.add_request([rng.randrange(cfg["vocab_size"]) for _ in range(prompt_len)],
+                              SamplingParams(max_tokens=steps + warmup + 1)) for _ in range(batch)]
+    started = time.perf_counter()
+    while any(engine.sequence(i).state != SeqState.DECODING for i in ids):
+        engine.step()
+    torch.cuda.synchronize()
+    log(f"batch {batch}: prefilled {batch * prompt_len} tokens in {time.perf_counter() - started:.1f} s")
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    first_context = engine.sequence(ids[0]).num_computed + 1
+    start = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - start
+    last_context = engine.sequence(ids[0]).num_computed
+    assert all(engine.sequence(i).num_generated == warmup + steps + 1 for i in ids), "a sequence fell behind"
+    mean_context = (first_context + last_context) / 2
+    replays = engine.runner.graph_replays
+    del engine
+    torch.cuda.empty_cache()
+    return seconds, mean_context, replays
+
+
+def measure_prefill(model, cfg, tokens, repeats=3):
+    import random
+
+    import torch
+    from tie_amd.sampling.params import SamplingParams
+
+    engine = make_engine(model, 1, tokens + 16, tokens)
+    rng = random.Random(7)
+    best = None
+    for i in range(repeats + 1):               # the first run warms up
+        prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(tokens)]
+        sid = engine.add_request(prompt, SamplingParams(max_tokens=1))
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        engine.step()                          # the whole prompt in one step, one logits row, one sampled token
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - start
+        assert engine.sequence(sid).num_generated == 1
+        engine.release(sid)
+        if i > 0:
+            best = seconds if best is None else min(best, seconds)
+    del engine
+    torch.cuda.empty_cache()
+    return best
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
+    parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the 36 of the shape (0 = all)")
+    parser.add_argument("--skip-points", action="store_true", help="skip batch 1, batch 64 and the prefill")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures a single-GPU engine: --gpus {args.gpus} is not supported, run it with --gpus 1")
+        return 2
+
+    import torch
+
+    import pathlib
+    sys.path.insert(0, str(pathlib.Path(__file__).resolve().parent))
+    import tie_amd  # noqa: F401
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 1
+    cfg = dict(QWEN3_8B)
+    layers_of_shape = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    log(f"building {cfg['num_hidden_layers']} layers of the Qwen3-8B shape with random bf16 weights")
+    started = time.perf_counter()
+    model = build_model(cfg)
+    log(f"model ready in {time.perf_counter() - started:.1f} s")
+
+    chunk = 2048
+    seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk)
+    ms_per_step = seconds / args.steps * 1e3
+    value = args.batch * args.steps / seconds
+    step_bytes = weight_bytes_per_step(cfg, args.batch) + args.batch * mean_context * kv_bytes_per_token(cfg)
+    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+    log(f"decode batch {args.batch}: {ms_per_step:.3f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s ({replays} replays)")
+
+    result = {
+        "metric": "decode tok/s @ batch 8, Qwen3-8B bf16 (plus prefill tok/s @ 2048 and batch 1/64 points)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "model": "Qwen3-8B shape, random weights", "layers": layers_of_shape, "layers_run": cfg["num_hidden_layers"],
+            "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+            "global_batch": args.batch, "seq_len": args.context, "kv_block": BLOCK_SIZE, "kv_dtype": "bf16",
+            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU", "sampling": "greedy",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.skip_points:
+        t = measure_prefill(model, cfg, PREFILL_TOKENS)
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        result["prefill"] = {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS, "ms": round(t * 1e3, 3),
+                             "frac": round(flops / t / PEAK_FLOPS["bf16"], 4)}
+        log(f"prefill {PREFILL_TOKENS}: {t * 1e3:.2f} ms, {PREFILL_TOKENS / t:.0f} tok/s, "
+            f"{flops / t / 1e12:.1f} TFLOP/s")
+        points = {}
+        for b in (1, 64):
+            s, _, _ = measure_decode(model, cfg, b, args.context, max(8, args.steps // 2), args.warmup, chunk)
+            points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 2)
+            log(f"decode batch {b}: {points[f'decode_b{b}']:.1f} tok/s")
+        result["points"] = points
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -246,6 +246,32 @@ def test_skinny_gemm_bf16(M, N, K):
     assert torch.equal(one[0], out[M - 1])
 
 
+
+@pytest.mark.parametrize("M,N,K", [(65, 70, 96), (100, 384, 200), (128, 128, 64), (300, 200, 4096), (2048, 256, 512),
+                                   (257, 129, 72), (1, 64, 64)])
+@pytest.mark.parametrize("tile", [1, 2])
+def test_gemm_bf16(M, N, K, tile):
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=31, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=32, scale=0.1, dtype=torch.bfloat16).cuda()
+    want = plain.linear(x.cpu(), w.cpu())
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    kernels.gemm_bf16(x, w, out, tile=tile)
+    close(out, want, 1e-5, f"gemm {M}x{N}x{K} tile {tile}")
+    base = rnd(M, N, seed=33).cuda()
+    acc = base.clone()
+    kernels.gemm_bf16(x, w, acc, accumulate=True, tile=tile)
+    close(acc, want + base.cpu().to(F64), 1e-5, "gemm accumulate")
+    half = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    kernels.gemm_bf16(x, w, half, tile=tile)
+    close(half, want, 5e-3, "gemm bfloat16 output")
+    # a row's result does not depend on the other rows of the call
+    few = torch.empty(min(M, 3), N, dtype=torch.float32, device="cuda")
+    kernels.gemm_bf16(x[:3].contiguous(), w, few, tile=tile)
+    assert torch.equal(few, out[:3])
+
+
 def run_decode(case, S, H, Dh, nsplit, window=None):
     from tie_amd import kernels
 
@@ -287,6 +313,47 @@ def test_attention_decode_bf16_window_edges(window):
     for nsplit in (1, 4):
         out = run_decode(case, S, 4, 32, nsplit, window=window)
         close(out, case["want"], 1e-2, f"decode window {window} splits {nsplit}")
+
+
+
+def run_prefill(case, H, KVH, lens_new, window=None):
+    from tie_amd import kernels
+
+    q = case["q"]
+    out = torch.full_like(q, float("nan"))
+    items = torch.tensor(kernels.prefill_items(lens_new, H // KVH), dtype=torch.int32).cuda()
+    kernels.attention_prefill_bf16(q, case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                   case["tables"], items, H, (q.shape[1] // H) ** -0.5, window)
+    return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
+                                         (16, 1, 64, 4), (12, 2, 64, 16), (2, 1, 256, 32)])
+def test_attention_prefill_bf16_mixed_batch(H, KVH, Dh, bs):
+    # a whole prompt, a portion that continues a cached prefix, single decoded tokens, a one-token prompt, 70 rows
+    lens_new, lens_ctx = [13, 5, 1, 1, 1, 70, 2], [13, 29, 40, 300, 1, 150, 33]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=lens_new, lens_ctx=lens_ctx, seed=23, dtype=torch.bfloat16)
+    out = run_prefill(case, H, KVH, lens_new)
+    close(out, case["want"], 1e-2, f"prefill attention H={H} KVH={KVH} Dh={Dh} bs={bs}")
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "far", "last"])
+def test_attention_prefill_bf16_finds_one_far_key(where):
+    spike = {"first": lambda ctx: 0, "page_edge": lambda ctx: 16 * 3 - 1, "tile_edge": lambda ctx: 32 * 7,
+             "far": lambda ctx: ctx - 259, "last": lambda ctx: ctx - 2}[where]
+    lens_new = [40, 7]
+    case, S = attention_case(8, 2, 64, 16, lens_new=lens_new, lens_ctx=[700, 523], seed=25, dtype=torch.bfloat16, spike=spike)
+    out = run_prefill(case, 8, 2, lens_new)
+    close(out, case["want"], 1e-2, f"spike at {where}")
+    assert float(out[39].float().min()) > 4.9 and float(out[46].float().min()) > 4.9
+
+
+@pytest.mark.parametrize("window", [1, 5, 32, 33, 100])
+def test_attention_prefill_bf16_window_edges(window):
+    lens_new, lens_ctx = [9, 1, 20, 50], [30, 41, 20, 200]
+    case, S = attention_case(4, 2, 32, 4, lens_new=lens_new, lens_ctx=lens_ctx, seed=27, dtype=torch.bfloat16, window=window)
+    out = run_prefill(case, 4, 2, lens_new, window=window)
+    close(out, case["want"], 1e-2, f"prefill window {window}")
 
 
 def test_argmax_and_sample_kernels():

@@ -61,6 +61,7 @@ class StepBatch:
         self.plan_context = 0      # the context length kernels size their grids for (>= max_context)
         self.max_new_tokens = 0
         self.all_decode = False
+        self.memo: Dict = {}       # per-step values kernels derive once and share between layers
 
 
 def _align(n: int, to: int = 4) -> int:

@@ -28,10 +28,12 @@ _SOURCES = {
     "gemm_generic": ("tie_gemm_generic", "gemm_generic.hip"),
     "attention_generic": ("tie_attention_generic", "attention_generic.hip"),
     "skinny_gemm_bf16": ("tie_skinny_gemm_bf16", "skinny_gemm_bf16.hip"),
+    "gemm_bf16": ("tie_gemm_bf16", "gemm_bf16.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
     "attention_decode_bf16": ("tie_attention_decode_bf16", "attention_decode_bf16.hip"),
+    "attention_prefill_bf16": ("tie_attention_prefill_bf16", "attention_prefill_bf16.hip"),
 }
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))   # head sizes the matrix-core attention kernels are built for
 
@@ -59,6 +61,14 @@ _SIGNATURES = {
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
+    "gemm_bf16": {
+        "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    },
+    "attention_prefill_bf16": {
+        "tie_attention_prefill_rows_per_item": [_c_int],
+        "tie_attention_prefill_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int,
+                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+    },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
         "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
@@ -70,7 +80,7 @@ _SIGNATURES = {
 _libs = {}
 
 
-def library_list(head_dims=(16, 32, 64, 128)):
+def library_list(head_dims=(16, 32, 48, 64, 80, 128, 256)):
     """``(name, source, defines)`` of every library, for building them all up front.
 
     The per-head-size libraries are listed for ``head_dims``; any other head size is compiled the
@@ -259,10 +269,36 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
         _stream()), "skinny_gemm_bf16")
 
 
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0) -> None:
+    """out (+)= x @ w.T for bfloat16 operands on the matrix cores, any number of rows; K % 8 == 0.
+
+    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x128; 0 lets the kernel choose).
+    """
+    _gpu(x, "matmul input")
+    _gpu(w, "matmul weight")
+    _gpu(out, "matmul output")
+    M, K = x.shape
+    N, K2 = w.shape
+    if K != K2 or tuple(out.shape) != (M, N):
+        raise InvalidArgument(f"matmul: input {list(x.shape)}, weight {list(w.shape)}, output {list(out.shape)}")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise InvalidArgument("gemm_bf16 takes bfloat16 operands")
+    if K % 8:
+        raise InvalidArgument(f"gemm_bf16 takes K % 8 == 0, got K={K}")
+    if accumulate and out.dtype != torch.float32:
+        raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only")
+    _check(_lib("gemm_bf16").tie_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
+                                           int(accumulate), M, N, K, tile, _stream()), "gemm_bf16")
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     """out (+)= x @ w.T, on the fastest kernel that takes these operands."""
-    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= 64 and x.shape[1] % 8 == 0:
-        skinny_gemm_bf16(x, w, out, accumulate)
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and \
+            not (accumulate and out.dtype != torch.float32):
+        if x.shape[0] <= 64:
+            skinny_gemm_bf16(x, w, out, accumulate)
+        else:
+            gemm_bf16(x, w, out, accumulate)
     else:
         gemm_generic(x, w, out, accumulate)
 
@@ -424,6 +460,53 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         block_tables.shape[1], float(scale), int(window or 0), nsplit, _stream()), "attention_decode_bf16")
 
 
+def prefill_items(new_tokens, group_size: int) -> "list":
+    """Work items ``(sequence, first 16-row tile)`` of the prefill attention kernel for one step.
+
+    An item covers 16, 32 or 64 consecutive new rows of a sequence, depending on how many query
+    heads share a KV head (up to four (head, row tile) pairs run side by side in one wave).
+    """
+    heads_at_once = min(group_size, 4)
+    tiles_per_item = max(1, 4 // heads_at_once)
+    rows = 16 * tiles_per_item
+    items = []
+    for s, n in enumerate(new_tokens):
+        for j in range(-(-n // rows)):
+            items.append((s, j * tiles_per_item))
+    return items
+
+
+def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                           query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
+                           items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None) -> None:
+    """Causal attention of the new rows of the sequences ``items`` names over their cached keys."""
+    _gpu(q, "queries")
+    _gpu(out, "attention output")
+    _gpu(k_cache, "k cache")
+    _gpu(v_cache, "v cache")
+    NB, KVH, bs, Dh = k_cache.shape
+    _check_cache(k_cache, v_cache, KVH, bs, Dh)
+    H = num_heads
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise InvalidArgument("attention_prefill_bf16 takes bfloat16 queries, cache and output")
+    if q.shape[1] != H * Dh or out.shape != q.shape:
+        raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
+    if Dh not in MFMA_HEAD_DIMS or H % KVH or bs % 4:
+        raise InvalidArgument(f"attention_prefill_bf16 takes head sizes in steps of 16 up to 256 and block sizes in "
+                              f"steps of 4; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+    _i32(query_start, "query_start")
+    _i32(context_lens, "context_lens")
+    _i32(block_tables, "block tables")
+    _i32(items, "work items")
+    if items.dim() != 2 or items.shape[1] != 2 or items.shape[0] == 0:
+        raise InvalidArgument("work items must be a non-empty [n, 2] tensor")
+    lib = _lib("attention_prefill_bf16", Dh)
+    _check(lib.tie_attention_prefill_bf16(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
+        context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
+        block_tables.shape[1], float(scale), int(window or 0), _stream()), "attention_prefill_bf16")
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
                     num_heads: int, scale: float, window: Optional[int] = None, scratch=None) -> None:
     """Causal attention over the paged cache for one step's batch, on the fastest kernel that takes it.
@@ -434,8 +517,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """
     NB, KVH, bs, Dh = k_cache.shape
     fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
-            and num_heads % KVH == 0 and num_heads // KVH <= 16 and bs % 4 == 0)
-    if fast and batch.all_decode and scratch is not None:
+            and num_heads % KVH == 0 and bs % 4 == 0 and scratch is not None)
+    if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
         nsplit = decode_splits(S, KVH, batch.plan_context)
         part_o = part_ml = None
@@ -444,6 +527,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
         attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                               S, num_heads, scale, window, nsplit, part_o, part_ml)
+        return
+    if fast:
+        key = ("prefill_items", num_heads // KVH)
+        items = batch.memo.get(key)
+        if items is None:          # the same for every layer of the step: built once
+            host = torch.tensor(prefill_items(batch.host_new_tokens, num_heads // KVH), dtype=torch.int32)
+            items = batch.memo[key] = host.to(q.device)
+        attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
+                               items, num_heads, scale, window)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window)
