@@ -85,7 +85,13 @@ def make_engine(model, batch, context, max_tokens_per_step):
 
 
 def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
-    """Decode ``steps`` timed steps at ``batch`` sequences whose context ends at ``context`` tokens."""
+    """Times ``steps`` decode steps of ``batch`` sequences whose contexts end at (just below) ``context`` tokens.
+
+    The prompts are prefilled through the engine first (untimed). Sequences that finish their prompt
+    early decode while the others still prefill, so every prompt is shortened by the number of steps
+    the prefill phase takes: no sequence outgrows ``context`` before the timed steps are over.
+    Returns (seconds, mean context length over the timed steps and sequences, graph replays).
+    """
     import random
 
     import torch
@@ -94,30 +100,39 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
 
     engine = make_engine(model, batch, context, chunk)
     rng = random.Random(batch)
-    prompt_len = context - (steps + warmup) - 1
+    slack = -(-batch * context // chunk) + batch + 2          # steps the prefill phase may take
+    prompt_len = context - (steps + warmup) - slack - 1
+    assert prompt_len > 0, "context too short for this many steps"
     ids = [engine.add_request([rng.randrange(cfg["vocab_size"]) for _ in range(prompt_len)],
-                              SamplingParams(max_tokens=steps + warmup + 1)) for _ in range(batch)]
+                              SamplingParams(max_tokens=steps + warmup + slack + 1)) for _ in range(batch)]
     started = time.perf_counter()
+    last_log = started
     while any(engine.sequence(i).state != SeqState.DECODING for i in ids):
         engine.step()
+        if time.perf_counter() - last_log > 20:
+            done = sum(engine.sequence(i).state == SeqState.DECODING for i in ids)
+            log(f"batch {batch}: prefilling, {done} of {batch} sequences done")
+            last_log = time.perf_counter()
     torch.cuda.synchronize()
-    log(f"batch {batch}: prefilled {batch * prompt_len} tokens in {time.perf_counter() - started:.1f} s")
+    log(f"batch {batch}: prefilled {batch * prompt_len} tokens in {time.perf_counter() - started:.1f} s "
+        f"({engine.stats().steps} steps)")
     for _ in range(warmup):
         engine.step()
     torch.cuda.synchronize()
-    first_context = engine.sequence(ids[0]).num_computed + 1
+    first = sum(engine.sequence(i).num_computed + 1 for i in ids) / batch
     start = time.perf_counter()
     for _ in range(steps):
         engine.step()
     torch.cuda.synchronize()
     seconds = time.perf_counter() - start
-    last_context = engine.sequence(ids[0]).num_computed
-    assert all(engine.sequence(i).num_generated == warmup + steps + 1 for i in ids), "a sequence fell behind"
-    mean_context = (first_context + last_context) / 2
+    last = sum(engine.sequence(i).num_computed for i in ids) / batch
+    assert all(engine.sequence(i).state == SeqState.DECODING for i in ids), "a sequence finished during the timed steps"
+    assert max(engine.sequence(i).num_computed for i in ids) <= context
+    assert engine.stats().preemptions == 0
     replays = engine.runner.graph_replays
     del engine
     torch.cuda.empty_cache()
-    return seconds, mean_context, replays
+    return seconds, (first + last) / 2, replays
 
 
 def measure_prefill(model, cfg, tokens, repeats=3):
@@ -178,7 +193,7 @@ def main():
     model = build_model(cfg)
     log(f"model ready in {time.perf_counter() - started:.1f} s")
 
-    chunk = 2048
+    chunk = 8192
     seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk)
     ms_per_step = seconds / args.steps * 1e3
     value = args.batch * args.steps / seconds

@@ -88,41 +88,63 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;   // elements of one page, K or V
   const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
 
+  // Fragments of one 32-key tile: keys for the first product (two 16-key sub-tiles), values for the second.
+  // Positions are clamped to pos for the address only; what lies beyond pos is masked in the softmax.
+  auto load_keys = [&](int base, Frag (&kf)[2][KSTEPS]) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kp = min(base + u * 16 + col, pos);
+      const bf16_t* kr = k_cache + static_cast<size_t>(table[kp / block_size]) * page_stride + head_off +
+                         static_cast<size_t>(kp % block_size) * DH;
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) {
+        const int d = st * 32 + quad * 8;
+        kf[u][st].u4 = d < DH ? *reinterpret_cast<const uint4*>(kr + d) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto load_values = [&](int base, Frag (&vf)[DTILES]) {
+    const int k0 = min(base + quad * 4, pos);               // a run of 4 positions inside one page
+    const int k1 = min(base + 16 + quad * 4, pos);
+    const bf16_t* v0 = v_cache + static_cast<size_t>(table[k0 / block_size]) * page_stride + head_off +
+                       (k0 % block_size) / 4 * 4;
+    const bf16_t* v1 = v_cache + static_cast<size_t>(table[k1 / block_size]) * page_stride + head_off +
+                       (k1 % block_size) / 4 * 4;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+      const size_t d_off = static_cast<size_t>(dt * 16 + col) * block_size;
+      vf[dt].u2[0] = *reinterpret_cast<const uint2*>(v0 + d_off);
+      vf[dt].u2[1] = *reinterpret_cast<const uint2*>(v1 + d_off);
+    }
+  };
+
+  // The loads of tile t + 1 are issued before the arithmetic of tile t, so memory latency and the
+  // matrix cores overlap.
+  Frag kf[2][KSTEPS], vf[DTILES], kf_next[2][KSTEPS], vf_next[DTILES];
+  if (tile_begin < tile_end) {
+    load_keys(tile_begin * 32, kf_next);
+    load_values(tile_begin * 32, vf_next);
+  }
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const int base = tile * 32;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) kf[u][st] = kf_next[u][st];
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) vf[dt] = vf_next[dt];
+    if (tile + 1 < tile_end) {
+      load_keys(base + 32, kf_next);
+      load_values(base + 32, vf_next);
+    }
     // ---- first product: two 16-key tiles
     floatx4 sc[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int kp = min(base + u * 16 + col, pos);          // clamped: rows beyond pos are masked below
-      const bf16_t* kr = k_cache + static_cast<size_t>(table[kp / block_size]) * page_stride + head_off +
-                         static_cast<size_t>(kp % block_size) * DH;
-      Frag kf[KSTEPS];
-#pragma unroll
-      for (int st = 0; st < KSTEPS; ++st) {
-        const int d = st * 32 + quad * 8;
-        kf[st].u4 = d < DH ? *reinterpret_cast<const uint4*>(kr + d) : make_uint4(0, 0, 0, 0);
-      }
       sc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st)
-        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[st].v, qf[st].v, sc[u], 0, 0, 0);
-    }
-    // ---- values for the second product: issue the loads before the softmax arithmetic
-    Frag vf[DTILES];
-    {
-      const int k0 = min(base + quad * 4, pos);               // run of 4 positions inside one page
-      const int k1 = min(base + 16 + quad * 4, pos);
-      const bf16_t* v0 = v_cache + static_cast<size_t>(table[k0 / block_size]) * page_stride + head_off +
-                         (k0 % block_size) / 4 * 4;
-      const bf16_t* v1 = v_cache + static_cast<size_t>(table[k1 / block_size]) * page_stride + head_off +
-                         (k1 % block_size) / 4 * 4;
-#pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt) {
-        const size_t d_off = static_cast<size_t>(dt * 16 + col) * block_size;
-        vf[dt].u2[0] = *reinterpret_cast<const uint2*>(v0 + d_off);
-        vf[dt].u2[1] = *reinterpret_cast<const uint2*>(v1 + d_off);
-      }
+        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][st].v, qf[st].v, sc[u], 0, 0, 0);
     }
     // ---- softmax of this lane's column over its 8 keys, then across the four quads
     float sv[8];
@@ -185,28 +207,35 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 }
 
 // Merges the splits of one (sequence, query head): m = max m_i, L = sum l_i e^(m_i - m),
-// out = sum o_i e^(m_i - m) / L, splits in ascending order.
+// out = sum o_i e^(m_i - m) / L, splits in ascending order. The weights e^(m_i - m) are computed
+// once by the first threads and shared through LDS.
+#define MERGE_MAX_SPLITS 256
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                               bf16_t* __restrict__ out, const int* __restrict__ query_start,
                                               const int* __restrict__ seq_ids, int H, int nsplit) {
+  __shared__ float weight[MERGE_MAX_SPLITS];
+  __shared__ float weighted_sum[MERGE_MAX_SPLITS];
+  __shared__ float scratch[16];
   const int h = blockIdx.x;
   const int z = blockIdx.y;
   const int s = seq_ids ? seq_ids[z] : z;
   const int t = query_start[s];
   const size_t slot0 = (static_cast<size_t>(z) * H + h) * nsplit;
-  float m = -INFINITY;
-  for (int i = 0; i < nsplit; ++i) m = fmaxf(m, part_ml[(slot0 + i) * 2]);
-  float L = 0.f;
-  for (int i = 0; i < nsplit; ++i) {
-    const float mi = part_ml[(slot0 + i) * 2];
-    if (mi != -INFINITY) L += part_ml[(slot0 + i) * 2 + 1] * expf(mi - m);
+  const int i = threadIdx.x;
+  const float mi = i < nsplit ? part_ml[(slot0 + i) * 2] : -INFINITY;
+  const float li = i < nsplit ? part_ml[(slot0 + i) * 2 + 1] : 0.f;
+  const float m = block_max(mi, scratch);
+  const float wi = (mi == -INFINITY) ? 0.f : expf(mi - m);
+  if (i < nsplit) {
+    weight[i] = wi;
+    weighted_sum[i] = wi * li;
   }
+  __syncthreads();
+  float L = 0.f;
+  for (int k = 0; k < nsplit; ++k) L += weighted_sum[k];   // ascending order, the same in every thread
   for (int d = threadIdx.x; d < DH; d += blockDim.x) {
     float o = 0.f;
-    for (int i = 0; i < nsplit; ++i) {
-      const float mi = part_ml[(slot0 + i) * 2];
-      if (mi != -INFINITY) o += part_o[(slot0 + i) * DH + d] * expf(mi - m);
-    }
+    for (int k = 0; k < nsplit; ++k) o += part_o[(slot0 + k) * DH + d] * weight[k];
     out[(static_cast<size_t>(t) * H + h) * DH + d] = float_to_bf16(o / L);
   }
 }
@@ -219,7 +248,7 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
                                          int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
                                          int window, int nsplit, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
-      block_size <= 0 || block_size % 4 != 0 || max_blocks <= 0 || nsplit <= 0)
+      block_size <= 0 || block_size % 4 != 0 || max_blocks <= 0 || nsplit <= 0 || nsplit > MERGE_MAX_SPLITS)
     return TIE_BAD_ARGUMENT;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr)) return TIE_BAD_ARGUMENT;
   const dim3 grid(nsplit, KVH, num_seqs);
@@ -229,7 +258,8 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
       block_size, max_blocks, scale, window, nsplit);
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
-  attention_decode_merge_kernel<<<dim3(H, num_seqs), DH < 64 ? 64 : DH, 0, stream>>>(
+  const int merge_threads = (nsplit > DH ? nsplit : DH) <= 64 ? 64 : ((nsplit > DH ? nsplit : DH) <= 128 ? 128 : 256);
+  attention_decode_merge_kernel<<<dim3(H, num_seqs), merge_threads, 0, stream>>>(
       part_o, part_ml, static_cast<bf16_t*>(out), query_start, seq_ids, H, nsplit);
   return tie_launch_status();
 }

@@ -14,13 +14,23 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
   const int t = blockIdx.x;
   const TW* row = table + static_cast<size_t>(ids[t]) * D;
   float* o = out + static_cast<size_t>(t) * D;
+  if (D % 8 == 0) {  // rows start 16-byte aligned: move 8 elements a thread
+    for (int d = threadIdx.x * 8; d < D; d += blockDim.x * 8) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = load_as_float(row + d + i);
+      *reinterpret_cast<float4*>(o + d) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(o + d + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+    return;
+  }
   for (int d = threadIdx.x; d < D; d += blockDim.x) o[d] = load_as_float(row + d);
 }
 
 extern "C" int tie_embed(const void* table, int table_dtype, const int* ids, float* out, int T, int D,
                          hipStream_t stream) {
   if (T <= 0 || D <= 0) return TIE_BAD_ARGUMENT;
-  const int threads = D >= 1024 ? 256 : 64;
+  const int threads = D >= 2048 ? 256 : 64;
   if (table_dtype == TIE_F32) {
     embed_kernel<float><<<T, threads, 0, stream>>>(static_cast<const float*>(table), ids, out, D);
   } else if (table_dtype == TIE_BF16) {
@@ -53,9 +63,52 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, const float* __restric
   }
 }
 
+// The same for float32 rows of up to 16 values a thread (n % 4 == 0): the row is read once and
+// stays in registers between the sum of squares and the scaling.
+template <typename TO>
+__global__ void rms_norm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, float eps,
+                                    TO* __restrict__ out, const int* __restrict__ rows, int n) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* xr = x + static_cast<size_t>(rows ? rows[r] : r) * n;
+  TO* o = out + static_cast<size_t>(r) * n;
+  float4 v[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    v[j] = i < n ? *reinterpret_cast<const float4*>(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    if (i >= n) continue;
+    const float4 wv = *reinterpret_cast<const float4*>(w + i);
+    store_from_float(o + i, (v[j].x * inv) * wv.x);
+    store_from_float(o + i + 1, (v[j].y * inv) * wv.y);
+    store_from_float(o + i + 2, (v[j].z * inv) * wv.z);
+    store_from_float(o + i + 3, (v[j].w * inv) * wv.w);
+  }
+}
+
 extern "C" int tie_rms_norm(const void* x, int x_dtype, const float* w, float eps, void* out, int out_dtype,
                             const int* rows, int R, int n, hipStream_t stream) {
   if (R <= 0 || n <= 0) return TIE_BAD_ARGUMENT;
+  if (x_dtype == TIE_F32 && n % 4 == 0 && n <= 16384 && n >= 256) {
+    const int threads = n <= 1024 ? 64 : (n <= 4096 ? 256 : (n <= 8192 ? 512 : 1024));
+    if (out_dtype == TIE_F32)
+      rms_norm_row_kernel<float><<<R, threads, 0, stream>>>(static_cast<const float*>(x), w, eps,
+                                                            static_cast<float*>(out), rows, n);
+    else if (out_dtype == TIE_BF16)
+      rms_norm_row_kernel<bf16_t><<<R, threads, 0, stream>>>(static_cast<const float*>(x), w, eps,
+                                                             static_cast<bf16_t*>(out), rows, n);
+    else
+      return TIE_BAD_ARGUMENT;
+    return tie_launch_status();
+  }
   const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
 #define LAUNCH(TX, TO)                                                                                   \
   rms_norm_kernel<TX, TO><<<R, threads, 0, stream>>>(static_cast<const TX*>(x), w, eps, static_cast<TO*>(out), \
@@ -249,57 +302,87 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
 // ------------------------------------------------------------------ argmax
 // out[r] = index of the first maximum of logits[r, :] (ties go to the lowest id,
 // as std::max_element in src/sampling/sampler.cpp:24); -1 if the row holds a NaN.
-__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
-  __shared__ float best_v[16];
-  __shared__ int best_i[16];
-  __shared__ int saw_nan;
-  const int r = blockIdx.x;
+// Two stages so that a few long rows still fill the GPU: ARGMAX_CHUNKS workgroups scan a slice of
+// a row each, then one wave per row picks among their candidates.
+#define ARGMAX_CHUNKS 64
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__global__ void argmax_partial_kernel(const float* __restrict__ logits, float* __restrict__ part_v,
+                                      int* __restrict__ part_i, int V) {
+  __shared__ float best_v[4];
+  __shared__ int best_i[4];
+  const int r = blockIdx.y, chunk = blockIdx.x;
   const float* row = logits + static_cast<size_t>(r) * V;
-  if (threadIdx.x == 0) saw_nan = 0;
-  __syncthreads();
+  const int per = (V + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+  const int begin = chunk * per, end = min(V, begin + per);
   float bv = -INFINITY;
-  int bi = V;  // sentinel: larger than any index
+  int bi = 0x7fffffff;
   bool nan = false;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
     const float v = row[i];
     nan |= (v != v);
-    if (v > bv || (v == bv && i < bi)) {
+    if (better(v, i, bv, bi)) {
       bv = v;
       bi = i;
     }
   }
-  if (nan) saw_nan = 1;
+  if (nan) {  // a NaN beats everything and is remembered as index -1
+    bv = INFINITY;
+    bi = -1;
+  }
 #pragma unroll
   for (int off = TIE_WAVE / 2; off > 0; off >>= 1) {
     const float ov = __shfl_xor(bv, off, TIE_WAVE);
     const int oi = __shfl_xor(bi, off, TIE_WAVE);
-    if (ov > bv || (ov == bv && oi < bi)) {
+    if (better(ov, oi, bv, bi)) {
       bv = ov;
       bi = oi;
     }
   }
-  const int lane = threadIdx.x & (TIE_WAVE - 1);
-  const int wave = threadIdx.x / TIE_WAVE;
+  const int lane = threadIdx.x & (TIE_WAVE - 1), wave = threadIdx.x / TIE_WAVE;
   if (lane == 0) {
     best_v[wave] = bv;
     best_i[wave] = bi;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int waves = blockDim.x / TIE_WAVE;
-    for (int w = 1; w < waves; ++w) {
-      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+    for (int w = 1; w < static_cast<int>(blockDim.x) / TIE_WAVE; ++w)
+      if (better(best_v[w], best_i[w], bv, bi)) {
         bv = best_v[w];
         bi = best_i[w];
       }
-    }
-    out[r] = saw_nan ? -1 : bi;
+    part_v[r * ARGMAX_CHUNKS + chunk] = bv;
+    part_i[r * ARGMAX_CHUNKS + chunk] = bi;
   }
 }
 
-extern "C" int tie_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
-  if (R <= 0 || V <= 0) return TIE_BAD_ARGUMENT;
-  argmax_kernel<<<R, 1024, 0, stream>>>(logits, out, V);
+__global__ void argmax_final_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i,
+                                    int* __restrict__ out) {
+  const int r = blockIdx.x;
+  float bv = part_v[r * ARGMAX_CHUNKS + threadIdx.x];
+  int bi = part_i[r * ARGMAX_CHUNKS + threadIdx.x];
+#pragma unroll
+  for (int off = TIE_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, TIE_WAVE);
+    const int oi = __shfl_xor(bi, off, TIE_WAVE);
+    if (better(ov, oi, bv, bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if (threadIdx.x == 0) out[r] = bi;
+}
+
+// part_v / part_i: workspace of R * 64 floats / ints.
+extern "C" int tie_argmax(const float* logits, int* out, float* part_v, int* part_i, int R, int V,
+                          hipStream_t stream) {
+  if (R <= 0 || R > 65535 || V <= 0 || part_v == nullptr || part_i == nullptr) return TIE_BAD_ARGUMENT;
+  static_assert(ARGMAX_CHUNKS == TIE_WAVE, "the final stage is one wave per row");
+  argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, R), 256, 0, stream>>>(logits, part_v, part_i, V);
+  int status = tie_launch_status();
+  if (status != TIE_OK) return status;
+  argmax_final_kernel<<<R, TIE_WAVE, 0, stream>>>(part_v, part_i, out);
   return tie_launch_status();
 }
 

@@ -2,11 +2,11 @@
 // (1..64), bfloat16 operands, float32 accumulation on v_mfma_f32_16x16x32_bf16.
 //
 // The product is bound by reading w once from HBM, so the kernel is built around that stream:
-// a workgroup of four waves owns 16 rows of w; the waves split K into four contiguous ranges;
+// a workgroup of four (or eight) waves owns 16 rows of w; the waves split K into contiguous ranges;
 // every lane reads 16 bytes of "its" row per MFMA (row = lane % 16, k-chunk = lane / 16), which
 // is exactly the B-operand layout, so weights go from memory to the matrix core with no staging.
 // The few rows of x are the A operand, read through the caches (they are shared by every
-// workgroup); rows beyond M are zeros. The four partial sums meet in LDS and are added in a fixed
+// workgroup); rows beyond M are zeros. The waves' partial sums meet in LDS and are added in a fixed
 // order, so the result does not depend on timing. M > 16 runs 2 or 4 row tiles of x against each
 // weight fragment.
 //
@@ -16,7 +16,6 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-#define SK_WAVES 4
 #define SK_UNROLL 4
 
 __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p) {
@@ -29,7 +28,7 @@ __device__ __forceinline__ bf16x8_t zero_frag() {
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
-template <int MT, typename TO>
+template <int MT, typename TO, int SK_WAVES>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
@@ -99,19 +98,20 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     for (int v = 0; v < 4; ++v) red[wave][mt][(g * 4 + v) * 16 + r] = acc[mt][v];
   __syncthreads();
 
-  const int e = threadIdx.x;  // 256 threads <-> 16 x 16 outputs of a tile
-  const int n = n0 + (e & 15);
-  if (n >= N) return;
+  for (int e = threadIdx.x; e < 256; e += SK_WAVES * TIE_WAVE) {  // 16 x 16 outputs of a tile
+    const int n = n0 + (e & 15);
+    if (n >= N) continue;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + (e >> 4);
-    if (m >= M) continue;
-    float sum = red[0][mt][e];
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + (e >> 4);
+      if (m >= M) continue;
+      float sum = red[0][mt][e];
 #pragma unroll
-    for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][e];
-    TO* o = out + static_cast<size_t>(m) * N + n;
-    if (accumulate) sum = load_as_float(o) + sum;
-    store_from_float(o, sum);
+      for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][e];
+      TO* o = out + static_cast<size_t>(m) * N + n;
+      if (accumulate) sum = load_as_float(o) + sum;
+      store_from_float(o, sum);
+    }
   }
 }
 
@@ -120,13 +120,17 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0) return TIE_BAD_ARGUMENT;
   const dim3 grid((N + 15) / 16);
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-#define LAUNCH(MT, TO)                                                                                          \
-  skinny_gemm_kernel<MT, TO><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                                          \
+  // Few workgroups (small N) or long rows: eight waves a workgroup keep more loads in flight.
+  const bool wide = grid.x <= 512 || K >= 8192;   // by the shape of w alone: every M sums in the same order
+#define LAUNCH(MT, TO, WAVES)                                                                                   \
+  skinny_gemm_kernel<MT, TO, WAVES><<<grid, WAVES * TIE_WAVE, 0, stream>>>(                                      \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate)
   if (out_dtype == TIE_F32) {
-    if (mt == 1) LAUNCH(1, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(4, float);
+    if (wide) { if (mt == 1) LAUNCH(1, float, 8); else if (mt == 2) LAUNCH(2, float, 8); else LAUNCH(4, float, 8); }
+    else { if (mt == 1) LAUNCH(1, float, 4); else if (mt == 2) LAUNCH(2, float, 4); else LAUNCH(4, float, 4); }
   } else if (out_dtype == TIE_BF16) {
-    if (mt == 1) LAUNCH(1, bf16_t); else if (mt == 2) LAUNCH(2, bf16_t); else LAUNCH(4, bf16_t);
+    if (wide) { if (mt == 1) LAUNCH(1, bf16_t, 8); else if (mt == 2) LAUNCH(2, bf16_t, 8); else LAUNCH(4, bf16_t, 8); }
+    else { if (mt == 1) LAUNCH(1, bf16_t, 4); else if (mt == 2) LAUNCH(2, bf16_t, 4); else LAUNCH(4, bf16_t, 4); }
   } else {
     return TIE_BAD_ARGUMENT;
   }

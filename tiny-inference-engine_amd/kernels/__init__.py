@@ -46,7 +46,7 @@ _SIGNATURES = {
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-        "tie_argmax": [_c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
@@ -393,12 +393,22 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         int(window or 0), _stream()), "paged_attention_generic")
 
 
+_argmax_workspace = {}
+
+
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
     """out[r] = lowest index of the maximum of logits[r]; -1 marks a row with a NaN."""
     _f32(logits, "logits")
     R, V = logits.shape
     _i32(out, "argmax output", R)
-    _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), R, V, _stream()), "argmax")
+    key = str(logits.device)
+    ws = _argmax_workspace.get(key)
+    if ws is None or ws[0].numel() < R * 64:
+        rows = max(R, 64)
+        ws = _argmax_workspace[key] = (torch.empty(rows * 64, dtype=torch.float32, device=logits.device),
+                                       torch.empty(rows * 64, dtype=torch.int32, device=logits.device))
+    _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), ws[0].data_ptr(), ws[1].data_ptr(), R, V,
+                                          _stream()), "argmax")
 
 
 def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
@@ -417,7 +427,7 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
 
 def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
     """How many ways the keys of each sequence are split so that a decode step fills the GPU."""
-    target_waves = 1024
+    target_waves = 2048
     by_occupancy = -(-target_waves // max(1, num_seqs * num_kv_heads))
     by_length = max(1, max_context // 128)          # at least four 32-key tiles a split
     return max(1, min(by_occupancy, by_length))
