@@ -1,0 +1,322 @@
+"""The parts of a model, each alone and in other arrangements than Qwen3's, on the GPU.
+
+* each built-in part against its plain function, built from a PartSpec as the model builder does;
+* a run order that names a layer twice and lets the second call read the first call's cache;
+* an attention window, which Qwen3 does not have, through the same part and cache manager;
+* a toy mixer with a per-request state of its own, a toy position encoding and a toy architecture,
+  all defined HERE and registered from outside: built, loaded with random weights, and stepped
+  through the framework's step function without a change to the framework's files.
+"""
+
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import trace_helpers as th
+from conftest import TINY_B, load_plain_weights
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+
+
+def close(got, want, rel, what=""):
+    got, want = got.detach().cpu().to(F64), want.detach().cpu().to(F64)
+    err = float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+    assert err <= rel, f"{what}: relative error {err:.3e} > {rel:.0e}"
+
+
+class FakeBatch:
+    num_tokens = 0
+
+
+def make_ctx(T, mode="float32"):
+    from tie_amd.parts.base import StepContext, Workspace
+
+    batch = FakeBatch()
+    batch.num_tokens = T
+    return StepContext(batch, mode, torch.device("cuda:0"), Workspace("cuda:0"), None, None)
+
+
+def fetcher(tensors, mode="float32"):
+    from tie_amd.weights.binder import place_tensor
+    from tie_amd.weights.safetensors_io import StoredTensor
+
+    return lambda name, role: place_tensor(StoredTensor.from_tensor(name, tensors[name]), role, mode, "cuda:0")
+
+
+def test_norm_embedding_feed_forward_and_head_parts_alone():
+    from tie_amd.parts import PartSpec, build_part
+
+    g = torch.Generator().manual_seed(1)
+    T, D, I, V = 7, 96, 200, 50
+    w = {"n": 1 + 0.1 * torch.randn(D, generator=g), "e": torch.randn(V, D, generator=g) * 0.5,
+         "g": torch.randn(I, D, generator=g) * 0.1, "u": torch.randn(I, D, generator=g) * 0.1,
+         "d": torch.randn(D, I, generator=g) * 0.1, "h": torch.randn(V, D, generator=g) * 0.1}
+    fetch = fetcher(w)
+    ctx = make_ctx(T)
+    x = torch.randn(T, D, generator=g)
+
+    norm = build_part("norm", PartSpec("rms_norm", {"dim": D, "eps": 1e-5, "weight": "n"}))
+    assert [(s.name, s.shape, s.role) for s in norm.tensors()] == [("n", (D,), "vector")]
+    norm.load_all(fetch, "float32", "cuda:0")
+    close(norm.forward(ctx, x.cuda()), plain.rms_norm(x, w["n"], 1e-5), 1e-5, "norm part")
+
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab": V, "hidden": D, "weight": "e"}))
+    emb.load_all(fetch, "float32", "cuda:0")
+    ids = [3, 49, 0, 3, 17, 8, 21]
+    got = emb.forward(ctx, torch.tensor(ids, dtype=torch.int32, device="cuda"))
+    assert torch.equal(got.cpu(), w["e"][ids])
+
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden": D, "intermediate": I,
+                                                         "names": {"gate": "g", "up": "u", "down": "d"}}))
+    assert sorted(s.name for s in ffn.tensors()) == ["d", "g", "u"]
+    ffn.load_all(fetch, "float32", "cuda:0")
+    residual = x.cuda().clone()
+    ffn.forward(ctx, x.cuda(), residual)                      # the part ADDS its result to the residual
+    close(residual, x.to(F64) + plain.swiglu(x, w["g"], w["u"], w["d"]), 1e-5, "feed-forward part")
+
+    for tied in (None, "e"):
+        head = build_part("head", PartSpec("lm_head", {"vocab": V, "hidden": D, "weight": "h", "tied_to": tied,
+                                                       "norm": PartSpec("rms_norm", {"dim": D, "eps": 1e-5, "weight": "n"})}))
+        head.load_all(fetch, "float32", "cuda:0")
+        rows = torch.tensor([6, 0, 2], dtype=torch.int32, device="cuda")
+        want = plain.linear(plain.rms_norm(x[[6, 0, 2]], w["n"], 1e-5), w[tied or "h"])
+        close(head.forward(ctx, x.cuda(), rows), want, 1e-5, f"head part tied={tied}")
+        names = {s.name: s.optional for s in head.all_tensors()}
+        assert names == ({"h": False, "n": False} if tied is None else {"e": False, "h": True, "n": False})
+
+
+def test_position_part_holds_the_reference_frequencies():
+    from tie_amd.parts import PartSpec, build_part
+
+    for theta, dim in ((1e4, 16), (1e6, 128), (5e5, 80)):
+        part = build_part("position", PartSpec("rope_neox", {"head_dim": dim, "theta": theta}))
+        part.load_all(None, "float32", "cuda:0")
+        inv_freq, rotary_dim, pairing = part.rotary_table()
+        assert rotary_dim == dim and pairing == "rotate_half"
+        assert np.array_equal(inv_freq.cpu().numpy(), plain.rope_inv_freq(theta, dim))   # bit for bit
+
+
+# ------------------------------------------------------------------ other arrangements of the attention part
+def attention_model(order, window=None, layers=2):
+    """A model of ``layers`` attention + SwiGLU layers in Qwen3's tensor names with a free run order and window."""
+    from tie_amd.config.qwen3 import Qwen3Config
+    from tie_amd.models import LayerCall, Model
+    from tie_amd.models.qwen3 import build_qwen3_spec
+
+    cfg = dict(TINY_B, num_hidden_layers=layers)
+    spec = build_qwen3_spec(Qwen3Config.from_json(cfg))
+    new_layers = []
+    for layer in spec.layers:
+        mixer = dataclasses.replace(layer.mixer, params={**layer.mixer.params, "window": window})
+        new_layers.append(dataclasses.replace(layer, mixer=mixer))
+    spec = dataclasses.replace(spec, layers=tuple(new_layers), order=tuple(LayerCall(*o) for o in order))
+    return Model(spec), cfg
+
+
+def plain_with_order(weights, cfg, tokens, order, window=None):
+    """Whole-sequence forward with a run order; a call that reads another call's cache uses its keys and values."""
+    cfg = plain.normalized_config(cfg)
+    T = len(tokens)
+    H, KVH, Dh, eps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    pos = list(range(T))
+    x = plain.embed(weights["model.embed_tokens.weight"], tokens)
+    kept = {}
+    for index, (layer, source) in enumerate(order):
+        p = f"model.layers.{layer}."
+        h = plain.rms_norm(x, weights[p + "input_layernorm.weight"], eps)
+        q = plain.rope_neox(plain.rms_norm(plain.linear(h, weights[p + "self_attn.q_proj.weight"]).view(T, H, Dh),
+                                           weights[p + "self_attn.q_norm.weight"], eps), pos, cfg["rope_theta"])
+        if source is None:
+            k = plain.rope_neox(plain.rms_norm(plain.linear(h, weights[p + "self_attn.k_proj.weight"]).view(T, KVH, Dh),
+                                               weights[p + "self_attn.k_norm.weight"], eps), pos, cfg["rope_theta"])
+            v = plain.linear(h, weights[p + "self_attn.v_proj.weight"]).view(T, KVH, Dh)
+            kept[index] = (k, v)
+        else:
+            k, v = kept[source]
+        a = plain.causal_attention(q, k, v, float(np.float32(1.0) / np.sqrt(np.float32(Dh))), window).reshape(T, H * Dh)
+        x = x + plain.linear(a, weights[p + "self_attn.o_proj.weight"])
+        h = plain.rms_norm(x, weights[p + "post_attention_layernorm.weight"], eps)
+        x = x + plain.swiglu(h, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
+                             weights[p + "mlp.down_proj.weight"])
+    x = plain.rms_norm(x, weights["model.norm.weight"], eps)
+    return plain.linear(x, weights["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype,tolerance", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("order,window", [
+    (((0, None), (1, None), (0, None)), None),            # layer 0 runs twice, each call with a cache of its own
+    (((0, None), (1, None), (0, 0), (1, 1)), None),       # the later calls read the earlier calls' caches
+    (((0, None), (1, None)), 7),                          # a window of 7 keys: pages go back while requests run
+    (((0, None), (1, 0)), 20),
+])
+def test_run_orders_shared_caches_and_windows(tmp_path, order, window, dtype, tolerance):
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.weights.loader import load_model_folder
+    from tie_amd.weights.random_init import write_random_model
+
+    model, cfg = attention_model(order, window)
+    planes = sum(1 for _, src in order if src is None)
+    assert model.cache_plan.groups[0].num_planes == planes and model.cache_plan.groups[0].need.window == window
+    folder = write_random_model(tmp_path / "m", cfg, seed=3, dtype="float32" if dtype == "float32" else "bfloat16")
+    model.load(load_model_folder(folder).tensors, dtype, "cuda:0")
+    weights = load_plain_weights(folder)
+    requests = th.make_requests(cfg["vocab_size"], [45, 70, 33], seed=8)
+    want = {rid: plain_with_order(weights, cfg, toks, order, window).float() for rid, toks in requests.items()}
+    steps, peak = th.mixed(requests, max_live=3, seed=2)
+    replayer = TraceReplayer(model, peak if window is None else 96, block_size=4)   # a window needs few pages
+    got = th.collect(replayer, steps)
+    for rid, ref in want.items():
+        mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
+        close(mine, ref, tolerance, f"order {order} window {window} request {rid}")
+    assert replayer.cache.num_free() == replayer.cache.num_blocks
+
+
+# ------------------------------------------------------------------ toy parts, defined and registered here
+def register_toy_parts():
+    from tie_amd.cache.spec import FixedState
+    from tie_amd.parts import Mixer, Position, TensorSpec, register_part
+
+    @register_part("mixer", "toy_decay")
+    class ToyDecayMixer(Mixer):
+        """s_t = decay * s_{t-1} + W_in h_t ; out_t = W_out s_t, with s kept per request in a state slot."""
+
+        def __init__(self, params):
+            super().__init__(params)
+            self.hidden, self.width, self.decay = params["hidden"], params["width"], params["decay"]
+            self.names = params["names"]
+
+        def cache_need(self):
+            return FixedState((self.width,), "float32")
+
+        def tensors(self):
+            return [TensorSpec(self.names["in"], (self.width, self.hidden), "matrix", ("normal", 0.2)),
+                    TensorSpec(self.names["out"], (self.hidden, self.width), "matrix", ("normal", 0.2))]
+
+        def load(self, fetch, mode, device):
+            self.w_in, self.w_out = fetch(self.names["in"], "matrix"), fetch(self.names["out"], "matrix")
+
+        def forward(self, ctx, h, cache, residual):
+            u = h.float() @ self.w_in.float().T                               # [T, width]
+            row = 0
+            for n, slot in zip(ctx.batch.host_new_tokens, ctx.batch.host_state_slots):
+                state = cache.state[slot]                                     # carried across portions and steps
+                for t in range(row, row + n):                                 # tokens of a sequence in order
+                    state.mul_(self.decay).add_(u[t])
+                    residual[t] += state @ self.w_out.float().T
+                row += n
+
+    @register_part("position", "toy_shift")
+    class ToyShiftPosition(Position):
+        """Not a rotation: adds position * slope to the first dimension of every query and key head."""
+
+        def __init__(self, params):
+            super().__init__(params)
+            self.slope = params["slope"]
+
+        def apply(self, ctx, q, k, positions):
+            shift = positions.float() * self.slope
+            q[:, :, 0] += shift[:, None]
+            k[:, :, 0] += shift[:, None]
+
+
+def toy_spec(cfg):
+    from tie_amd.models import LayerCall, LayerSpec, ModelSpec
+    from tie_amd.parts import PartSpec
+
+    D, eps = cfg["hidden_size"], cfg["eps"]
+    norm = lambda name: PartSpec("rms_norm", {"dim": D, "eps": eps, "weight": name})
+    layers = []
+    for l, kind in enumerate(cfg["mixers"]):
+        p = f"layers.{l}."
+        if kind == "decay":
+            mixer = PartSpec("toy_decay", {"hidden": D, "width": cfg["state_width"], "decay": cfg["decay"],
+                                           "names": {"in": p + "mix.in", "out": p + "mix.out"}})
+        else:
+            mixer = PartSpec("paged_attention", {
+                "hidden": D, "num_heads": cfg["heads"], "num_kv_heads": cfg["kv_heads"], "head_dim": cfg["head_dim"],
+                "scale": cfg["head_dim"] ** -0.5, "window": None, "qk_norm": None,
+                "position": PartSpec("toy_shift", {"slope": cfg["slope"]}),
+                "names": {"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}})
+        ffn = PartSpec("swiglu", {"hidden": D, "intermediate": cfg["intermediate"],
+                                  "names": {"gate": p + "gate", "up": p + "up", "down": p + "down"}})
+        layers.append(LayerSpec(PartSpec("pre_norm"), mixer, ffn,
+                                {"pre_mixer": norm(p + "n1"), "pre_feed_forward": norm(p + "n2")}))
+    return ModelSpec("ToyStateLM", cfg["vocab_size"], D, cfg["max_positions"],
+                     PartSpec("token_embedding", {"vocab": cfg["vocab_size"], "hidden": D, "weight": "embed"}),
+                     tuple(layers), tuple(LayerCall(l) for l in range(len(layers))),
+                     PartSpec("lm_head", {"vocab": cfg["vocab_size"], "hidden": D, "norm": norm("final_norm"),
+                                          "weight": "head", "tied_to": "embed"}))
+
+
+def toy_plain(weights, cfg, tokens):
+    T, D = len(tokens), cfg["hidden_size"]
+    x = plain.embed(weights["embed"], tokens)
+    for l, kind in enumerate(cfg["mixers"]):
+        p = f"layers.{l}."
+        h = plain.rms_norm(x, weights[p + "n1"], cfg["eps"])
+        if kind == "decay":
+            u = plain.linear(h, weights[p + "mix.in"])
+            s = torch.zeros(cfg["state_width"], dtype=F64)
+            out = []
+            for t in range(T):
+                s = cfg["decay"] * s + u[t]
+                out.append(plain.linear(s[None], weights[p + "mix.out"])[0])
+            x = x + torch.stack(out)
+        else:
+            H, KVH, Dh = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+            q = plain.linear(h, weights[p + "q"]).view(T, H, Dh).clone()
+            k = plain.linear(h, weights[p + "k"]).view(T, KVH, Dh).clone()
+            v = plain.linear(h, weights[p + "v"]).view(T, KVH, Dh)
+            shift = torch.arange(T, dtype=F64) * cfg["slope"]
+            q[:, :, 0] += shift[:, None]
+            k[:, :, 0] += shift[:, None]
+            a = plain.causal_attention(q, k, v, Dh ** -0.5).reshape(T, H * Dh)
+            x = x + plain.linear(a, weights[p + "o"])
+        h = plain.rms_norm(x, weights[p + "n2"], cfg["eps"])
+        x = x + plain.swiglu(h, weights[p + "gate"], weights[p + "up"], weights[p + "down"])
+    return plain.linear(plain.rms_norm(x, weights["final_norm"], cfg["eps"]), weights["embed"])
+
+
+def test_a_toy_architecture_registered_from_outside_runs_through_the_step_function(tmp_path):
+    from tie_amd.cache.spec import FixedState, PagedKV
+    from tie_amd.config.registry import register_architecture, unregister_architecture
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.parts import unregister_part
+    from tie_amd.weights.random_init import write_random_model
+
+    register_toy_parts()
+    register_architecture("ToyStateLM", lambda values: dict(values), toy_spec, model_types=("toy_state",))
+    try:
+        cfg = {"architectures": ["ToyStateLM"], "vocab_size": 90, "hidden_size": 48, "intermediate": 72,
+               "heads": 3, "kv_heads": 1, "head_dim": 16, "state_width": 20, "decay": 0.8, "slope": 0.01,
+               "eps": 1e-5, "max_positions": 256, "mixers": ["decay", "attention", "decay"]}
+        folder = write_random_model(tmp_path / "toy", cfg, seed=4, dtype="float32")   # the parts' TensorSpecs drive it
+        replayer = TraceReplayer.from_folder(folder, "float32", 192, block_size=4)    # config.json names the class
+        plan = replayer.model.cache_plan
+        assert [type(g.need) for g in plan.groups] == [FixedState, PagedKV] and plan.groups[0].num_planes == 2
+        weights = load_plain_weights(folder)
+        requests = th.make_requests(cfg["vocab_size"], [40, 64, 23, 51], seed=6)
+        want = {rid: toy_plain(weights, cfg, toks).float() for rid, toks in requests.items()}
+        steps, peak = th.mixed(requests, max_live=3, seed=5)          # portions beside single tokens; slots reused
+        got = th.collect(replayer, steps)
+        for rid, ref in want.items():
+            mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
+            close(mine, ref, 1e-4, f"toy model request {rid}")
+        assert replayer.cache.num_free_state_slots == replayer.cache.max_state_slots
+        # generation through the engine works for it too: the scheduler hands out and takes back state slots
+        import tie_amd
+        engine = tie_amd.create_engine(replayer.model, kv_blocks=64, block_size=4, max_seqs=2, max_tokens_per_step=16)
+        prompt = requests["r2"]
+        out = engine.generate(prompt, tie_amd.SamplingParams(max_tokens=5))
+        tokens = list(prompt)
+        for t in out:
+            assert t == int(torch.argmax(toy_plain(weights, cfg, tokens)[-1]))
+            tokens.append(t)
+    finally:
+        unregister_architecture("ToyStateLM")
+        unregister_part("mixer", "toy_decay")
+        unregister_part("position", "toy_shift")

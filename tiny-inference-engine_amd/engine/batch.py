@@ -57,6 +57,7 @@ class StepBatch:
         # host copies for planning
         self.host_new_tokens: List[int] = []
         self.host_context_lens: List[int] = []
+        self.host_state_slots: List[int] = []
         self.max_context = 0
         self.plan_context = 0      # the context length kernels size their grids for (>= max_context)
         self.max_new_tokens = 0
@@ -182,6 +183,7 @@ class BatchBuilder:
             query_start[s + 1] = row
             batch.host_new_tokens.append(n)
             batch.host_context_lens.append(e.start + n)
+            batch.host_state_slots.append(e.cache.state_slot)
 
         dev_t[:offset].copy_(host_t[:offset], non_blocking=True)
         if self.device.type == "cuda":

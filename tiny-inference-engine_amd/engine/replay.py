@@ -43,7 +43,8 @@ class TraceReplayer:
         num_blocks = math.ceil(max_tokens / block_size)
         self.cache = CacheManager(model.cache_plan, block_size=block_size, num_blocks=num_blocks,
                                   dtype=cache_dtype, device=model.device, max_state_slots=8)
-        self.runner = ModelRunner(model, self.cache, max_seq_len=num_blocks * block_size, use_graphs=use_graphs)
+        # A request may outgrow the pool where windows give pages back, so only the model's context limits it.
+        self.runner = ModelRunner(model, self.cache, use_graphs=use_graphs)
         self.requests: Dict[str, RequestCache] = {}
         self.lengths: Dict[str, int] = {}
 
