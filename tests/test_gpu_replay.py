@@ -144,3 +144,35 @@ def test_recorded_decode_steps_replay_to_the_eager_result(folders):
         if a is not None:
             assert torch.equal(a, b), f"step {step['step']} differs between eager launches and the replayed graph"
     assert graphs.runner.graph_replays >= 10 and eager.runner.graph_replays == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """A short prompt, then every further token one by one, up to the model's context."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders[dtype]["B"]
+    requests = th.make_requests(cfg["vocab_size"], [250], seed=31)
+    want = reference_logits(folder, cfg, requests)
+    got = th.collect(TraceReplayer.from_folder(folder, dtype, 256, block_size=16),
+                     th.prefill_then_decode(requests, tail=243))
+    check(got, want, dtype, f"B/{dtype}/long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_first_tokens_of_a_sequence(folders, name, dtype):
+    """Position 0 alone, the first few positions one by one, and prompts of one, two and three tokens."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders[dtype][name]
+    requests = th.make_requests(cfg["vocab_size"], [1, 2, 3, 6], seed=33)
+    want = reference_logits(folder, cfg, requests)
+    rep = lambda: TraceReplayer.from_folder(folder, dtype, 256, block_size=BLOCK_SIZE[name])
+    check(th.collect(rep(), th.whole(requests)), want, dtype, f"{name}/{dtype}/first tokens whole")
+    check(th.collect(rep(), th.prefill_then_decode(requests, tail=32)), want, dtype, f"{name}/{dtype}/first tokens one by one")
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:1], "want": [0]} for rid, toks in requests.items()], "end": ["r0"]}]
+    for i in range(1, 6):
+        entries = [{"id": rid, "tokens": [toks[i]], "want": [0]} for rid, toks in requests.items() if len(toks) > i]
+        steps.append({"step": i, "entries": entries, "end": [rid for rid, toks in requests.items() if len(toks) == i + 1]})
+    check(th.collect(rep(), steps), want, dtype, f"{name}/{dtype}/first tokens together")
