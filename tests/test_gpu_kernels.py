@@ -397,3 +397,23 @@ def test_kernels_refuse_what_they_cannot_take():
                                       torch.zeros(1, 1, 1024, 4).cuda(), 1, 1, 1024, 4)
     with pytest.raises(InvalidArgument):
         kernels.embed(torch.zeros(4, 8, dtype=torch.float16).cuda(), i32([0]), torch.zeros(1, 8).cuda())
+
+
+@pytest.mark.parametrize("M", [1, 8, 40, 65, 300])
+@pytest.mark.parametrize("I,K", [(8, 64), (200, 96), (1000, 512)])
+def test_gated_product_is_silu_gate_times_up(M, I, K):
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=41, dtype=torch.bfloat16).cuda()
+    gate = rnd(I, K, seed=42, scale=0.2, dtype=torch.bfloat16).cuda()
+    up = rnd(I, K, seed=43, scale=0.2, dtype=torch.bfloat16).cuda()
+    w = kernels.interleave_gate_up(gate, up)
+    assert torch.equal(w[:8], gate[:8]) and torch.equal(w[8:16], up[:8])
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kernels.linear_swiglu(x, w, out)
+    g, u = plain.linear(x.cpu(), gate.cpu()), plain.linear(x.cpu(), up.cpu())
+    close(out, g / (1 + torch.exp(-g)) * u, 6e-3, f"gated product M={M} I={I}")
+    if M <= 64:
+        big = torch.empty_like(out)
+        kernels.gemm_bf16(x, w, big, gated=True)                    # both kernels hold the same epilogue
+        close(big, out.float(), 8e-3, "gated product, tiled kernel")

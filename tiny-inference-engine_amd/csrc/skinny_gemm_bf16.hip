@@ -32,7 +32,7 @@ template <int MT, typename TO, int SK_WAVES>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
-                                                                         int accumulate) {
+                                                                         int accumulate, int gated) {
   __shared__ float red[SK_WAVES][MT][256];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -99,8 +99,10 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   __syncthreads();
 
   for (int e = threadIdx.x; e < 256; e += SK_WAVES * TIE_WAVE) {  // 16 x 16 outputs of a tile
-    const int n = n0 + (e & 15);
+    const int c = e & 15;
+    const int n = n0 + c;
     if (n >= N) continue;
+    if (gated && c >= 8) continue;       // gated: columns 0..7 are gates, 8..15 the ups of the same outputs
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mt * 16 + (e >> 4);
@@ -108,6 +110,13 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
       float sum = red[0][mt][e];
 #pragma unroll
       for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][e];
+      if (gated) {
+        float up = red[0][mt][e + 8];
+#pragma unroll
+        for (int wv = 1; wv < SK_WAVES; ++wv) up += red[wv][mt][e + 8];
+        store_from_float(out + static_cast<size_t>(m) * (N / 2) + blockIdx.x * 8 + c, sum / (1.0f + __expf(-sum)) * up);
+        continue;
+      }
       TO* o = out + static_cast<size_t>(m) * N + n;
       if (accumulate) sum = load_as_float(o) + sum;
       store_from_float(o, sum);
@@ -115,16 +124,19 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   }
 }
 
-extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int M,
-                                    int N, int K, hipStream_t stream) {
+// gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
+// and receives silu(gate) * up.
+extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
+                                    int M, int N, int K, hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0) return TIE_BAD_ARGUMENT;
+  if (gated && (accumulate || N % 16 != 0)) return TIE_BAD_ARGUMENT;
   const dim3 grid((N + 15) / 16);
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   // Few workgroups (small N) or long rows: eight waves a workgroup keep more loads in flight.
   const bool wide = grid.x <= 512 || K >= 8192;   // by the shape of w alone: every M sums in the same order
 #define LAUNCH(MT, TO, WAVES)                                                                                   \
   skinny_gemm_kernel<MT, TO, WAVES><<<grid, WAVES * TIE_WAVE, 0, stream>>>(                                      \
-      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate)
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, gated)
   if (out_dtype == TIE_F32) {
     if (wide) { if (mt == 1) LAUNCH(1, float, 8); else if (mt == 2) LAUNCH(2, float, 8); else LAUNCH(4, float, 8); }
     else { if (mt == 1) LAUNCH(1, float, 4); else if (mt == 2) LAUNCH(2, float, 4); else LAUNCH(4, float, 4); }

@@ -59,10 +59,10 @@ _SIGNATURES = {
                                         _c_int, _c_void],
     },
     "skinny_gemm_bf16": {
-        "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
     "gemm_bf16": {
-        "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
     "attention_prefill_bf16": {
         "tie_attention_prefill_rows_per_item": [_c_int],
@@ -251,44 +251,68 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate
         _code(out, "matmul output"), int(accumulate), T, N, K, _stream()), "gemm_generic")
 
 
-def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores."""
+def _bf16_product_operands(x, w, out, gated, what):
     _gpu(x, "matmul input")
     _gpu(w, "matmul weight")
     _gpu(out, "matmul output")
     M, K = x.shape
     N, K2 = w.shape
-    if K != K2 or tuple(out.shape) != (M, N):
+    width = N // 2 if gated else N
+    if K != K2 or tuple(out.shape) != (M, width):
         raise InvalidArgument(f"matmul: input {list(x.shape)}, weight {list(w.shape)}, output {list(out.shape)}")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise InvalidArgument("skinny_gemm_bf16 takes bfloat16 operands")
-    if M > 64 or K % 8:
-        raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows and K % 8 == 0, got M={M}, K={K}")
+        raise InvalidArgument(f"{what} takes bfloat16 operands")
+    if K % 8:
+        raise InvalidArgument(f"{what} takes K % 8 == 0, got K={K}")
+    if gated and (N % 16 or out.dtype != torch.bfloat16):
+        raise InvalidArgument(f"{what}: a gated product needs N % 16 == 0 and a bfloat16 output")
+    return M, N, K
+
+
+def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+                     gated: bool = False) -> None:
+    """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores.
+
+    ``gated``: w is a gate/up pair interleaved by ``interleave_gate_up`` and out receives silu(gate) * up.
+    """
+    M, N, K = _bf16_product_operands(x, w, out, gated, "skinny_gemm_bf16")
+    if M > 64:
+        raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows, got {M}")
+    if gated and accumulate:
+        raise InvalidArgument("a gated product does not accumulate")
     _check(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16(
-        x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), M, N, K,
+        x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
         _stream()), "skinny_gemm_bf16")
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0) -> None:
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0,
+              gated: bool = False) -> None:
     """out (+)= x @ w.T for bfloat16 operands on the matrix cores, any number of rows; K % 8 == 0.
 
-    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x128; 0 lets the kernel choose).
+    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256; 0 lets the kernel choose);
+    ``gated`` as in ``skinny_gemm_bf16``.
     """
-    _gpu(x, "matmul input")
-    _gpu(w, "matmul weight")
-    _gpu(out, "matmul output")
-    M, K = x.shape
-    N, K2 = w.shape
-    if K != K2 or tuple(out.shape) != (M, N):
-        raise InvalidArgument(f"matmul: input {list(x.shape)}, weight {list(w.shape)}, output {list(out.shape)}")
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise InvalidArgument("gemm_bf16 takes bfloat16 operands")
-    if K % 8:
-        raise InvalidArgument(f"gemm_bf16 takes K % 8 == 0, got K={K}")
-    if accumulate and out.dtype != torch.float32:
-        raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only")
+    M, N, K = _bf16_product_operands(x, w, out, gated, "gemm_bf16")
+    if accumulate and (gated or out.dtype != torch.float32):
+        raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only, and not in a gated product")
     _check(_lib("gemm_bf16").tie_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
-                                           int(accumulate), M, N, K, tile, _stream()), "gemm_bf16")
+                                           int(accumulate), int(gated), M, N, K, tile, _stream()), "gemm_bf16")
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The weight layout of a gated product: blocks of 16 rows = 8 gate rows then the 8 up rows of the same outputs."""
+    I, K = gate.shape
+    if up.shape != gate.shape or I % 8:
+        raise InvalidArgument(f"gate {list(gate.shape)} and up {list(up.shape)} must match, with a multiple of 8 rows")
+    return torch.stack([gate.reshape(I // 8, 8, K), up.reshape(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tensor) -> None:
+    """out = silu(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only."""
+    if x.shape[0] <= 64:
+        skinny_gemm_bf16(x, w_interleaved, out, gated=True)
+    else:
+        gemm_bf16(x, w_interleaved, out, gated=True)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
