@@ -170,6 +170,8 @@ def main():
     parser.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the 36 of the shape (0 = all)")
     parser.add_argument("--skip-points", action="store_true", help="skip batch 1, batch 64 and the prefill")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="run only the 2048-token prefill (for profiling); prints its figures alone")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures a single-GPU engine: --gpus {args.gpus} is not supported, run it with --gpus 1")
@@ -192,6 +194,14 @@ def main():
     started = time.perf_counter()
     model = build_model(cfg)
     log(f"model ready in {time.perf_counter() - started:.1f} s")
+
+    if args.prefill_only:
+        t = measure_prefill(model, cfg, PREFILL_TOKENS)
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS,
+                                      "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS["bf16"], 4)},
+                          "layers_run": cfg["num_hidden_layers"]}), flush=True)
+        return 0
 
     chunk = 8192
     seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk)

@@ -132,6 +132,15 @@ def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
     assert torch.equal(q2, qkv[:, :H * Dh])
     kernels.qk_norm_rope_kv_write(qkv, q2, None, None, 0.0, inv_freq, i32([0] * T), i32(slots), kc, vc, H, KVH, Dh, bs)
     assert torch.equal(q2, qkv[:, :H * Dh])
+    # the projection as three planes of partial sums: the same as their sum handed over in one piece
+    planes = rnd(3, T, (H + 2 * KVH) * Dh, seed=11).cuda()
+    summed = (planes[0] + planes[1]) + planes[2]
+    kc1, vc1, kc3, vc3 = (torch.zeros_like(c) for c in (kc, vc, kc, vc))
+    q1, q3 = torch.empty_like(q), torch.empty_like(q)
+    kernels.qk_norm_rope_kv_write(summed, q1, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc1, vc1, H, KVH, Dh, bs)
+    kernels.qk_norm_rope_kv_write(planes[0], q3, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc3, vc3, H, KVH,
+                                  Dh, bs, planes=3, plane_stride=planes.stride(0))
+    assert torch.equal(q1, q3) and torch.equal(kc1, kc3) and torch.equal(vc1, vc3)
 
 
 def attention_case(H, KVH, Dh, bs, lens_new, lens_ctx, seed, dtype=torch.float32, window=None, spike=None):
@@ -244,6 +253,37 @@ def test_skinny_gemm_bf16(M, N, K):
     one = torch.empty(1, N, dtype=torch.float32, device="cuda")
     kernels.skinny_gemm_bf16(x[M - 1:M].contiguous(), w, one)
     assert torch.equal(one[0], out[M - 1])
+    # cut along K: planes of partial sums that add up to the product, again the same for a row alone
+    for splits in (2, 3):
+        planes = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device="cuda")
+        kernels.skinny_gemm_bf16(x, w, planes, splits=splits)
+        close(planes.cpu().to(F64).sum(0), want, 1e-5, f"skinny gemm in {splits} planes")
+        alone = torch.empty(splits, 1, N, dtype=torch.float32, device="cuda")
+        kernels.skinny_gemm_bf16(x[M - 1:M].contiguous(), w, alone, splits=splits)
+        assert torch.equal(alone[:, 0], planes[:, M - 1])
+
+
+@pytest.mark.parametrize("R,n", [(1, 24), (5, 200), (8, 4096), (64, 1024), (3, 20000)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_add_partials_alone_and_with_rms_norm(R, n, out_dtype):
+    from tie_amd import kernels
+
+    x = rnd(R, n, seed=51).cuda()
+    planes = rnd(3, R, n, seed=52).cuda()
+    w = (1 + 0.1 * rnd(n, seed=53)).cuda()
+    total = x.cpu().to(F64) + planes.cpu().to(F64).sum(0)
+    added = x.clone()
+    kernels.add_partials(added, planes)
+    close(added, total, 1e-6, "add_partials")
+    both = x.clone()
+    out = torch.full((R, n), float("nan"), dtype=out_dtype, device="cuda")
+    kernels.add_partials(both, planes, w, 1e-5, out)
+    assert torch.equal(both, added)                    # the stream holds the same sum either way
+    close(out, plain.rms_norm(total, w.cpu(), 1e-5), 1e-5 if out_dtype == torch.float32 else 5e-3, "add + rms_norm")
+    # and the norm of the sum is the norm kernel's own result on the updated stream
+    separate = torch.empty_like(out)
+    kernels.rms_norm(added, w, 1e-5, separate)
+    assert torch.equal(separate, out)
 
 
 

@@ -235,6 +235,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
   for (int k = 0; k < nsplit; ++k) L += weighted_sum[k];   // ascending order, the same in every thread
   for (int d = threadIdx.x; d < DH; d += blockDim.x) {
     float o = 0.f;
+#pragma unroll 8
     for (int k = 0; k < nsplit; ++k) o += part_o[(slot0 + k) * DH + d] * weight[k];
     out[(static_cast<size_t>(t) * H + h) * DH + d] = float_to_bf16(o / L);
   }

@@ -63,34 +63,68 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, const float* __restric
   }
 }
 
-// The same for float32 rows of up to 16 values a thread (n % 4 == 0): the row is read once and
-// stays in registers between the sum of squares and the scaling.
-template <typename TO>
-__global__ void rms_norm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, float eps,
-                                    TO* __restrict__ out, const int* __restrict__ rows, int n) {
+// Float32 rows of up to four float4 a thread (n % 4 == 0) stay in registers between the sum of
+// squares and the scaling. With COUNT > 0 the row first receives COUNT planes of partial sums
+// (x[r] += p_0[r] + p_1[r] + ..., written back): see the section on partial sums below. All loads
+// of a thread are issued before the first use; the kernel is bound by latency, not by bytes.
+template <typename TO, int COUNT, int V>
+__global__ void rms_norm_row_kernel(float* __restrict__ x, const float* __restrict__ partials, size_t plane_stride,
+                                    const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                    const int* __restrict__ rows, int n) {
   __shared__ float scratch[16];
-  const int r = blockIdx.x;
-  const float* xr = x + static_cast<size_t>(rows ? rows[r] : r) * n;
-  TO* o = out + static_cast<size_t>(r) * n;
-  float4 v[4];
+  const size_t row = static_cast<size_t>(rows ? rows[blockIdx.x] : blockIdx.x) * n;
+  TO* o = out + static_cast<size_t>(blockIdx.x) * n;
+  float4 v[V], p[COUNT > 0 ? COUNT : 1][V], wv[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    const bool in = i < n;
+    v[j] = in ? *reinterpret_cast<const float4*>(x + row + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    wv[j] = in ? *reinterpret_cast<const float4*>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int s = 0; s < COUNT; ++s)
+      p[s][j] = in ? *reinterpret_cast<const float4*>(partials + static_cast<size_t>(s) * plane_stride + row + i)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < V; ++j) {
+#pragma unroll
+    for (int s = 0; s < COUNT; ++s) {
+      v[j].x += p[s][j].x;
+      v[j].y += p[s][j].y;
+      v[j].z += p[s][j].z;
+      v[j].w += p[s][j].w;
+    }
     const int i = (threadIdx.x + j * blockDim.x) * 4;
-    v[j] = i < n ? *reinterpret_cast<const float4*>(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (COUNT > 0 && i < n) *reinterpret_cast<float4*>(x + row + i) = v[j];
     ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
   }
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < V; ++j) {
     const int i = (threadIdx.x + j * blockDim.x) * 4;
     if (i >= n) continue;
-    const float4 wv = *reinterpret_cast<const float4*>(w + i);
-    store_from_float(o + i, (v[j].x * inv) * wv.x);
-    store_from_float(o + i + 1, (v[j].y * inv) * wv.y);
-    store_from_float(o + i + 2, (v[j].z * inv) * wv.z);
-    store_from_float(o + i + 3, (v[j].w * inv) * wv.w);
+    store_from_float(o + i, (v[j].x * inv) * wv[j].x);
+    store_from_float(o + i + 1, (v[j].y * inv) * wv[j].y);
+    store_from_float(o + i + 2, (v[j].z * inv) * wv[j].z);
+    store_from_float(o + i + 3, (v[j].w * inv) * wv[j].w);
+  }
+}
+
+template <typename TO, int COUNT>
+static void launch_rms_norm_row(float* x, const float* partials, size_t stride, const float* w, float eps, TO* out,
+                                const int* rows, int R, int n, hipStream_t stream) {
+  // As many threads as the row has float4, up to 1024: measured faster than fewer threads with more loads each.
+  const int quads = n / 4;
+  if (quads <= 1024) {
+    const int threads = (quads + TIE_WAVE - 1) / TIE_WAVE * TIE_WAVE;
+    rms_norm_row_kernel<TO, COUNT, 1><<<R, threads, 0, stream>>>(x, partials, stride, w, eps, out, rows, n);
+  } else if (quads <= 2048) {
+    rms_norm_row_kernel<TO, COUNT, 2><<<R, 1024, 0, stream>>>(x, partials, stride, w, eps, out, rows, n);
+  } else {
+    rms_norm_row_kernel<TO, COUNT, 4><<<R, 1024, 0, stream>>>(x, partials, stride, w, eps, out, rows, n);
   }
 }
 
@@ -98,15 +132,10 @@ extern "C" int tie_rms_norm(const void* x, int x_dtype, const float* w, float ep
                             const int* rows, int R, int n, hipStream_t stream) {
   if (R <= 0 || n <= 0) return TIE_BAD_ARGUMENT;
   if (x_dtype == TIE_F32 && n % 4 == 0 && n <= 16384 && n >= 256) {
-    const int threads = n <= 1024 ? 64 : (n <= 4096 ? 256 : (n <= 8192 ? 512 : 1024));
-    if (out_dtype == TIE_F32)
-      rms_norm_row_kernel<float><<<R, threads, 0, stream>>>(static_cast<const float*>(x), w, eps,
-                                                            static_cast<float*>(out), rows, n);
-    else if (out_dtype == TIE_BF16)
-      rms_norm_row_kernel<bf16_t><<<R, threads, 0, stream>>>(static_cast<const float*>(x), w, eps,
-                                                             static_cast<bf16_t*>(out), rows, n);
-    else
-      return TIE_BAD_ARGUMENT;
+    float* xf = static_cast<float*>(const_cast<void*>(x));   // without planes the kernel only reads it
+    if (out_dtype == TIE_F32) launch_rms_norm_row<float, 0>(xf, nullptr, 0, w, eps, static_cast<float*>(out), rows, R, n, stream);
+    else if (out_dtype == TIE_BF16) launch_rms_norm_row<bf16_t, 0>(xf, nullptr, 0, w, eps, static_cast<bf16_t*>(out), rows, R, n, stream);
+    else return TIE_BAD_ARGUMENT;
     return tie_launch_status();
   }
   const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
@@ -170,6 +199,61 @@ extern "C" int tie_cast(const void* x, int in_dtype, void* out, int out_dtype, l
   return tie_launch_status();
 }
 
+// ------------------------------------------------- partial sums (+ RMSNorm)
+// A matrix product cut along K leaves `count` planes of partial sums, plane_stride floats apart.
+// x[r, i] += p_0[r, i] + p_1[r, i] + ... in plane order (float32, the residual stream), and, with a
+// norm weight, out[r, :] = RMSNorm(x[r, :]) * w of the updated row in the same pass: the row is
+// read once, and the product's result never makes a round trip of its own through memory.
+__device__ __forceinline__ float add_planes(float v, const float* __restrict__ p, size_t plane_stride, int count) {
+  for (int s = 0; s < count; ++s) v += p[static_cast<size_t>(s) * plane_stride];
+  return v;
+}
+
+template <typename TO>
+__global__ void add_partials_rms_norm_kernel(float* __restrict__ x, const float* __restrict__ partials,
+                                             size_t plane_stride, int count, const float* __restrict__ w, float eps,
+                                             TO* __restrict__ out, int n) {
+  __shared__ float scratch[16];
+  const size_t row = static_cast<size_t>(blockIdx.x) * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = add_planes(x[row + i], partials + row + i, plane_stride, count);
+    x[row + i] = v;     // read back below by the thread that wrote it
+    ss += v * v;
+  }
+  if (w == nullptr) return;
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) store_from_float(out + row + i, (x[row + i] * inv) * w[i]);
+}
+
+// w (and out) null: only the addition.
+extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long plane_stride, int count, const float* w,
+                                         float eps, void* out, int out_dtype, int R, int n, hipStream_t stream) {
+  if (R <= 0 || n <= 0 || count <= 0 || plane_stride < static_cast<long>(R) * n || (w != nullptr && out == nullptr))
+    return TIE_BAD_ARGUMENT;
+  if (w != nullptr && out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
+  const size_t stride = static_cast<size_t>(plane_stride);
+  if (w != nullptr && n % 4 == 0 && plane_stride % 4 == 0 && n <= 16384 && n >= 256 && count <= 3) {
+#define ROW(TO, COUNT) launch_rms_norm_row<TO, COUNT>(x, partials, stride, w, eps, static_cast<TO*>(out), nullptr, R, n, stream)
+    if (out_dtype == TIE_F32) {
+      if (count == 1) ROW(float, 1); else if (count == 2) ROW(float, 2); else ROW(float, 3);
+    } else {
+      if (count == 1) ROW(bf16_t, 1); else if (count == 2) ROW(bf16_t, 2); else ROW(bf16_t, 3);
+    }
+#undef ROW
+    return tie_launch_status();
+  }
+  const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
+  if (w == nullptr || out_dtype == TIE_F32)
+    add_partials_rms_norm_kernel<float><<<R, threads, 0, stream>>>(x, partials, stride, count, w, eps,
+                                                                   static_cast<float*>(out), n);
+  else
+    add_partials_rms_norm_kernel<bf16_t><<<R, threads, 0, stream>>>(x, partials, stride, count, w, eps,
+                                                                    static_cast<bf16_t*>(out), n);
+  return tie_launch_status();
+}
+
 // ------------------------------------------ QK-norm + rotary + cache write
 // One wave per (token, head slot). Head slots 0..H-1 are query heads, then KVH
 // key heads, then KVH value heads of the fused projection row
@@ -185,8 +269,17 @@ extern "C" int tie_cast(const void* x, int in_dtype, void* out, int out_dtype, l
 // Norm weights or inv_freq may be null: that step is then skipped. With k_dense set, keys are
 // written there (row stride k_row) instead of into the cache; without write_kv and k_dense only
 // the query heads are processed. q_out and k_dense may alias qkv (each wave holds its head in
-// registers before it writes).
+// registers before it writes). The input may come as `planes` partial sums, plane_stride elements
+// apart (a product cut along K): they are added in plane order as they are read.
 #define TIE_MAX_PAIRS 4  // head_dim <= 512
+
+template <typename TX>
+__device__ __forceinline__ float load_planes(const TX* p, size_t plane_stride, int planes) {
+  float v = load_as_float(p);
+  if (planes == 2) return v + load_as_float(p + plane_stride);   // the usual cut: both loads in flight together
+  for (int s = 1; s < planes; ++s) v += load_as_float(p + static_cast<size_t>(s) * plane_stride);
+  return v;
+}
 
 template <typename TX, typename TQ, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
@@ -194,7 +287,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
                                              const float* __restrict__ inv_freq,
                                              const int* __restrict__ positions, const int* __restrict__ slots,
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
-                                             int KVH, int Dh, int block_size, int in_row, int q_row, int k_row) {
+                                             int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
+                                             size_t plane_stride, int planes) {
   const int t = blockIdx.y;
   const int slot_index = blockIdx.x;
   const int lane = threadIdx.x;
@@ -208,7 +302,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     const int h = slot_index - H - KVH;
     const int slot = slots[t];
     TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + h) * Dh * block_size + slot % block_size;
-    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + static_cast<size_t>(d) * block_size, load_as_float(in + d));
+    for (int d = lane; d < Dh; d += TIE_WAVE) store_from_float(dst + static_cast<size_t>(d) * block_size, load_planes(in + d, plane_stride, planes));
     return;
   }
 
@@ -220,8 +314,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     x1[i] = 0.f;
     x2[i] = 0.f;
     if (p < half) {
-      x1[i] = load_as_float(in + p);
-      x2[i] = load_as_float(in + p + half);
+      x1[i] = load_planes(in + p, plane_stride, planes);
+      x2[i] = load_planes(in + p + half, plane_stride, planes);
       ss += x1[i] * x1[i] + x2[i] * x2[i];
     }
   }
@@ -276,7 +370,8 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                                          const int* positions, const int* slots, void* k_cache, void* v_cache,
                                          int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
-                                         hipStream_t stream) {
+                                         long plane_stride, int planes, hipStream_t stream) {
+  if (planes < 1 || (planes > 1 && plane_stride < static_cast<long>(T) * in_row)) return TIE_BAD_ARGUMENT;
   if (T <= 0 || H <= 0 || KVH <= 0 || Dh <= 0 || Dh % 2 != 0 || Dh > 2 * TIE_MAX_PAIRS * TIE_WAVE ||
       block_size <= 0 || T > 65535 || q_row < H * Dh)
     return TIE_BAD_ARGUMENT;
@@ -289,7 +384,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, positions, slots,       \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
-      block_size, in_row, q_row, k_row)
+      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);

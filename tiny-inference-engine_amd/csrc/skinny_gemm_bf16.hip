@@ -1,14 +1,20 @@
 // The decode-time matrix product for gfx950: out[M, N] (+)= x[M, K] . w[N, K]^T for few rows M
 // (1..64), bfloat16 operands, float32 accumulation on v_mfma_f32_16x16x32_bf16.
 //
-// The product is bound by reading w once from HBM, so the kernel is built around that stream:
-// a workgroup of four (or eight) waves owns 16 rows of w; the waves split K into contiguous ranges;
-// every lane reads 16 bytes of "its" row per MFMA (row = lane % 16, k-chunk = lane / 16), which
-// is exactly the B-operand layout, so weights go from memory to the matrix core with no staging.
-// The few rows of x are the A operand, read through the caches (they are shared by every
-// workgroup); rows beyond M are zeros. The waves' partial sums meet in LDS and are added in a fixed
-// order, so the result does not depend on timing. M > 16 runs 2 or 4 row tiles of x against each
-// weight fragment.
+// The product is bound by reading w once from HBM, so the kernel is built around that stream.
+// A workgroup of four waves owns RT tiles of 16 rows of w and one of `splits` ranges of K; its
+// waves split that range into contiguous parts. Every lane reads 16 bytes of "its" row per MFMA
+// (row = lane % 16, k-chunk = lane / 16), which is exactly the B-operand layout, so weights go from
+// memory to the matrix core with no staging. The few rows of x are the A operand, read through the
+// caches (they are shared by every workgroup); rows beyond M are zeros. One x fragment feeds the
+// RT weight tiles of the wave, which is what keeps the x traffic below the weight traffic when M
+// grows: RT is chosen per launch from M and the number of workgroups that results. The waves'
+// partial sums meet in LDS and are added in a fixed order.
+//
+// With splits > 1 the output is [splits, M, N] float32 partial sums, one plane per range of K, for
+// the consumer to add up in plane order (no atomics, no fences: the result is the same in every
+// run). How K is cut depends on K and splits alone, never on M or RT, so a row's sums are formed in
+// the same order whatever else is in the batch.
 //
 // Requires K % 8 == 0 (16-byte loads); other shapes go to the generic kernel.
 #include "common.h"
@@ -16,7 +22,7 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-#define SK_UNROLL 4
+#define SK_WAVES 4
 
 __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p) {
   const uint4 v = *reinterpret_cast<const uint4*>(p);
@@ -28,20 +34,23 @@ __device__ __forceinline__ bf16x8_t zero_frag() {
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
-template <int MT, typename TO, int SK_WAVES>
+// MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 loaded ahead of the MFMAs.
+template <int MT, int RT, int U, typename TO>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
-                                                                         int accumulate, int gated) {
-  __shared__ float red[SK_WAVES][MT][256];
+                                                                         int accumulate, int gated, int per_wave) {
+  __shared__ float red[SK_WAVES][MT][RT][256];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const int r = lane & 15;   // row of the 16-row tile (of w for B, of x for A)
   const int g = lane >> 4;   // which 8-element chunk of the 32-wide k block
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * RT;
 
   // Rows beyond N are clamped for the loads; their columns are dropped at the store.
-  const bf16_t* wp = w + static_cast<size_t>(min(n0 + r, N - 1)) * K;
+  const bf16_t* wp[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) wp[t] = w + static_cast<size_t>(min(n0 + t * 16 + r, N - 1)) * K;
   const bf16_t* xp[MT];
   bool xvalid[MT];
 #pragma unroll
@@ -51,43 +60,50 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     xp[mt] = x + static_cast<size_t>(xvalid[mt] ? m : 0) * K;
   }
 
-  // This wave's k range, in blocks of 32.
+  // This wave's k range, in blocks of 32: part (split, wave) of gridDim.y * SK_WAVES equal parts.
   const int kblocks = (K + 31) / 32;
-  const int per_wave = (kblocks + SK_WAVES - 1) / SK_WAVES;
-  const int kb_begin = wave * per_wave;
+  const int kb_begin = min(kblocks, (static_cast<int>(blockIdx.y) * SK_WAVES + wave) * per_wave);
   const int kb_end = min(kblocks, kb_begin + per_wave);
 
-  floatx4 acc[MT];
+  floatx4 acc[MT][RT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   int kb = kb_begin;
-  // Main loop: SK_UNROLL blocks at a time, all loads issued before the first MFMA.
-  for (; kb + SK_UNROLL <= kb_end && (kb + SK_UNROLL) * 32 <= K; kb += SK_UNROLL) {
-    bf16x8_t b[SK_UNROLL];
-    bf16x8_t a[MT][SK_UNROLL];
+  // Main loop: U blocks at a time, all loads issued before the first MFMA.
+  for (; kb + U <= kb_end && (kb + U) * 32 <= K; kb += U) {
+    bf16x8_t b[RT][U];
+    bf16x8_t a[MT][U];
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int k = (kb + u) * 32 + g * 8;
-      b[u] = load_frag(wp + k);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) b[t][u] = load_frag(wp[t] + k);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) a[mt][u] = xvalid[mt] ? load_frag(xp[mt] + k) : zero_frag();
     }
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt][u], b[u], acc[mt], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt][u], b[t][u], acc[mt][t], 0, 0, 0);
   }
-  // Remainder, one block at a time; the last block may be partly or wholly beyond K.
+  // Remainder, one block at a time; the last block may be partly beyond K.
   for (; kb < kb_end; ++kb) {
     const int k = kb * 32 + g * 8;
     const bool kvalid = k < K;  // K % 8 == 0: a chunk is whole or absent
-    const bf16x8_t b = kvalid ? load_frag(wp + k) : zero_frag();
+    bf16x8_t a[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8_t a = (kvalid && xvalid[mt]) ? load_frag(xp[mt] + k) : zero_frag();
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+    for (int mt = 0; mt < MT; ++mt) a[mt] = (kvalid && xvalid[mt]) ? load_frag(xp[mt] + k) : zero_frag();
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const bf16x8_t b = kvalid ? load_frag(wp[t] + k) : zero_frag();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], b, acc[mt][t], 0, 0, 0);
     }
   }
 
@@ -95,57 +111,105 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][mt][(g * 4 + v) * 16 + r] = acc[mt][v];
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[wave][mt][t][(g * 4 + v) * 16 + r] = acc[mt][t][v];
   __syncthreads();
 
-  for (int e = threadIdx.x; e < 256; e += SK_WAVES * TIE_WAVE) {  // 16 x 16 outputs of a tile
-    const int c = e & 15;
-    const int n = n0 + c;
-    if (n >= N) continue;
+  const bool partial = gridDim.y > 1;   // then TO is float and out holds one [M, N] plane per split
+  for (int e = threadIdx.x; e < 256 * RT * MT; e += SK_WAVES * TIE_WAVE) {
+    const int ee = e & 255;            // 16 x 16 outputs of a tile
+    const int t = (e >> 8) % RT;
+    const int mt = e / (256 * RT);
+    const int c = ee & 15;
+    const int m = mt * 16 + (ee >> 4);
+    const int n = n0 + t * 16 + c;
+    if (m >= M || n >= N) continue;
     if (gated && c >= 8) continue;       // gated: columns 0..7 are gates, 8..15 the ups of the same outputs
+    float sum = red[0][mt][t][ee];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = mt * 16 + (e >> 4);
-      if (m >= M) continue;
-      float sum = red[0][mt][e];
+    for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][t][ee];
+    if (gated) {
+      float up = red[0][mt][t][ee + 8];
 #pragma unroll
-      for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][e];
-      if (gated) {
-        float up = red[0][mt][e + 8];
-#pragma unroll
-        for (int wv = 1; wv < SK_WAVES; ++wv) up += red[wv][mt][e + 8];
-        store_from_float(out + static_cast<size_t>(m) * (N / 2) + blockIdx.x * 8 + c, sum / (1.0f + __expf(-sum)) * up);
-        continue;
-      }
-      TO* o = out + static_cast<size_t>(m) * N + n;
-      if (accumulate) sum = load_as_float(o) + sum;
-      store_from_float(o, sum);
+      for (int wv = 1; wv < SK_WAVES; ++wv) up += red[wv][mt][t][ee + 8];
+      store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
+      continue;
     }
+    TO* o = out + (static_cast<size_t>(partial ? blockIdx.y : 0) * M + m) * N + n;
+    if (accumulate) sum = load_as_float(o) + sum;
+    store_from_float(o, sum);
   }
 }
 
+static int compute_units() {
+  static int cached = 0;
+  if (cached == 0) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      count = 256;
+    cached = count;
+  }
+  return cached;
+}
+
+// Weight tiles per workgroup. More tiles reuse each x fragment more often (x costs about half a
+// weight tile's traffic per 16 rows of it) but leave fewer workgroups, which hurts when their number
+// is not a multiple of the compute units. Does not change any sum.
+static int choose_rt(int M, int N, int splits) {
+  if (M <= 4) return 1;
+  const int cus = compute_units();
+  const int tiles = (N + 15) / 16;
+  int best = 1;
+  double best_cost = 0;
+  for (int rt = 1; rt <= (M > 8 ? 4 : 3); ++rt) {
+    const long wgs = static_cast<long>((tiles + rt - 1) / rt) * splits;
+    const double fill = static_cast<double>(wgs) / static_cast<double>((wgs + cus - 1) / cus * cus);
+    const double cost = (1.0 + 0.5 * (M / 16.0) / rt) / fill;
+    if (rt == 1 || cost <= best_cost) {
+      best = rt;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+// Ranges of K that a product over w[N, K] is cut into when its caller takes partial sums: weights with
+// few rows would otherwise give too few workgroups. By the shape of w alone.
+extern "C" int tie_skinny_gemm_splits(int N, int K) { return (N < 8192 && K >= 512) ? 2 : 1; }
+
 // gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
 // and receives silu(gate) * up.
+// splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
-                                    int M, int N, int K, hipStream_t stream) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0) return TIE_BAD_ARGUMENT;
-  if (gated && (accumulate || N % 16 != 0)) return TIE_BAD_ARGUMENT;
-  const dim3 grid((N + 15) / 16);
+                                    int M, int N, int K, int splits, hipStream_t stream) {
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1 || splits > 64) return TIE_BAD_ARGUMENT;
+  if (gated && (accumulate || N % 16 != 0 || splits != 1)) return TIE_BAD_ARGUMENT;
+  if (splits > 1 && (accumulate || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  // Few workgroups (small N) or long rows: eight waves a workgroup keep more loads in flight.
-  const bool wide = grid.x <= 512 || K >= 8192;   // by the shape of w alone: every M sums in the same order
-#define LAUNCH(MT, TO, WAVES)                                                                                   \
-  skinny_gemm_kernel<MT, TO, WAVES><<<grid, WAVES * TIE_WAVE, 0, stream>>>(                                      \
-      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, gated)
-  if (out_dtype == TIE_F32) {
-    if (wide) { if (mt == 1) LAUNCH(1, float, 8); else if (mt == 2) LAUNCH(2, float, 8); else LAUNCH(4, float, 8); }
-    else { if (mt == 1) LAUNCH(1, float, 4); else if (mt == 2) LAUNCH(2, float, 4); else LAUNCH(4, float, 4); }
-  } else if (out_dtype == TIE_BF16) {
-    if (wide) { if (mt == 1) LAUNCH(1, bf16_t, 8); else if (mt == 2) LAUNCH(2, bf16_t, 8); else LAUNCH(4, bf16_t, 8); }
-    else { if (mt == 1) LAUNCH(1, bf16_t, 4); else if (mt == 2) LAUNCH(2, bf16_t, 4); else LAUNCH(4, bf16_t, 4); }
-  } else {
-    return TIE_BAD_ARGUMENT;
-  }
+  const int rt = choose_rt(M, N, splits);
+  const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
+  const int kblocks = (K + 31) / 32;
+  const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
+#define LAUNCH(MT, RT, U, TO)                                                                                \
+  skinny_gemm_kernel<MT, RT, U, TO><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                                \
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
+      gated, per_wave)
+#define LAUNCH_RT(MT, TO)                                  \
+  if (rt == 1) LAUNCH(MT, 1, 4, TO);                       \
+  else if (rt == 2) LAUNCH(MT, 2, 4, TO);                  \
+  else if (rt == 3) LAUNCH(MT, 3, 2, TO);                  \
+  else LAUNCH(MT, 4, 2, TO)
+#define LAUNCH_MT(TO)                                      \
+  if (mt == 1) { LAUNCH_RT(1, TO); }                       \
+  else if (mt == 2) { LAUNCH_RT(2, TO); }                  \
+  else { LAUNCH_RT(4, TO); }
+  if (out_dtype == TIE_F32) { LAUNCH_MT(float) }
+  else if (out_dtype == TIE_BF16) { LAUNCH_MT(bf16_t) }
+  else return TIE_BAD_ARGUMENT;
+#undef LAUNCH_MT
+#undef LAUNCH_RT
 #undef LAUNCH
   return tie_launch_status();
 }

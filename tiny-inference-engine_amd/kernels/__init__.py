@@ -20,7 +20,7 @@ from . import build
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
-_c_int, _c_float, _c_void = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+_c_int, _c_float, _c_void, _c_long = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_long
 
 # library key -> (file stem, source)
 _SOURCES = {
@@ -45,7 +45,9 @@ _SIGNATURES = {
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_void],
+        "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
+                                      _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
@@ -59,7 +61,9 @@ _SIGNATURES = {
                                         _c_int, _c_void],
     },
     "skinny_gemm_bf16": {
-        "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_skinny_gemm_splits": [_c_int, _c_int],
+        "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                 _c_void],
     },
     "gemm_bf16": {
         "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -217,6 +221,31 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
                                             _stream()), "rms_norm")
 
 
+def add_partials(x: torch.Tensor, partials: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                 out: Optional[torch.Tensor] = None) -> None:
+    """x += partials[0] + partials[1] + ... (float32, in plane order); with ``weight``, out = RMSNorm(x) * weight too.
+
+    ``partials`` is the ``[S, R, n]`` output of a product cut along K (``skinny_gemm_bf16(splits=S)``).
+    """
+    _gpu(x, "partial sums' target")
+    _gpu(partials, "partial sums")
+    if x.dtype != torch.float32 or partials.dtype != torch.float32 or partials.dim() != 3 or x.dim() != 2 or \
+            tuple(partials.shape[1:]) != tuple(x.shape):
+        raise InvalidArgument(f"add_partials: target {list(x.shape)} {x.dtype}, partial sums {list(partials.shape)} "
+                              f"{partials.dtype}; both must be float32 and the planes shaped like the target")
+    R, n = x.shape
+    code = F32
+    if weight is not None:
+        _f32(weight, "rms_norm weight", (n,))
+        _gpu(out, "rms_norm output")
+        if tuple(out.shape) != (R, n):
+            raise InvalidArgument(f"rms_norm output {list(out.shape)} does not match input {[R, n]}")
+        code = _code(out, "rms_norm output")
+    _check(_lib("elementwise").tie_add_partials_rms_norm(
+        x.data_ptr(), partials.data_ptr(), R * n, partials.shape[0], _ptr(weight), float(eps), _ptr(out), code, R, n,
+        _stream()), "add_partials")
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up of shape [T, 2I]."""
     _gpu(gate_up, "swiglu input")
@@ -269,20 +298,33 @@ def _bf16_product_operands(x, w, out, gated, what):
     return M, N, K
 
 
+def skinny_splits(N: int, K: int) -> int:
+    """Ranges of K a decode-time product over a ``[N, K]`` weight is best cut into when its caller adds partial sums."""
+    return int(_lib("skinny_gemm_bf16").tie_skinny_gemm_splits(N, K))
+
+
 def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-                     gated: bool = False) -> None:
+                     gated: bool = False, splits: int = 1) -> None:
     """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores.
 
     ``gated``: w is a gate/up pair interleaved by ``interleave_gate_up`` and out receives silu(gate) * up.
+    ``splits`` > 1: out is ``[splits, M, N]`` float32 and receives one plane of partial sums per range
+    of K, for the consumer to add (``add_partials``, or a kernel that takes planes).
     """
-    M, N, K = _bf16_product_operands(x, w, out, gated, "skinny_gemm_bf16")
+    if splits > 1:
+        if out.dim() != 3 or out.shape[0] != splits or out.dtype != torch.float32 or accumulate or gated:
+            raise InvalidArgument(f"skinny_gemm_bf16: {splits} splits need a float32 output of {splits} planes, "
+                                  f"got {list(out.shape)} {out.dtype}, and neither accumulate nor gated")
+        M, N, K = _bf16_product_operands(x, w, out[0], gated, "skinny_gemm_bf16")
+    else:
+        M, N, K = _bf16_product_operands(x, w, out, gated, "skinny_gemm_bf16")
     if M > 64:
         raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows, got {M}")
     if gated and accumulate:
         raise InvalidArgument("a gated product does not accumulate")
     _check(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16(
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
-        _stream()), "skinny_gemm_bf16")
+        int(splits), _stream()), "skinny_gemm_bf16")
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0,
@@ -331,8 +373,12 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
                           k_weight: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
                           positions: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                           v_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
-                          block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None) -> None:
+                          block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
+                          planes: int = 1, plane_stride: int = 0) -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
+
+    With ``planes`` > 1, ``qkv`` is the first of that many planes of partial sums, ``plane_stride``
+    elements apart, which are added as they are read.
 
     ``qkv`` is ``[T, >= (H + 2 KVH) * Dh]`` (rows may be wider than what is read). ``q_out`` is a
     ``[T, H * Dh]`` tensor or a view into ``qkv`` itself (rows ``qkv.stride(0)`` apart). With
@@ -378,8 +424,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
         _ptr(k_weight), float(eps), _ptr(inv_freq), positions.data_ptr(), _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
-        _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, _stream()),
-        "qk_norm_rope_kv_write")
+        _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
+        _stream()), "qk_norm_rope_kv_write")
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,

@@ -94,7 +94,9 @@ class Model:
             layer = self.layers[call.layer]
             layer.block.forward(ctx, x, layer, ctx.cache_of(index))
             if self.layer_hook is not None:
+                ctx.settle()
                 self.layer_hook(index, x)
+        ctx.settle()     # the last layer's product may still be owed to the stream
         if batch.num_logit_rows == 0:
             return None
         return self.head.forward(ctx, x, batch.logit_rows)

@@ -77,16 +77,22 @@ class PagedAttention(Mixer):
         step = cache.step
         eps = float(self.qk_norm["eps"]) if self.qk_norm else 0.0
 
-        qkv = ctx.scratch("attention.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-        self.qkv(h, qkv)
+        width = self.q_dim + 2 * self.kv_dim
         q = ctx.scratch("attention.q", (T, self.q_dim))
         table = self.position.rotary_table()
+        # Decode-size steps: the projection comes as planes of partial sums, added by the kernel that reads them.
+        planes = self.qkv.partial_planes(ctx, h, "attention.qkv") if table is not None else None
+        if planes is not None:
+            qkv = planes[0]
+        else:
+            qkv = ctx.scratch("attention.qkv", (T, width), torch.float32)
+            self.qkv(h, qkv)
         if table is not None:
             inv_freq = table[0]
             kernels.qk_norm_rope_kv_write(
                 qkv, q, self.q_norm_weight, self.k_norm_weight, eps, inv_freq, ctx.batch.positions,
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
-                write_kv=cache.writes)
+                write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width)
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.
@@ -105,4 +111,4 @@ class PagedAttention(Mixer):
         attn = ctx.scratch("attention.out", (T, self.q_dim))
         kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window,
                                 scratch=ctx.scratch)
-        self.out(attn, residual, accumulate=True)
+        self.out(attn, residual, accumulate=True, ctx=ctx)

@@ -16,7 +16,9 @@ takes them at load time (``load``) and runs on a StepContext.
 The residual stream is float32 in both compute modes; ``h`` (a norm's output,
 a matrix product's input) has the activation dtype of the mode. Mixers and
 feed-forwards ADD their result to the ``residual`` tensor they are given, which
-lets the last matrix product of a part fold the addition into its epilogue.
+lets the last matrix product of a part fold the addition into its epilogue, or
+leave it owed to the stream (``StepContext.defer_add``) for the next norm to add
+in the pass in which it reads the stream anyway.
 """
 
 from __future__ import annotations
@@ -141,6 +143,7 @@ class StepContext:
         self.cache_plan = cache_plan
         self.act_dtype = torch.float32 if mode == FLOAT32 else torch.bfloat16
         self.notes: Dict[Any, Any] = {}   # per-step memo shared by parts (e.g. one plan for all layers)
+        self._owed = None                  # (target, planes): target += planes[0] + planes[1] + ... is still to be done
 
     @property
     def num_tokens(self) -> int:
@@ -148,6 +151,30 @@ class StepContext:
 
     def scratch(self, name: str, shape, dtype: torch.dtype = None) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype or self.act_dtype)
+
+    # A product cut along K hands its planes of partial sums to the step instead of adding them; the
+    # next reader of the target adds them in its own pass (a norm does) or has them added by settle().
+    def defer_add(self, target: torch.Tensor, planes: torch.Tensor) -> None:
+        self.settle()
+        self._owed = (target, planes)
+
+    def take_owed(self, target: torch.Tensor) -> Optional[torch.Tensor]:
+        """The planes still owed to ``target`` (the caller now adds them itself), or None; other debts are settled."""
+        if self._owed is None:
+            return None
+        owed_to, planes = self._owed
+        if owed_to.data_ptr() == target.data_ptr() and owed_to.shape == target.shape:
+            self._owed = None
+            return planes
+        self.settle()
+        return None
+
+    def settle(self) -> None:
+        if self._owed is not None:
+            from .. import kernels
+            target, planes = self._owed
+            self._owed = None
+            kernels.add_partials(target, planes)
 
     def cache_of(self, call_index: int):
         """The cache binding of run-order entry ``call_index`` (None if its mixer has no cache)."""
@@ -188,6 +215,8 @@ class StateBinding:
 
 
 class Norm(Part):
+    adds_owed = False   # True: forward() adds partial sums owed to x (ctx.take_owed) in its own pass
+
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
                 out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
         raise NotImplementedError
@@ -225,7 +254,17 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """The arrangement of one layer's parts. ``layer`` carries .mixer, .feed_forward and .norms."""
+    """The arrangement of one layer's parts. ``layer`` carries .mixer, .feed_forward and .norms.
+
+    An arrangement settles what is owed to the residual stream before it hands the stream to a part
+    that does not add the debt itself (``normed`` does so for norms).
+    """
+
+    @staticmethod
+    def normed(ctx: StepContext, norm, x: torch.Tensor) -> torch.Tensor:
+        if not norm.adds_owed:
+            ctx.settle()
+        return norm.forward(ctx, x)
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
         raise NotImplementedError

@@ -19,9 +19,9 @@ class PreNormBlock(Block):
     NORMS = ("pre_mixer", "pre_feed_forward")
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
-        h = layer.norms["pre_mixer"].forward(ctx, x)
+        h = self.normed(ctx, layer.norms["pre_mixer"], x)
         layer.mixer.forward(ctx, h, cache, x)
-        h = layer.norms["pre_feed_forward"].forward(ctx, x)
+        h = self.normed(ctx, layer.norms["pre_feed_forward"], x)
         layer.feed_forward.forward(ctx, h, x)
 
     @classmethod

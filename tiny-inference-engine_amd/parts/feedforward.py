@@ -53,4 +53,4 @@ class SwiGLU(FeedForward):
             gate_up = ctx.scratch("swiglu.gate_up", (T, 2 * self.intermediate))
             self.gate_up(h, gate_up)
             kernels.swiglu(gate_up, act)
-        self.down(act, residual, accumulate=True)
+        self.down(act, residual, accumulate=True, ctx=ctx)

@@ -27,6 +27,7 @@ class Linear:
         self.in_features = in_features
         self.init_std = init_std
         self.weight: torch.Tensor = None
+        self._splits = None
 
     @property
     def total_out(self) -> int:
@@ -46,6 +47,31 @@ class Linear:
             parts = [p.to(torch.float32) for p in parts]
         self.weight = torch.cat(parts, dim=0).contiguous()
 
-    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ctx=None) -> torch.Tensor:
+        """out (+)= x @ W^T. With ``ctx`` an accumulating product may leave its addition owed to ``out``.
+
+        A decode-size product over a weight of few rows is cut along K into planes of partial sums;
+        the step context remembers that their sum is still to be added, and the next norm over
+        ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once.
+        """
+        if ctx is not None and accumulate and out.dtype == torch.float32:
+            planes = self.partial_planes(ctx, x, "linear.partials")
+            if planes is not None:
+                ctx.defer_add(out, planes)
+                return out
         kernels.linear(x, self.weight, out, accumulate)
         return out
+
+    def partial_planes(self, ctx, x: torch.Tensor, name: str):
+        """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None."""
+        M, K = x.shape
+        w = self.weight
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or M > 64 or K % 8:
+            return None
+        if self._splits is None:
+            self._splits = kernels.skinny_splits(w.shape[0], K)
+        if self._splits <= 1:
+            return None
+        planes = ctx.scratch(name, (self._splits, M, w.shape[0]), torch.float32)
+        kernels.skinny_gemm_bf16(x, w, planes, splits=self._splits)
+        return planes

@@ -18,6 +18,8 @@ from .base import Norm, StepContext, TensorSpec, register_part
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
+    adds_owed = True
+
     def __init__(self, params):
         super().__init__(params)
         self.dim = int(params["dim"])
@@ -35,5 +37,11 @@ class RMSNorm(Norm):
                 out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
         count = x.shape[0] if rows is None else rows.numel()
         out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
+        owed = ctx.take_owed(x)
+        if owed is not None and rows is None:
+            kernels.add_partials(x, owed, self.weight, self.eps, out)   # x += owed sums; out = norm(x), one pass
+            return out
+        if owed is not None:
+            kernels.add_partials(x, owed)
         kernels.rms_norm(x, self.weight, self.eps, out, rows)
         return out
