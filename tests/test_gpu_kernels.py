@@ -377,10 +377,19 @@ def test_attention_prefill_bf16_mixed_batch(H, KVH, Dh, bs):
     close(out, case["want"], 1e-2, f"prefill attention H={H} KVH={KVH} Dh={Dh} bs={bs}")
 
 
-@pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "far", "last"])
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(8, 2, 128, 16), (2, 2, 64, 8), (6, 3, 32, 4)])
+def test_attention_prefill_bf16_long_portions(H, KVH, Dh, bs):
+    # several key tiles per workgroup, row tiles that end inside a tile, a long cached prefix
+    lens_new, lens_ctx = [300, 130, 64, 33], [300, 1000, 64, 129]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=lens_new, lens_ctx=lens_ctx, seed=24, dtype=torch.bfloat16)
+    out = run_prefill(case, H, KVH, lens_new)
+    close(out, case["want"], 1e-2, f"prefill attention, long portions, H={H} KVH={KVH} Dh={Dh} bs={bs}")
+
+
+@pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "tile_edge_64", "far", "last"])
 def test_attention_prefill_bf16_finds_one_far_key(where):
     spike = {"first": lambda ctx: 0, "page_edge": lambda ctx: 16 * 3 - 1, "tile_edge": lambda ctx: 32 * 7,
-             "far": lambda ctx: ctx - 259, "last": lambda ctx: ctx - 2}[where]
+             "tile_edge_64": lambda ctx: 64 * 5 - 1, "far": lambda ctx: ctx - 259, "last": lambda ctx: ctx - 2}[where]
     lens_new = [40, 7]
     case, S = attention_case(8, 2, 64, 16, lens_new=lens_new, lens_ctx=[700, 523], seed=25, dtype=torch.bfloat16, spike=spike)
     out = run_prefill(case, 8, 2, lens_new)

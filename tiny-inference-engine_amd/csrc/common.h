@@ -22,12 +22,17 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
 }
 
 // Round to nearest even; NaN stays NaN (quieted).
-__device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<bf16_t>(u >> 16);
+// Round to nearest even, NaN stays NaN: gfx950 converts in hardware (v_cvt_pk_bf16_f32).
+typedef __bf16 tie_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float tie_floatx2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const tie_floatx2_t f = {lo, hi};
+  const tie_bf16x2_t b = __builtin_convertvector(f, tie_bf16x2_t);
+  return *reinterpret_cast<const uint32_t*>(&b);
 }
+
+__device__ __forceinline__ bf16_t float_to_bf16(float f) { return static_cast<bf16_t>(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T>
 __device__ __forceinline__ float load_as_float(const T* p);

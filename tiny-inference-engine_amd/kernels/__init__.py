@@ -541,18 +541,17 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
 
 
 def prefill_items(new_tokens, group_size: int) -> "list":
-    """Work items ``(sequence, first 16-row tile)`` of the prefill attention kernel for one step.
+    """Work items ``(sequence, first new row)`` of the prefill attention kernel for one step.
 
-    An item covers 16, 32 or 64 consecutive new rows of a sequence, depending on how many query
-    heads share a KV head (up to four (head, row tile) pairs run side by side in one wave).
+    An item is one workgroup: 32, 64 or 128 consecutive new rows of a sequence, depending on how
+    many query heads share a KV head (four (head, 32-row tile) pairs run side by side).
     """
     heads_at_once = min(group_size, 4)
-    tiles_per_item = max(1, 4 // heads_at_once)
-    rows = 16 * tiles_per_item
+    rows = 32 * (1 if heads_at_once >= 3 else 4 // heads_at_once)
     items = []
     for s, n in enumerate(new_tokens):
-        for j in range(-(-n // rows)):
-            items.append((s, j * tiles_per_item))
+        for first in range(0, n, rows):
+            items.append((s, first))
     return items
 
 

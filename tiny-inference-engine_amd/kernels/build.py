@@ -33,6 +33,10 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
+# Flags of single sources. The prefill attention rescales its output accumulators with ordinary
+# multiplications every few tiles: the matrix instructions then work on vector registers directly.
+SOURCE_FLAGS = {"attention_prefill_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
 
@@ -73,7 +77,7 @@ def library_filename(name: str, source: str, defines: Mapping[str, object]) -> s
         h.update(path.name.encode())
         h.update(path.read_bytes())
     h.update(repr(sorted((k, str(v)) for k, v in defines.items())).encode())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + SOURCE_FLAGS.get(source, [])).encode())
     return f"{name}-{h.hexdigest()[:12]}.so"
 
 
@@ -89,7 +93,8 @@ def compile_library(name: str, source: str, defines: Optional[Mapping[str, objec
     out_dir = _build_dir()
     target = out_dir / filename
     tmp = out_dir / f".{filename}.{os.getpid()}.{threading.get_ident()}.tmp"
-    cmd = [_hipcc(), *FLAGS, *[f"-D{k}={v}" for k, v in sorted(defines.items())], "-I", str(CSRC),
+    cmd = [_hipcc(), *FLAGS, *SOURCE_FLAGS.get(source, []), *[f"-D{k}={v}" for k, v in sorted(defines.items())],
+           "-I", str(CSRC),
            "-o", str(tmp), str(CSRC / source)]
     _log(f"compiling {source} -> {target.name} (hipcc, {ARCH})")
     started = time.time()
