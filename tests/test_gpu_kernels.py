@@ -132,6 +132,17 @@ def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
     assert torch.equal(q2, qkv[:, :H * Dh])
     kernels.qk_norm_rope_kv_write(qkv, q2, None, None, 0.0, inv_freq, i32([0] * T), i32(slots), kc, vc, H, KVH, Dh, bs)
     assert torch.equal(q2, qkv[:, :H * Dh])
+    # cos and sin from the per-step table: the same bits as computing them per head
+    table = torch.empty(T, Dh, device="cuda")
+    kernels.rope_angles(i32(positions), inv_freq, table)
+    angle = torch.tensor(positions, dtype=torch.float32)[:, None] * inv_freq.cpu()[None, :]
+    close(table[:, :Dh // 2], torch.cos(angle.to(F64)), 2e-6, "cos table")
+    kc2, vc2, q4 = torch.zeros_like(kc), torch.zeros_like(vc), torch.empty_like(q)
+    kernels.qk_norm_rope_kv_write(qkv, q4, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc2, vc2, H, KVH, Dh, bs,
+                                  angles=table)
+    kc0, vc0, q0 = torch.zeros_like(kc), torch.zeros_like(vc), torch.empty_like(q)
+    kernels.qk_norm_rope_kv_write(qkv, q0, qw, kw, eps, inv_freq, i32(positions), i32(slots), kc0, vc0, H, KVH, Dh, bs)
+    assert torch.equal(q4, q0) and torch.equal(kc2, kc0) and torch.equal(vc2, vc0)
     # the projection as three planes of partial sums: the same as their sum handed over in one piece
     planes = rnd(3, T, (H + 2 * KVH) * Dh, seed=11).cuda()
     summed = (planes[0] + planes[1]) + planes[2]
@@ -289,7 +300,7 @@ def test_add_partials_alone_and_with_rms_norm(R, n, out_dtype):
 
 @pytest.mark.parametrize("M,N,K", [(65, 70, 96), (100, 384, 200), (128, 128, 64), (300, 200, 4096), (2048, 256, 512),
                                    (257, 129, 72), (1, 64, 64)])
-@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("tile", [1, 2, 3])
 def test_gemm_bf16(M, N, K, tile):
     from tie_amd import kernels
 

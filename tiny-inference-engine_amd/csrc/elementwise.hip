@@ -285,6 +285,7 @@ template <typename TX, typename TQ, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
                                              const float* __restrict__ k_w, float eps,
                                              const float* __restrict__ inv_freq,
+                                             const float* __restrict__ angles,
                                              const int* __restrict__ positions, const int* __restrict__ slots,
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
                                              int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
@@ -348,7 +349,12 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
       b = (b * inv) * w[p + half];
     }
     float o1 = a, o2 = b;
-    if (inv_freq != nullptr) {
+    if (angles != nullptr) {   // cos and sin of this token's angles, computed once for all heads and layers
+      const float cs = angles[static_cast<size_t>(t) * Dh + p];
+      const float sn = angles[static_cast<size_t>(t) * Dh + half + p];
+      o1 = a * cs - b * sn;
+      o2 = b * cs + a * sn;
+    } else if (inv_freq != nullptr) {
       const float angle = pos * inv_freq[p];
       float sn, cs;
       sincosf(angle, &sn, &cs);
@@ -365,9 +371,31 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   }
 }
 
+// angles[t, 0:Dh/2] = cos(float(positions[t]) * inv_freq[i]), angles[t, Dh/2:Dh] = sin of the same: what
+// the kernel below would compute per head and layer, once per step instead.
+__global__ void rope_angles_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                   float* __restrict__ angles, int T, int half) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * half) return;
+  const int t = i / half, p = i % half;
+  float sn, cs;
+  sincosf(static_cast<float>(positions[t]) * inv_freq[p], &sn, &cs);
+  angles[static_cast<size_t>(t) * 2 * half + p] = cs;
+  angles[static_cast<size_t>(t) * 2 * half + half + p] = sn;
+}
+
+extern "C" int tie_rope_angles(const int* positions, const float* inv_freq, float* angles, int T, int half,
+                               hipStream_t stream) {
+  if (T <= 0 || half <= 0) return TIE_BAD_ARGUMENT;
+  const long n = static_cast<long>(T) * half;
+  rope_angles_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, stream>>>(positions, inv_freq, angles, T, half);
+  return tie_launch_status();
+}
+
+// angles (optional): the table of tie_rope_angles for these positions; then inv_freq is not read.
 extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int q_dtype,
                                          const float* q_w, const float* k_w, float eps, const float* inv_freq,
-                                         const int* positions, const int* slots, void* k_cache, void* v_cache,
+                                         const float* angles, const int* positions, const int* slots, void* k_cache, void* v_cache,
                                          int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
                                          long plane_stride, int planes, hipStream_t stream) {
@@ -382,7 +410,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   const dim3 grid(heads, T);
 #define LAUNCH(TX, TQ, TC)                                                                                   \
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
-      static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, positions, slots,       \
+      static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
       block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);

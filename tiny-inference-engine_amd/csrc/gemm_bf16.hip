@@ -14,8 +14,8 @@
 // so any M, N >= 1 and any K with K % 8 == 0 are taken. The accumulation order over k is fixed by
 // the tile shape alone, so a row's result does not depend on the other rows of the call.
 //
-// The product is bound by the L2: every workgroup re-reads its operand tiles from there, so the
-// 256 x 256 tile (half the bytes per flop of 128 x 128) is used wherever it still fills the GPU.
+// Every workgroup re-reads its operand tiles from the L2, so the 256 x 256 tile (half the bytes per
+// flop of 128 x 128) is used wherever it still fills the GPU, and 256 x 128 where only that does.
 //
 // Workgroups are numbered so that each of the 8 XCDs (which have an L2 each) works on a
 // contiguous band of the output and walks it column-tile by column-tile: the weights of a column
@@ -231,7 +231,8 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
 
 // out_dtype: TIE_F32 or TIE_BF16; accumulate adds into a float32 output; gated (bfloat16 output of N / 2
 // columns, N % 16 == 0) applies silu(gate) * up to interleaved column blocks.
-// tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64).
+// tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
+//       3 = 256x128 (eight waves of 64x64).
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
                              int N, int K, int tile, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0) return TIE_BAD_ARGUMENT;
@@ -240,11 +241,13 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   if (gated && (accumulate || out_dtype != TIE_BF16 || N % 16 != 0)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
   if (tile == 0) {
-    // The product is bound by re-reading operand tiles from L2: a 256x256 tile needs half the bytes
-    // per flop of a 128x128 one. Take it once it gives most CUs a tile.
-    const long t256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
-    tile = t256 >= 160 ? 2 : 1;
+    // Larger tiles need fewer operand bytes per flop; take the largest that still gives most CUs a tile.
+    const long rows256 = (M + 255) / 256;
+    if (rows256 * ((N + 255) / 256) >= 160) tile = 2;
+    else if (rows256 * ((N + 127) / 128) >= 192) tile = 3;
+    else tile = 1;
   }
   if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, stream);
+  if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, stream);
   return launch_gemm<128, 128, 64, 2, 2>(x, w, out, epi, M, N, K, stream);
 }

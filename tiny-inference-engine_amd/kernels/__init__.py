@@ -43,7 +43,8 @@ _SIGNATURES = {
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
-        "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void,
+        "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_void],
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
@@ -331,7 +332,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
               gated: bool = False) -> None:
     """out (+)= x @ w.T for bfloat16 operands on the matrix cores, any number of rows; K % 8 == 0.
 
-    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256; 0 lets the kernel choose);
+    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256, 3 = 256x128; 0 lets the kernel choose);
     ``gated`` as in ``skinny_gemm_bf16``.
     """
     M, N, K = _bf16_product_operands(x, w, out, gated, "gemm_bf16")
@@ -369,13 +370,27 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool
         gemm_generic(x, w, out, accumulate)
 
 
+def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = [cos(float(positions[t]) * inv_freq), sin(...)]: the rotation table of one step, ``[T, 2 * half]`` float32."""
+    T = positions.numel()
+    half = inv_freq.numel()
+    _i32(positions, "positions", T)
+    _f32(inv_freq, "inv_freq", (half,))
+    _f32(out, "rope angles", (T, 2 * half))
+    _check(_lib("elementwise").tie_rope_angles(positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), T, half,
+                                               _stream()), "rope_angles")
+
+
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
                           k_weight: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
                           positions: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                           v_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
                           block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
-                          planes: int = 1, plane_stride: int = 0) -> None:
+                          planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None) -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
+
+    ``angles`` (from ``rope_angles`` for the same positions and ``inv_freq``) spares the kernel the
+    sines and cosines.
 
     With ``planes`` > 1, ``qkv`` is the first of that many planes of partial sums, ``plane_stride``
     elements apart, which are added as they are read.
@@ -404,6 +419,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
             _f32(wt, nm, (Dh,))
     if inv_freq is not None:
         _f32(inv_freq, "inv_freq", (Dh // 2,))
+    if angles is not None:
+        _f32(angles, "rope angles", (T, Dh))
     _i32(positions, "positions", T)
     cache_code = _code(q_out, "q output")
     k_row = 0
@@ -422,7 +439,8 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         cache_code = _code(k_cache, "k cache")
     _check(_lib("elementwise").tie_qk_norm_rope_kv_write(
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
-        _ptr(k_weight), float(eps), _ptr(inv_freq), positions.data_ptr(), _ptr(slots) if write_kv else None,
+        _ptr(k_weight), float(eps), _ptr(inv_freq), _ptr(angles), positions.data_ptr(),
+        _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
         _stream()), "qk_norm_rope_kv_write")

@@ -92,7 +92,8 @@ class PagedAttention(Mixer):
             kernels.qk_norm_rope_kv_write(
                 qkv, q, self.q_norm_weight, self.k_norm_weight, eps, inv_freq, ctx.batch.positions,
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
-                write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width)
+                write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
+                angles=self.position.angles(ctx))
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.

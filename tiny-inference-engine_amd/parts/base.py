@@ -235,6 +235,10 @@ class Position(Part):
     def rotary_table(self):
         return None
 
+    def angles(self, ctx: "StepContext") -> Optional[torch.Tensor]:
+        """Optional: ``[T, rotary_dim]`` float32 cos | sin of this step's positions, for the fused kernel."""
+        return None
+
     def apply(self, ctx: StepContext, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
         raise NotImplementedError
 

@@ -12,6 +12,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from .. import kernels
 from ..errors import InvalidArgument
 from .base import Position, register_part
 
@@ -38,6 +39,17 @@ class RopeNeox(Position):
 
     def rotary_table(self):
         return self.inv_freq, self.head_dim, "rotate_half"
+
+    def angles(self, ctx) -> torch.Tensor:
+        """cos | sin of this step's positions, ``[T, head_dim]`` float32: computed once a step, shared by all layers."""
+        key = ("rope_angles", self.head_dim, self.theta)
+        table = ctx.notes.get(key)
+        if table is None:
+            table = ctx.scratch(f"rope.angles:{self.head_dim}:{self.theta}", (ctx.num_tokens, self.head_dim),
+                                torch.float32)
+            kernels.rope_angles(ctx.batch.positions, self.inv_freq, table)
+            ctx.notes[key] = table
+        return table
 
 
 @register_part("position", "none")
