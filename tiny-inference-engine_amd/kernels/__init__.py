@@ -85,7 +85,7 @@ _SIGNATURES = {
 _libs = {}
 
 
-def library_list(head_dims=(16, 32, 48, 64, 80, 128, 256)):
+def library_list(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 256)):
     """``(name, source, defines)`` of every library, for building them all up front.
 
     The per-head-size libraries are listed for ``head_dims``; any other head size is compiled the
