@@ -9,14 +9,15 @@
 //                                          B = Q (held in registers)          2 x HEAD_DIM/32 MFMAs
 //   online softmax per column g in float32: running maximum, sum, rescale of the accumulator
 //   O^T[d, g]  += V^T[d, key] . P^T[key, g]   A = V^T rows (the cache keeps values transposed inside a
-//                                          page, so 4 positions of one dimension are 8 bytes),
+//                                          page, so 8 positions of one dimension are 16 bytes),
 //                                          B = P, which is exactly what the lane already holds
 //                                          from the first product              HEAD_DIM/16 MFMAs
 //
 // Nothing passes through LDS and no lane ever needs another lane's scores. Splits of the keys
 // run as separate waves; a second kernel merges their (maximum, sum, accumulator) triples in a
 // fixed order. Keys are always cut at multiples of 32 positions, so what is computed for a
-// position does not depend on the batch around it.
+// position does not depend on the batch around it. Block-table lookups run two tiles ahead of the
+// arithmetic and the data loads one tile ahead, so neither waits for the other.
 //
 // Formula: src/backend/cpu/cpu_backend.cpp:261-319 (score = scale * q.k, causal by position,
 // online softmax, query head h reads KV head h / (H / KVH)).
@@ -36,19 +37,22 @@ constexpr int DH = HEAD_DIM;
 constexpr int KSTEPS = (DH + 31) / 32;  // k blocks of the first product
 constexpr int DTILES = DH / 16;         // row tiles of the second product
 
-union Frag {
-  bf16x8_t v;
-  uint4 u4;
-  uint2 u2[2];
-  bf16_t h[8];
-};
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));   // native vectors: fragments stay in registers
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
+__device__ __forceinline__ bf16x8_t frag(u32x4_t v) { return *reinterpret_cast<const bf16x8_t*>(&v); }
+
+// Keys of a 32-key tile are taken in runs of 8: row r of 16-key sub-tile u is key (r / 4) * 8 + u * 4 + r % 4
+// of the tile. The scores a lane then holds (rows quad * 4 + v of both sub-tiles) are those of the 8
+// consecutive keys quad * 8 .. + 7, which is also how the values of one dimension lie in a page: with
+// WIDE (block sizes in steps of 8) a lane reads them in one 16-byte piece.
+template <bool WIDE>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int max_blocks, float scale, int window, int nsplit) {
+    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit) {
   const int lane = threadIdx.x;
   const int col = lane & 15;   // query head within the group (column of every tile)
   const int quad = lane >> 4;  // 0..3
@@ -69,14 +73,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   const int tile_end = min(num_tiles, tile_begin + per_split);
 
   // Q as the B operand: lane (col = g, quad) holds Q[g][step*32 + quad*8 .. +8].
-  Frag qf[KSTEPS];
+  u32x4_t qf[KSTEPS];
   {
     const bool valid = col < G;
     const bf16_t* qr = q + (static_cast<size_t>(t) * H + static_cast<size_t>(kvh) * G + (valid ? col : 0)) * DH;
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
       const int d = st * 32 + quad * 8;
-      qf[st].u4 = (valid && d < DH) ? *reinterpret_cast<const uint4*>(qr + d) : make_uint4(0, 0, 0, 0);
+      qf[st] = (valid && d < DH) ? *reinterpret_cast<const u32x4_t*>(qr + d) : u32x4_t{0, 0, 0, 0};
     }
   }
 
@@ -87,43 +91,65 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 
   const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;   // elements of one page, K or V
   const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
+  // Positions are clamped into [start, pos] for addresses only (pages outside that range may be gone or
+  // never have been there); what lies outside is masked in the softmax.
+  auto page_of = [&](int kp) { return block_shift >= 0 ? kp >> block_shift : kp / block_size; };
+  auto offset_of = [&](int kp) { return block_shift >= 0 ? kp & (block_size - 1) : kp % block_size; };
+  // This lane's keys of a tile: rows of the two sub-tiles, and the runs of values it reads.
+  const int krow0 = (col >> 2) * 8 + (col & 3);        // sub-tile 1: + 4
+  constexpr int VG = WIDE ? 8 : 4;
 
-  // Fragments of one 32-key tile: keys for the first product (two 16-key sub-tiles), values for the second.
-  // Positions are clamped to pos for the address only; what lies beyond pos is masked in the softmax.
-  auto load_keys = [&](int base, Frag (&kf)[2][KSTEPS]) {
+  // Pages first, one tile further ahead than the data, so that no data load waits for a lookup.
+  struct Pages { int k[2]; int v[WIDE ? 1 : 2]; };
+  auto lookup = [&](int base, Pages& pg) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) pg.k[u] = table[page_of(min(max(base + krow0 + u * 4, start), pos))];
+#pragma unroll
+    for (int j = 0; j < (WIDE ? 1 : 2); ++j)
+      pg.v[j] = table[page_of(min(max(base + quad * 8 + j * 4, start / VG * VG), pos / VG * VG))];
+  };
+  auto load_keys = [&](int base, const Pages& pg, u32x4_t (&kf)[2][KSTEPS]) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int kp = min(base + u * 16 + col, pos);
-      const bf16_t* kr = k_cache + static_cast<size_t>(table[kp / block_size]) * page_stride + head_off +
-                         static_cast<size_t>(kp % block_size) * DH;
+      const int kp = min(max(base + krow0 + u * 4, start), pos);
+      const bf16_t* kr = k_cache + static_cast<size_t>(pg.k[u]) * page_stride + head_off +
+                         static_cast<size_t>(offset_of(kp)) * DH;
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st) {
         const int d = st * 32 + quad * 8;
-        kf[u][st].u4 = d < DH ? *reinterpret_cast<const uint4*>(kr + d) : make_uint4(0, 0, 0, 0);
+        kf[u][st] = d < DH ? *reinterpret_cast<const u32x4_t*>(kr + d) : u32x4_t{0, 0, 0, 0};
       }
     }
   };
-  auto load_values = [&](int base, Frag (&vf)[DTILES]) {
-    const int k0 = min(base + quad * 4, pos);               // a run of 4 positions inside one page
-    const int k1 = min(base + 16 + quad * 4, pos);
-    const bf16_t* v0 = v_cache + static_cast<size_t>(table[k0 / block_size]) * page_stride + head_off +
-                       (k0 % block_size) / 4 * 4;
-    const bf16_t* v1 = v_cache + static_cast<size_t>(table[k1 / block_size]) * page_stride + head_off +
-                       (k1 % block_size) / 4 * 4;
+  auto load_values = [&](int base, const Pages& pg, u32x4_t (&vf)[DTILES]) {
+    const bf16_t* vp[WIDE ? 1 : 2];
+#pragma unroll
+    for (int j = 0; j < (WIDE ? 1 : 2); ++j) {
+      const int kp = min(max(base + quad * 8 + j * 4, start / VG * VG), pos / VG * VG);
+      vp[j] = v_cache + static_cast<size_t>(pg.v[j]) * page_stride + head_off + offset_of(kp);
+    }
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
       const size_t d_off = static_cast<size_t>(dt * 16 + col) * block_size;
-      vf[dt].u2[0] = *reinterpret_cast<const uint2*>(v0 + d_off);
-      vf[dt].u2[1] = *reinterpret_cast<const uint2*>(v1 + d_off);
+      if (WIDE) {
+        vf[dt] = *reinterpret_cast<const u32x4_t*>(vp[0] + d_off);
+      } else {
+        const u32x2_t h0 = *reinterpret_cast<const u32x2_t*>(vp[0] + d_off);
+        const u32x2_t h1 = *reinterpret_cast<const u32x2_t*>(vp[WIDE ? 0 : 1] + d_off);
+        vf[dt] = u32x4_t{h0.x, h0.y, h1.x, h1.y};
+      }
     }
   };
 
   // The loads of tile t + 1 are issued before the arithmetic of tile t, so memory latency and the
-  // matrix cores overlap.
-  Frag kf[2][KSTEPS], vf[DTILES], kf_next[2][KSTEPS], vf_next[DTILES];
+  // matrix cores overlap; the pages of tile t + 2 are looked up at the same time.
+  u32x4_t kf[2][KSTEPS], vf[DTILES], kf_next[2][KSTEPS], vf_next[DTILES];
+  Pages pages;
   if (tile_begin < tile_end) {
-    load_keys(tile_begin * 32, kf_next);
-    load_values(tile_begin * 32, vf_next);
+    lookup(tile_begin * 32, pages);
+    load_keys(tile_begin * 32, pages, kf_next);
+    load_values(tile_begin * 32, pages, vf_next);
+    if (tile_begin + 1 < tile_end) lookup(tile_begin * 32 + 32, pages);
   }
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const int base = tile * 32;
@@ -134,41 +160,47 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) vf[dt] = vf_next[dt];
     if (tile + 1 < tile_end) {
-      load_keys(base + 32, kf_next);
-      load_values(base + 32, vf_next);
+      load_keys(base + 32, pages, kf_next);
+      load_values(base + 32, pages, vf_next);
+      if (tile + 2 < tile_end) lookup(base + 64, pages);
     }
-    // ---- first product: two 16-key tiles
+    // ---- first product: two 16-key sub-tiles
     floatx4 sc[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       sc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st)
-        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][st].v, qf[st].v, sc[u], 0, 0, 0);
+        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(kf[u][st]), frag(qf[st]), sc[u], 0, 0, 0);
     }
-    // ---- softmax of this lane's column over its 8 keys, then across the four quads
+    // ---- softmax of this lane's column over its 8 keys (quad * 8 + u * 4 + v), then across the four quads.
+    // Scores stay unscaled; scale * log2(e) > 0 enters in the exponent: p = 2^(s c - m c).
     float sv[8];
     float tile_max = -INFINITY;
+    const bool whole = base >= start && base + 31 <= pos;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int kp = base + u * 16 + quad * 4 + v;
-        const float x = (kp <= pos && kp >= start) ? sc[u][v] * scale : -INFINITY;
+        const int kp = base + quad * 8 + u * 4 + v;
+        const float x = (whole || (kp <= pos && kp >= start)) ? sc[u][v] : -INFINITY;
         sv[u * 4 + v] = x;
         tile_max = fmaxf(tile_max, x);
       }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, TIE_WAVE));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, TIE_WAVE));
     const float m_new = fmaxf(m, tile_max);
-    const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
-    Frag pf;
+    const float neg_mc = (m_new == -INFINITY) ? 0.f : -m_new * scale_log2e;
+    const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
+    u32x4_t pf;
     float psum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float p = (sv[i] == -INFINITY) ? 0.f : expf(sv[i] - m_new);
-      psum += p;
-      pf.h[i] = float_to_bf16(p);
+    for (int i = 0; i < 8; i += 2) {
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, neg_mc));       // masked: 0
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(sv[i + 1], scale_log2e, neg_mc));
+      psum += p0;
+      psum += p1;
+      pf[i / 2] = pack_bf16x2(p0, p1);
     }
     l = l * corr + psum;
     m = m_new;
@@ -177,7 +209,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     for (int dt = 0; dt < DTILES; ++dt) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[dt][v] *= corr;
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc[dt], 0, 0, 0);
+      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(vf[dt]), frag(pf), acc[dt], 0, 0, 0);
     }
   }
 
@@ -191,8 +223,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     const float inv = 1.0f / l;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) o[dt * 16 + quad * 4 + v] = float_to_bf16(acc[dt][v] * inv);
+      *reinterpret_cast<u32x2_t*>(o + dt * 16 + quad * 4) =
+          u32x2_t{pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv), pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv)};
     return;
   }
   const size_t slot = (static_cast<size_t>(blockIdx.z) * H + h) * nsplit + split;
@@ -201,13 +233,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   for (int dt = 0; dt < DTILES; ++dt)
     *reinterpret_cast<float4*>(po + dt * 16 + quad * 4) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
   if (quad == 0) {
-    part_ml[slot * 2] = m;
+    part_ml[slot * 2] = m * scale_log2e;     // the merge works in the exponent's units (base 2)
     part_ml[slot * 2 + 1] = l;
   }
 }
 
-// Merges the splits of one (sequence, query head): m = max m_i, L = sum l_i e^(m_i - m),
-// out = sum o_i e^(m_i - m) / L, splits in ascending order. The weights e^(m_i - m) are computed
+// Merges the splits of one (sequence, query head): m = max m_i, L = sum l_i 2^(m_i - m),
+// out = sum o_i 2^(m_i - m) / L, splits in ascending order (the maxima come scaled by
+// scale * log2(e), the units of the exponent). The weights 2^(m_i - m) are computed
 // once by the first threads and shared through LDS.
 #define MERGE_MAX_SPLITS 256
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -225,7 +258,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
   const float mi = i < nsplit ? part_ml[(slot0 + i) * 2] : -INFINITY;
   const float li = i < nsplit ? part_ml[(slot0 + i) * 2 + 1] : 0.f;
   const float m = block_max(mi, scratch);
-  const float wi = (mi == -INFINITY) ? 0.f : expf(mi - m);
+  const float wi = (mi == -INFINITY) ? 0.f : exp2f(mi - m);
   if (i < nsplit) {
     weight[i] = wi;
     weighted_sum[i] = wi * li;
@@ -249,14 +282,20 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
                                          int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
                                          int window, int nsplit, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
-      block_size <= 0 || block_size % 4 != 0 || max_blocks <= 0 || nsplit <= 0 || nsplit > MERGE_MAX_SPLITS)
+      block_size <= 0 || block_size % 4 != 0 || max_blocks <= 0 || nsplit <= 0 || nsplit > MERGE_MAX_SPLITS ||
+      !(scale > 0.f))   // the running maximum is kept on unscaled scores
     return TIE_BAD_ARGUMENT;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr)) return TIE_BAD_ARGUMENT;
   const dim3 grid(nsplit, KVH, num_seqs);
-  attention_decode_kernel<<<grid, TIE_WAVE, 0, stream>>>(
-      static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-      static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH,
-      block_size, max_blocks, scale, window, nsplit);
+  const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  const float scale_log2e = scale * 1.44269504088896340736f;
+#define LAUNCH(WIDE)                                                                                            \
+  attention_decode_kernel<WIDE><<<grid, TIE_WAVE, 0, stream>>>(                                                  \
+      static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),  \
+      static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH,     \
+      block_size, block_shift, max_blocks, scale_log2e, window, nsplit)
+  if (block_size % 8 == 0) LAUNCH(true); else LAUNCH(false);
+#undef LAUNCH
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
   const int merge_threads = (nsplit > DH ? nsplit : DH) <= 64 ? 64 : ((nsplit > DH ? nsplit : DH) <= 128 ? 128 : 256);

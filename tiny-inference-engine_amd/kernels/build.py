@@ -33,9 +33,10 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
-# Flags of single sources. The prefill attention rescales its output accumulators with ordinary
-# multiplications every few tiles: the matrix instructions then work on vector registers directly.
-SOURCE_FLAGS = {"attention_prefill_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+# Flags of single sources. The attention kernels rescale their output accumulators with ordinary
+# multiplications between matrix instructions: these then work on vector registers directly.
+SOURCE_FLAGS = {"attention_prefill_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+                "attention_decode_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
