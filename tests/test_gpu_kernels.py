@@ -426,6 +426,9 @@ def test_argmax_and_sample_kernels():
     out = torch.empty(4, dtype=torch.int32, device="cuda")
     kernels.argmax_rows(logits, out)
     assert out.tolist() == [int(torch.argmax(logits[0])), 30, -1, int(torch.argmax(logits[3]))]
+    top = torch.empty(4, device="cuda")
+    kernels.argmax_rows(logits, out, top)                     # the maximum itself comes along on request
+    assert out.tolist()[1] == 30 and float(top[1]) == 50.0 and float(top[0]) == float(logits[0].max())
     # frequencies of log {0.7, 0.2, 0.1} at temperature 1 (the reference's sampler test), many rows at once
     R = 4000
     rows = torch.log(torch.tensor([0.7, 0.2, 0.1])).repeat(R, 1).cuda()

@@ -481,7 +481,7 @@ __global__ void argmax_partial_kernel(const float* __restrict__ logits, float* _
 }
 
 __global__ void argmax_final_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i,
-                                    int* __restrict__ out) {
+                                    int* __restrict__ out, float* __restrict__ max_out) {
   const int r = blockIdx.x;
   float bv = part_v[r * ARGMAX_CHUNKS + threadIdx.x];
   int bi = part_i[r * ARGMAX_CHUNKS + threadIdx.x];
@@ -494,18 +494,21 @@ __global__ void argmax_final_kernel(const float* __restrict__ part_v, const int*
       bi = oi;
     }
   }
-  if (threadIdx.x == 0) out[r] = bi;
+  if (threadIdx.x == 0) {
+    out[r] = bi;
+    if (max_out != nullptr) max_out[r] = bv;
+  }
 }
 
-// part_v / part_i: workspace of R * 64 floats / ints.
-extern "C" int tie_argmax(const float* logits, int* out, float* part_v, int* part_i, int R, int V,
+// part_v / part_i: workspace of R * 64 floats / ints. max_out (optional): the maximum itself, per row.
+extern "C" int tie_argmax(const float* logits, int* out, float* max_out, float* part_v, int* part_i, int R, int V,
                           hipStream_t stream) {
   if (R <= 0 || R > 65535 || V <= 0 || part_v == nullptr || part_i == nullptr) return TIE_BAD_ARGUMENT;
   static_assert(ARGMAX_CHUNKS == TIE_WAVE, "the final stage is one wave per row");
   argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, R), 256, 0, stream>>>(logits, part_v, part_i, V);
   int status = tie_launch_status();
   if (status != TIE_OK) return status;
-  argmax_final_kernel<<<R, TIE_WAVE, 0, stream>>>(part_v, part_i, out);
+  argmax_final_kernel<<<R, TIE_WAVE, 0, stream>>>(part_v, part_i, out, max_out);
   return tie_launch_status();
 }
 

@@ -182,10 +182,7 @@ class Engine:
                     sampled.append(seq)
                 entries.append(StepEntry(seq.cache, begin, seq.tokens[begin:end], want))
             started = time.perf_counter()
-            logits = self.runner.step(entries)
-            if logits is not None:
-                torch.cuda.synchronize() if logits.is_cuda else None
-            self._stats.step_seconds += time.perf_counter() - started
+            logits = self.runner.step(entries)      # queued on the GPU; sampling below is queued right behind it
             self._stats.steps += 1
             self._stats.seqs_scheduled += len(batch.seqs)
             self._stats.prefill_tokens += prefill_tokens
@@ -202,6 +199,7 @@ class Engine:
             self.cache.trim(s.seq.cache, s.seq.num_computed)
         self.scheduler.complete(batch)
         if not sampled:
+            self._stats.step_seconds += time.perf_counter() - started
             return
 
         try:
@@ -211,6 +209,7 @@ class Engine:
                 if seq.state != SeqState.FINISHED:
                     self._finish(seq, FinishReason.ERROR)
             raise
+        self._stats.step_seconds += time.perf_counter() - started   # reading the tokens waited for the GPU
         for i, seq in enumerate(sampled):
             if seq.state == SeqState.FINISHED:      # cancelled by an earlier token callback of this step
                 continue

@@ -49,7 +49,7 @@ _SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_void],
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
                                       _c_int, _c_void],
-        "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
@@ -484,19 +484,21 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 _argmax_workspace = {}
 
 
-def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
-    """out[r] = lowest index of the maximum of logits[r]; -1 marks a row with a NaN."""
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor, max_out: Optional[torch.Tensor] = None) -> None:
+    """out[r] = lowest index of the maximum of logits[r]; -1 marks a row with a NaN. ``max_out[r]`` = that maximum."""
     _f32(logits, "logits")
     R, V = logits.shape
     _i32(out, "argmax output", R)
+    if max_out is not None:
+        _f32(max_out, "row maxima", (R,))
     key = str(logits.device)
     ws = _argmax_workspace.get(key)
     if ws is None or ws[0].numel() < R * 64:
         rows = max(R, 64)
         ws = _argmax_workspace[key] = (torch.empty(rows * 64, dtype=torch.float32, device=logits.device),
                                        torch.empty(rows * 64, dtype=torch.int32, device=logits.device))
-    _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), ws[0].data_ptr(), ws[1].data_ptr(), R, V,
-                                          _stream()), "argmax")
+    _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), _ptr(max_out), ws[0].data_ptr(),
+                                          ws[1].data_ptr(), R, V, _stream()), "argmax")
 
 
 def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,

@@ -92,11 +92,12 @@ class DeviceSampler:
         # Kernels work on all rows at once; each kind's result is read where it applies.
         host_argmax = host_max = None
         if greedy_rows or plain_rows:
-            argmax = torch.empty(R, dtype=torch.int32, device=logits.device)
-            kernels.argmax_rows(logits, argmax)
-            top = logits.gather(1, argmax.clamp(min=0).long().unsqueeze(1)).squeeze(1)
-            host_argmax = argmax.cpu().numpy()
-            host_max = top.cpu().numpy()
+            # index and maximum side by side in one buffer: one copy to the host, one wait for the GPU
+            both = torch.empty(2 * R, dtype=torch.int32, device=logits.device)
+            kernels.argmax_rows(logits, both[:R], both[R:].view(torch.float32))
+            host = both.cpu().numpy()
+            host_argmax = host[:R]
+            host_max = host[R:].view(np.float32)
             for i in greedy_rows + plain_rows:
                 if host_argmax[i] < 0:
                     raise InvalidArgument(f"a logit of row {i} is NaN")
