@@ -32,8 +32,11 @@ __device__ __forceinline__ bf16x8_t frag_of(uint4 v) { return *reinterpret_cast<
 
 // Loads the 16-byte chunks of a (ROWS x BK) slice that this thread stages: chunk c of row r for
 // (r, c) = (t / CPR + RPP i, t % CPR) with CPR = BK / 8 chunks a row and RPP = THREADS / CPR rows a
-// pass. Rows >= limit and k >= K give zeros.
-template <int ROWS, int BK, int THREADS>
+// pass. Rows >= limit and k >= K give zeros. With FULL the slice lies wholly below K and rows beyond
+// the limit are clamped to the last one instead (their products land in outputs that are never
+// stored): the loads then sit in straight-line code, which lets the compiler count the loads in
+// flight exactly instead of waiting for all of them wherever branches meet.
+template <int ROWS, int BK, int THREADS, bool FULL>
 __device__ __forceinline__ void load_slice(const bf16_t* __restrict__ base, int row0, int limit, int K, int k0,
                                            uint4 (&regs)[ROWS * (BK / 8) / THREADS]) {
   constexpr int CPR = BK / 8, RPP = THREADS / CPR;
@@ -43,8 +46,11 @@ __device__ __forceinline__ void load_slice(const bf16_t* __restrict__ base, int 
 #pragma unroll
   for (int i = 0; i < ROWS / RPP; ++i) {
     const int row = row0 + r + RPP * i;
-    regs[i] = (row < limit && k < K) ? *reinterpret_cast<const uint4*>(base + static_cast<size_t>(row) * K + k)
-                                     : make_uint4(0, 0, 0, 0);
+    if (FULL)
+      regs[i] = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(min(row, limit - 1)) * K + k);
+    else
+      regs[i] = (row < limit && k < K) ? *reinterpret_cast<const uint4*>(base + static_cast<size_t>(row) * K + k)
+                                       : make_uint4(0, 0, 0, 0);
   }
 }
 
@@ -106,15 +112,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
   // LDS and the loads of slice kt + 2 are in flight into the other.
   uint4 ra[2][BM * (BK / 8) / THREADS], rb[2][BN * (BK / 8) / THREADS];
   const int k_tiles = (K + GB_BK - 1) / GB_BK;
-  load_slice<BM, BK, THREADS>(x, row0, M, K, 0, ra[0]);
-  load_slice<BN, BK, THREADS>(w, col0, N, K, 0, rb[0]);
-  if (k_tiles > 1) {
-    load_slice<BM, BK, THREADS>(x, row0, M, K, GB_BK, ra[1]);
-    load_slice<BN, BK, THREADS>(w, col0, N, K, GB_BK, rb[1]);
-  }
+  const int k_full = K / GB_BK;   // slices that lie wholly below K
+  load_slice<BM, BK, THREADS, false>(x, row0, M, K, 0, ra[0]);
+  load_slice<BN, BK, THREADS, false>(w, col0, N, K, 0, rb[0]);
   store_slice<BM, BK, THREADS>(lds, ra[0]);
   store_slice<BN, BK, THREADS>(lds + BM * GB_STRIDE, rb[0]);
   __syncthreads();
+  // Slice 1 is in flight when the loop is entered, as it is whenever the loop comes round.
+  if (k_full > 1) {
+    load_slice<BM, BK, THREADS, true>(x, row0, M, K, GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, K, GB_BK, rb[1]);
+  } else if (k_tiles > 1) {
+    load_slice<BM, BK, THREADS, false>(x, row0, M, K, GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, false>(w, col0, N, K, GB_BK, rb[1]);
+  }
 
   // Fragments of k step s + 1 are read from LDS before the MFMAs of step s are issued, so the
   // matrix cores do not idle through the LDS latency.
@@ -147,12 +158,39 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
     }
   };
 
-  // Unrolled by two so that the register sets are addressed statically.
-  for (int kt = 0; kt < k_tiles; kt += 2) {
+  // Unrolled by two so that the register sets are addressed statically. The steady state runs while
+  // the two slices it fetches lie wholly below K: its body has no branches, so the compiler knows
+  // how many loads are in flight at every point and lets slice kt + 2 stay in flight while slice
+  // kt + 1 is written to LDS. The last slices go through the general code below.
+  int kt = 0;
+  auto steady_pair = [&](int k) {
+    load_slice<BM, BK, THREADS, true>(x, row0, M, K, (k + 2) * GB_BK, ra[0]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, K, (k + 2) * GB_BK, rb[0]);
+    compute(lds);
+    store_slice<BM, BK, THREADS>(lds + BUF, ra[1]);
+    store_slice<BN, BK, THREADS>(lds + BUF + BM * GB_STRIDE, rb[1]);
+    __syncthreads();
+    load_slice<BM, BK, THREADS, true>(x, row0, M, K, (k + 3) * GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, K, (k + 3) * GB_BK, rb[1]);
+    compute(lds + BUF);
+    store_slice<BM, BK, THREADS>(lds, ra[0]);
+    store_slice<BN, BK, THREADS>(lds + BM * GB_STRIDE, rb[0]);
+    __syncthreads();
+  };
+  // The compiler counts loads in flight exactly only within straight-line code: where the loop comes
+  // round it waits for all of them. Four pairs a round keep that to one slice in eight.
+  for (; kt + 9 < k_full; kt += 8) {
+    steady_pair(kt);
+    steady_pair(kt + 2);
+    steady_pair(kt + 4);
+    steady_pair(kt + 6);
+  }
+  for (; kt + 3 < k_full; kt += 2) steady_pair(kt);
+  for (; kt < k_tiles; kt += 2) {
     {  // even slice: in LDS buffer 0; slice kt + 1 sits in set 1; fetch kt + 2 into set 0
       if (kt + 2 < k_tiles) {
-        load_slice<BM, BK, THREADS>(x, row0, M, K, (kt + 2) * GB_BK, ra[0]);
-        load_slice<BN, BK, THREADS>(w, col0, N, K, (kt + 2) * GB_BK, rb[0]);
+        load_slice<BM, BK, THREADS, false>(x, row0, M, K, (kt + 2) * GB_BK, ra[0]);
+        load_slice<BN, BK, THREADS, false>(w, col0, N, K, (kt + 2) * GB_BK, rb[0]);
       }
       compute(lds);
       if (kt + 1 < k_tiles) {
@@ -163,8 +201,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
     }
     if (kt + 1 < k_tiles) {  // odd slice: in LDS buffer 1; slice kt + 2 sits in set 0; fetch kt + 3 into set 1
       if (kt + 3 < k_tiles) {
-        load_slice<BM, BK, THREADS>(x, row0, M, K, (kt + 3) * GB_BK, ra[1]);
-        load_slice<BN, BK, THREADS>(w, col0, N, K, (kt + 3) * GB_BK, rb[1]);
+        load_slice<BM, BK, THREADS, false>(x, row0, M, K, (kt + 3) * GB_BK, ra[1]);
+        load_slice<BN, BK, THREADS, false>(w, col0, N, K, (kt + 3) * GB_BK, rb[1]);
       }
       compute(lds + BUF);
       if (kt + 2 < k_tiles) {
