@@ -323,6 +323,20 @@ def test_gemm_bf16(M, N, K, tile):
     assert torch.equal(few, out[:3])
 
 
+@pytest.mark.parametrize("M,N,K,splits", [(65, 70, 1024, 2), (100, 384, 4096, 8), (300, 200, 1536, 3), (128, 128, 520, 2)])
+def test_gemm_bf16_in_planes(M, N, K, splits):
+    """K cut into ranges: one plane of partial sums a range, which add up to the product."""
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=34, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=35, scale=0.1, dtype=torch.bfloat16).cuda()
+    planes = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device="cuda")
+    kernels.gemm_bf16(x, w, planes, splits=splits)
+    close(planes.cpu().to(F64).sum(0), plain.linear(x.cpu(), w.cpu()), 1e-5, f"gemm {M}x{N}x{K} in {splits} planes")
+    assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(512, 4096, 4096) == 2
+    assert kernels.gemm_splits(2048, 4096, 4096) == 1 and kernels.gemm_splits(128, 4096, 256) == 1
+
+
 def run_decode(case, S, H, Dh, nsplit, window=None):
     from tie_amd import kernels
 

@@ -89,6 +89,44 @@ def test_norm_embedding_feed_forward_and_head_parts_alone():
         assert names == ({"h": False, "n": False} if tied is None else {"e": False, "h": True, "n": False})
 
 
+@pytest.mark.parametrize("T", [5, 64, 100, 300])
+def test_sums_a_product_leaves_owed_reach_the_stream_through_the_norm_or_settle(T):
+    """bfloat16, a long K: the down projection comes as planes of partial sums (decode product up to 64
+    rows, tiled product above) that the next norm adds - or ``settle`` does, for parts that know nothing of it."""
+    from tie_amd.parts import PartSpec, build_part
+
+    g = torch.Generator().manual_seed(3)
+    D, I = 256, 1024
+    w = {"n": 1 + 0.1 * torch.randn(D, generator=g), "g": torch.randn(I, D, generator=g) * 0.05,
+         "u": torch.randn(I, D, generator=g) * 0.05, "d": torch.randn(D, I, generator=g) * 0.05}
+    w = {k: (v.to(torch.bfloat16) if k != "n" else v) for k, v in w.items()}
+    fetch = fetcher(w, "bfloat16")
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden": D, "intermediate": I,
+                                                         "names": {"gate": "g", "up": "u", "down": "d"}}))
+    norm = build_part("norm", PartSpec("rms_norm", {"dim": D, "eps": 1e-5, "weight": "n"}))
+    ffn.load_all(fetch, "bfloat16", "cuda:0")
+    norm.load_all(fetch, "bfloat16", "cuda:0")
+    x = torch.randn(T, D, generator=g)
+    h = x.to(torch.bfloat16)
+    want = x.to(F64) + plain.swiglu(h.to(F64), w["g"], w["u"], w["d"])
+
+    ctx = make_ctx(T, "bfloat16")
+    residual = x.cuda().clone()
+    ffn.forward(ctx, h.cuda(), residual)
+    assert ctx._owed is not None, "a product over 1024 of K at this size is expected to leave its sum owed"
+    assert torch.equal(residual.cpu(), x)                          # nothing added yet
+    normed = norm.forward(ctx, residual)                           # adds what is owed, then normalises
+    assert ctx._owed is None
+    close(residual, want, 2e-3, "stream after the norm took the owed sums")
+    close(normed, plain.rms_norm(want, w["n"].to(F64), 1e-5), 1e-2, "norm of the updated stream")
+
+    ctx = make_ctx(T, "bfloat16")
+    residual2 = x.cuda().clone()
+    ffn.forward(ctx, h.cuda(), residual2)
+    ctx.settle()                                                   # what a block does before a part that does not know
+    assert ctx._owed is None and torch.equal(residual2, residual)
+
+
 def test_position_part_holds_the_reference_frequencies():
     from tie_amd.parts import PartSpec, build_part
 

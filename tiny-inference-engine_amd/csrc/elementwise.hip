@@ -234,12 +234,14 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
     return TIE_BAD_ARGUMENT;
   if (w != nullptr && out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
   const size_t stride = static_cast<size_t>(plane_stride);
-  if (w != nullptr && n % 4 == 0 && plane_stride % 4 == 0 && n <= 16384 && n >= 256 && count <= 3) {
+  if (w != nullptr && n % 4 == 0 && plane_stride % 4 == 0 && n <= 16384 && n >= 256 && (count <= 4 || count == 8)) {
 #define ROW(TO, COUNT) launch_rms_norm_row<TO, COUNT>(x, partials, stride, w, eps, static_cast<TO*>(out), nullptr, R, n, stream)
     if (out_dtype == TIE_F32) {
-      if (count == 1) ROW(float, 1); else if (count == 2) ROW(float, 2); else ROW(float, 3);
+      if (count == 1) ROW(float, 1); else if (count == 2) ROW(float, 2); else if (count == 3) ROW(float, 3);
+      else if (count == 4) ROW(float, 4); else ROW(float, 8);
     } else {
-      if (count == 1) ROW(bf16_t, 1); else if (count == 2) ROW(bf16_t, 2); else ROW(bf16_t, 3);
+      if (count == 1) ROW(bf16_t, 1); else if (count == 2) ROW(bf16_t, 2); else if (count == 3) ROW(bf16_t, 3);
+      else if (count == 4) ROW(bf16_t, 4); else ROW(bf16_t, 8);
     }
 #undef ROW
     return tie_launch_status();

@@ -32,12 +32,12 @@ __device__ __forceinline__ bf16x8_t frag_of(uint4 v) { return *reinterpret_cast<
 
 // Loads the 16-byte chunks of a (ROWS x BK) slice that this thread stages: chunk c of row r for
 // (r, c) = (t / CPR + RPP i, t % CPR) with CPR = BK / 8 chunks a row and RPP = THREADS / CPR rows a
-// pass. Rows >= limit and k >= K give zeros. With FULL the slice lies wholly below K and rows beyond
+// pass; rows are ld elements apart. Rows >= limit and k >= K give zeros. With FULL the slice lies wholly below K and rows beyond
 // the limit are clamped to the last one instead (their products land in outputs that are never
 // stored): the loads then sit in straight-line code, which lets the compiler count the loads in
 // flight exactly instead of waiting for all of them wherever branches meet.
 template <int ROWS, int BK, int THREADS, bool FULL>
-__device__ __forceinline__ void load_slice(const bf16_t* __restrict__ base, int row0, int limit, int K, int k0,
+__device__ __forceinline__ void load_slice(const bf16_t* __restrict__ base, int row0, int limit, int ld, int K, int k0,
                                            uint4 (&regs)[ROWS * (BK / 8) / THREADS]) {
   constexpr int CPR = BK / 8, RPP = THREADS / CPR;
   const int c = threadIdx.x % CPR;
@@ -47,9 +47,9 @@ __device__ __forceinline__ void load_slice(const bf16_t* __restrict__ base, int 
   for (int i = 0; i < ROWS / RPP; ++i) {
     const int row = row0 + r + RPP * i;
     if (FULL)
-      regs[i] = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(min(row, limit - 1)) * K + k);
+      regs[i] = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(min(row, limit - 1)) * ld + k);
     else
-      regs[i] = (row < limit && k < K) ? *reinterpret_cast<const uint4*>(base + static_cast<size_t>(row) * K + k)
+      regs[i] = (row < limit && k < K) ? *reinterpret_cast<const uint4*>(base + static_cast<size_t>(row) * ld + k)
                                        : make_uint4(0, 0, 0, 0);
   }
 }
@@ -68,10 +68,21 @@ __device__ __forceinline__ void store_slice(bf16_t* lds, const uint4 (&regs)[ROW
 //      3 = gated: columns come in blocks of 16 = 8 gate columns then 8 up columns of the same 8 outputs;
 //          out[m, block * 8 + j] = silu(gate_j) * up_j as bfloat16, out has N / 2 columns
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int EPI>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const bf16_t* __restrict__ x,
-                                                                          const bf16_t* __restrict__ w,
-                                                                          void* __restrict__ outp, int M, int N, int K,
-                                                                          int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const bf16_t* __restrict__ x_all,
+                                                                          const bf16_t* __restrict__ w_all,
+                                                                          void* __restrict__ out_all, int M, int N,
+                                                                          int K_all, int tiles_m, int tiles_n,
+                                                                          int slices_per_split) {
+  // blockIdx.y = which range of K this workgroup sums (one range: the whole of K); its result goes to
+  // plane blockIdx.y of the output. From here on x, w, K are that range's.
+  const int ld = K_all;
+  const int k_base = blockIdx.y * slices_per_split * BK;
+  const bf16_t* __restrict__ x = x_all + k_base;
+  const bf16_t* __restrict__ w = w_all + k_base;
+  const int K = min(K_all - k_base, slices_per_split * BK);
+  void* __restrict__ outp = gridDim.y > 1 ? static_cast<void*>(static_cast<float*>(out_all) +
+                                                                static_cast<size_t>(blockIdx.y) * M * N)
+                                          : out_all;
   constexpr int THREADS = WAVES_M * WAVES_N * 64;
   constexpr int GB_STRIDE = BK + GB_PAD;                // elements per staged row
   constexpr int GB_BK = BK;
@@ -113,18 +124,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
   uint4 ra[2][BM * (BK / 8) / THREADS], rb[2][BN * (BK / 8) / THREADS];
   const int k_tiles = (K + GB_BK - 1) / GB_BK;
   const int k_full = K / GB_BK;   // slices that lie wholly below K
-  load_slice<BM, BK, THREADS, false>(x, row0, M, K, 0, ra[0]);
-  load_slice<BN, BK, THREADS, false>(w, col0, N, K, 0, rb[0]);
+  load_slice<BM, BK, THREADS, false>(x, row0, M, ld, K, 0, ra[0]);
+  load_slice<BN, BK, THREADS, false>(w, col0, N, ld, K, 0, rb[0]);
   store_slice<BM, BK, THREADS>(lds, ra[0]);
   store_slice<BN, BK, THREADS>(lds + BM * GB_STRIDE, rb[0]);
   __syncthreads();
   // Slice 1 is in flight when the loop is entered, as it is whenever the loop comes round.
   if (k_full > 1) {
-    load_slice<BM, BK, THREADS, true>(x, row0, M, K, GB_BK, ra[1]);
-    load_slice<BN, BK, THREADS, true>(w, col0, N, K, GB_BK, rb[1]);
+    load_slice<BM, BK, THREADS, true>(x, row0, M, ld, K, GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, ld, K, GB_BK, rb[1]);
   } else if (k_tiles > 1) {
-    load_slice<BM, BK, THREADS, false>(x, row0, M, K, GB_BK, ra[1]);
-    load_slice<BN, BK, THREADS, false>(w, col0, N, K, GB_BK, rb[1]);
+    load_slice<BM, BK, THREADS, false>(x, row0, M, ld, K, GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, false>(w, col0, N, ld, K, GB_BK, rb[1]);
   }
 
   // Fragments of k step s + 1 are read from LDS before the MFMAs of step s are issued, so the
@@ -164,14 +175,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
   // kt + 1 is written to LDS. The last slices go through the general code below.
   int kt = 0;
   auto steady_pair = [&](int k) {
-    load_slice<BM, BK, THREADS, true>(x, row0, M, K, (k + 2) * GB_BK, ra[0]);
-    load_slice<BN, BK, THREADS, true>(w, col0, N, K, (k + 2) * GB_BK, rb[0]);
+    load_slice<BM, BK, THREADS, true>(x, row0, M, ld, K, (k + 2) * GB_BK, ra[0]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, ld, K, (k + 2) * GB_BK, rb[0]);
     compute(lds);
     store_slice<BM, BK, THREADS>(lds + BUF, ra[1]);
     store_slice<BN, BK, THREADS>(lds + BUF + BM * GB_STRIDE, rb[1]);
     __syncthreads();
-    load_slice<BM, BK, THREADS, true>(x, row0, M, K, (k + 3) * GB_BK, ra[1]);
-    load_slice<BN, BK, THREADS, true>(w, col0, N, K, (k + 3) * GB_BK, rb[1]);
+    load_slice<BM, BK, THREADS, true>(x, row0, M, ld, K, (k + 3) * GB_BK, ra[1]);
+    load_slice<BN, BK, THREADS, true>(w, col0, N, ld, K, (k + 3) * GB_BK, rb[1]);
     compute(lds + BUF);
     store_slice<BM, BK, THREADS>(lds, ra[0]);
     store_slice<BN, BK, THREADS>(lds + BM * GB_STRIDE, rb[0]);
@@ -189,8 +200,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
   for (; kt < k_tiles; kt += 2) {
     {  // even slice: in LDS buffer 0; slice kt + 1 sits in set 1; fetch kt + 2 into set 0
       if (kt + 2 < k_tiles) {
-        load_slice<BM, BK, THREADS, false>(x, row0, M, K, (kt + 2) * GB_BK, ra[0]);
-        load_slice<BN, BK, THREADS, false>(w, col0, N, K, (kt + 2) * GB_BK, rb[0]);
+        load_slice<BM, BK, THREADS, false>(x, row0, M, ld, K, (kt + 2) * GB_BK, ra[0]);
+        load_slice<BN, BK, THREADS, false>(w, col0, N, ld, K, (kt + 2) * GB_BK, rb[0]);
       }
       compute(lds);
       if (kt + 1 < k_tiles) {
@@ -201,8 +212,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
     }
     if (kt + 1 < k_tiles) {  // odd slice: in LDS buffer 1; slice kt + 2 sits in set 0; fetch kt + 3 into set 1
       if (kt + 3 < k_tiles) {
-        load_slice<BM, BK, THREADS, false>(x, row0, M, K, (kt + 3) * GB_BK, ra[1]);
-        load_slice<BN, BK, THREADS, false>(w, col0, N, K, (kt + 3) * GB_BK, rb[1]);
+        load_slice<BM, BK, THREADS, false>(x, row0, M, ld, K, (kt + 3) * GB_BK, ra[1]);
+        load_slice<BN, BK, THREADS, false>(w, col0, N, ld, K, (kt + 3) * GB_BK, rb[1]);
       }
       compute(lds + BUF);
       if (kt + 2 < k_tiles) {
@@ -244,10 +255,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
-static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, int N, int K, hipStream_t stream) {
+static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, int N, int K, int splits,
+                       hipStream_t stream) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int k_slices = (K + BK - 1) / BK;
+  const int per_split = (k_slices + splits - 1) / splits;
+  if ((k_slices + per_split - 1) / per_split != splits) return TIE_BAD_ARGUMENT;   // a range would be empty
   const size_t shared = sizeof(bf16_t) * 2 * (BM + BN) * (BK + GB_PAD);
-  const dim3 grid(tiles_m * tiles_n);
+  const dim3 grid(tiles_m * tiles_n, splits);
   // The two staging buffers may exceed the 64 KB a kernel can use without asking; gfx950 has 160 KB a CU.
 #define LAUNCH(EPI)                                                                                          \
   {                                                                                                          \
@@ -260,24 +275,45 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
       raised = true;                                                                                         \
     }                                                                                                        \
     gemm_bf16_kernel<BM, BN, BK, WAVES_M, WAVES_N, EPI><<<grid, WAVES_M * WAVES_N * 64, shared, stream>>>(    \
-        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n);       \
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n,        \
+        per_split);                                                                                          \
   }
   if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
 #undef LAUNCH
   return tie_launch_status();
 }
 
+// Ranges of K that a product of M rows over w[N, K] is best cut into when its caller adds planes of
+// partial sums: few rows over a narrow weight give too few workgroups otherwise.
+extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
+  const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles >= 256) return 1;
+  const int k_slices = (K + 63) / 64;
+  // 2, 4 or 8 ranges of at least 512 of K each, none of them empty.
+  for (int splits = 8; splits >= 2; splits /= 2) {
+    if (static_cast<long>(splits) * tiles > 256 && splits > 2) continue;   // more planes cost more than they fill
+    if (splits > k_slices / 8) continue;
+    const int per = (k_slices + splits - 1) / splits;
+    if ((k_slices + per - 1) / per == splits) return splits;
+  }
+  return 1;
+}
+
 // out_dtype: TIE_F32 or TIE_BF16; accumulate adds into a float32 output; gated (bfloat16 output of N / 2
 // columns, N % 16 == 0) applies silu(gate) * up to interleaved column blocks.
+// splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K
+// (128x128 tiles; neither accumulate nor gated).
 // tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
 //       3 = 256x128 (eight waves of 64x64).
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
-                             int N, int K, int tile, hipStream_t stream) {
-  if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0) return TIE_BAD_ARGUMENT;
+                             int N, int K, int tile, int splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1) return TIE_BAD_ARGUMENT;
   if (accumulate && out_dtype != TIE_F32) return TIE_BAD_ARGUMENT;
   if (out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || out_dtype != TIE_BF16 || N % 16 != 0)) return TIE_BAD_ARGUMENT;
+  if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
+  if (splits > 1) tile = 1;
   if (tile == 0) {
     // Larger tiles need fewer operand bytes per flop; take the largest that still gives most CUs a tile.
     const long rows256 = (M + 255) / 256;
@@ -285,7 +321,7 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
     else if (rows256 * ((N + 127) / 128) >= 192) tile = 3;
     else tile = 1;
   }
-  if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, stream);
-  if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, stream);
-  return launch_gemm<128, 128, 64, 2, 2>(x, w, out, epi, M, N, K, stream);
+  if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, splits, stream);
+  if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, splits, stream);
+  return launch_gemm<128, 128, 64, 2, 2>(x, w, out, epi, M, N, K, splits, stream);
 }

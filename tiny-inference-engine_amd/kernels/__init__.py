@@ -67,7 +67,9 @@ _SIGNATURES = {
                                  _c_void],
     },
     "gemm_bf16": {
-        "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+        "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int],
+        "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                          _c_void],
     },
     "attention_prefill_bf16": {
         "tie_attention_prefill_rows_per_item": [_c_int],
@@ -328,18 +330,30 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
         int(splits), _stream()), "skinny_gemm_bf16")
 
 
+def gemm_splits(M: int, N: int, K: int) -> int:
+    """Ranges of K a product of M > 64 rows over a ``[N, K]`` weight is best cut into when its caller adds partial sums."""
+    return int(_lib("gemm_bf16").tie_gemm_bf16_splits(M, N, K))
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0,
-              gated: bool = False) -> None:
+              gated: bool = False, splits: int = 1) -> None:
     """out (+)= x @ w.T for bfloat16 operands on the matrix cores, any number of rows; K % 8 == 0.
 
     ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256, 3 = 256x128; 0 lets the kernel choose);
-    ``gated`` as in ``skinny_gemm_bf16``.
+    ``gated`` and ``splits`` as in ``skinny_gemm_bf16`` (planes of partial sums, ``[splits, M, N]`` float32).
     """
-    M, N, K = _bf16_product_operands(x, w, out, gated, "gemm_bf16")
+    if splits > 1:
+        if out.dim() != 3 or out.shape[0] != splits or out.dtype != torch.float32 or accumulate or gated:
+            raise InvalidArgument(f"gemm_bf16: {splits} splits need a float32 output of {splits} planes, got "
+                                  f"{list(out.shape)} {out.dtype}, and neither accumulate nor gated")
+        M, N, K = _bf16_product_operands(x, w, out[0], gated, "gemm_bf16")
+    else:
+        M, N, K = _bf16_product_operands(x, w, out, gated, "gemm_bf16")
     if accumulate and (gated or out.dtype != torch.float32):
         raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only, and not in a gated product")
     _check(_lib("gemm_bf16").tie_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
-                                           int(accumulate), int(gated), M, N, K, tile, _stream()), "gemm_bf16")
+                                           int(accumulate), int(gated), M, N, K, tile, int(splits), _stream()),
+           "gemm_bf16")
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -28,6 +28,7 @@ class Linear:
         self.init_std = init_std
         self.weight: torch.Tensor = None
         self._splits = None
+        self._tiled_splits = {}
 
     @property
     def total_out(self) -> int:
@@ -63,15 +64,28 @@ class Linear:
         return out
 
     def partial_planes(self, ctx, x: torch.Tensor, name: str):
-        """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None."""
+        """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None.
+
+        Up to 64 rows the decode product decides by the weight's shape alone; above, the tiled
+        product is cut along K when its tiles alone would leave most of the GPU idle.
+        """
         M, K = x.shape
         w = self.weight
-        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or M > 64 or K % 8:
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8:
             return None
-        if self._splits is None:
-            self._splits = kernels.skinny_splits(w.shape[0], K)
-        if self._splits <= 1:
+        if M <= 64:
+            if self._splits is None:
+                self._splits = kernels.skinny_splits(w.shape[0], K)
+            splits = self._splits
+        else:
+            splits = self._tiled_splits.get(M)
+            if splits is None:
+                splits = self._tiled_splits[M] = kernels.gemm_splits(M, w.shape[0], K)
+        if splits <= 1:
             return None
-        planes = ctx.scratch(name, (self._splits, M, w.shape[0]), torch.float32)
-        kernels.skinny_gemm_bf16(x, w, planes, splits=self._splits)
+        planes = ctx.scratch(name, (splits, M, w.shape[0]), torch.float32)
+        if M <= 64:
+            kernels.skinny_gemm_bf16(x, w, planes, splits=splits)
+        else:
+            kernels.gemm_bf16(x, w, planes, splits=splits)
         return planes
