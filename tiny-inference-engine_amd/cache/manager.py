@@ -44,12 +44,14 @@ FREED = -1  # table entry of a page that a window has passed and that was given 
 class RequestCache:
     """What one request holds in the cache: a block table per group and a state slot."""
 
-    __slots__ = ("tables", "trimmed", "state_slot")
+    __slots__ = ("tables", "trimmed", "state_slot", "version", "rows")
 
     def __init__(self, num_groups: int):
         self.tables: List[List[int]] = [[] for _ in range(num_groups)]
         self.trimmed: List[int] = [0] * num_groups
         self.state_slot: int = -1
+        self.version: int = 0                     # grows whenever a table changes
+        self.rows: List[object] = [None] * num_groups   # a step builder's memo of each table as an array row
 
     def num_held(self) -> int:
         return sum(1 for table in self.tables for b in table if b != FREED)
@@ -177,6 +179,8 @@ class CacheManager:
                 tensor[:, slot].zero_()
         for g, pool in self.pools.items():
             table = req.tables[g]
+            if len(table) < want:
+                req.version += 1
             while len(table) < want:
                 table.append(pool.allocate())
         return True
@@ -202,6 +206,7 @@ class CacheManager:
         if length < 0:
             raise InvalidArgument(f"cannot truncate a block table to {length} tokens")
         keep = self.blocks_for(length)
+        req.version += 1
         for g, pool in self.pools.items():
             table = req.tables[g]
             while len(table) > keep:
@@ -232,6 +237,7 @@ class CacheManager:
                     pool.release(table[i])
                     table[i] = FREED
                     freed += 1
+                    req.version += 1
             req.trimmed[g] = max(req.trimmed[g], first_page)
         return freed
 
@@ -245,6 +251,7 @@ class CacheManager:
 
     def release(self, req: RequestCache) -> None:
         """Gives back everything the request holds (it ended, was cancelled or is preempted)."""
+        req.version += 1
         for g, pool in self.pools.items():
             for page in req.tables[g]:
                 if page != FREED:

@@ -11,6 +11,7 @@ geometry (``src/kv/paged_kv_cache.h:27-30``) - and no fixed-size state at all.
 from __future__ import annotations
 
 import dataclasses
+import functools
 from typing import List, Optional, Sequence, Tuple, Union
 
 from ..errors import InvalidArgument
@@ -71,11 +72,11 @@ class CachePlan:
     groups: Tuple[CacheGroup, ...]
     calls: Tuple[Optional[CallCache], ...]
 
-    @property
+    @functools.cached_property
     def paged_groups(self) -> List[int]:
         return [i for i, g in enumerate(self.groups) if isinstance(g.need, PagedKV)]
 
-    @property
+    @functools.cached_property
     def state_groups(self) -> List[int]:
         return [i for i, g in enumerate(self.groups) if isinstance(g.need, FixedState)]
 

@@ -99,6 +99,20 @@ class BatchBuilder:
         """Address of the device-side staging buffer; a recorded step is bound to it."""
         return 0 if self._dev is None else self._dev.data_ptr()
 
+    @staticmethod
+    def _table_row(cache, g: int, MB: int) -> np.ndarray:
+        """A request's block table of group ``g`` as a row of ``MB`` page numbers (0 where there is none).
+
+        Kept on the request between steps and rebuilt only when the table has changed."""
+        memo = cache.rows[g]
+        if memo is None or memo[0] != cache.version or memo[1].shape[0] != MB:
+            arr = np.zeros(MB, dtype=np.int32)
+            table = cache.tables[g][:MB]
+            if table:
+                arr[:len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)    # FREED (-1) -> 0
+            memo = cache.rows[g] = (cache.version, arr)
+        return memo[1]
+
     def build(self, entries: Sequence[StepEntry]) -> StepBatch:
         if not entries:
             raise InvalidArgument("a step needs at least one entry")
@@ -159,30 +173,45 @@ class BatchBuilder:
         row = 0
         r = 0
         query_start[0] = 0
+        slot_views = [view(("slots", g)) for g in groups]
+        table_views = [view(("tables", g)) for g in groups]
         for s, e in enumerate(entries):
             n = len(e.tokens)
-            ids = np.asarray(e.tokens, dtype=np.int64)
-            if ids.min() < 0 or ids.max() >= self.vocab_size:
-                bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
-                raise InvalidArgument(f"token id {bad} outside vocabulary of {self.vocab_size}")
-            tokens[row:row + n] = ids
-            positions[row:row + n] = np.arange(e.start, e.start + n, dtype=np.int32)
-            seq_of_row[row:row + n] = s
-            context_lens[s] = e.start + n
+            start = e.start
+            if n == 1:                                  # a decoded token: no arrays needed
+                tok = e.tokens[0]
+                if not 0 <= tok < self.vocab_size:
+                    raise InvalidArgument(f"token id {tok} outside vocabulary of {self.vocab_size}")
+                tokens[row] = tok
+                positions[row] = start
+                seq_of_row[row] = s
+            else:
+                ids = np.asarray(e.tokens, dtype=np.int64)
+                if ids.min() < 0 or ids.max() >= self.vocab_size:
+                    bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
+                    raise InvalidArgument(f"token id {bad} outside vocabulary of {self.vocab_size}")
+                tokens[row:row + n] = ids
+                positions[row:row + n] = np.arange(start, start + n, dtype=np.int32)
+                seq_of_row[row:row + n] = s
+            context_lens[s] = start + n
             state_slots[s] = max(e.cache.state_slot, 0)
             for w in e.want:
                 logit_rows[r] = row + w
                 r += 1
-            for g in groups:
+            for gi, g in enumerate(groups):
                 table = e.cache.tables[g]
-                view(("slots", g))[row:row + n] = self.cache.slots(e.cache, g, e.start, e.start + n)
-                trow = view(("tables", g))[s * MB:(s + 1) * MB]
-                trow[:len(table)] = [0 if b == FREED else b for b in table][:MB]
-                trow[len(table):] = 0
+                if n == 1:
+                    page = table[start // bs]
+                    if page == FREED:
+                        raise InvalidArgument(f"position {start} lies in a page that was already given back")
+                    slot_views[gi][row] = page * bs + start % bs
+                else:
+                    slot_views[gi][row:row + n] = self.cache.slots(e.cache, g, start, start + n)
+                table_views[gi][s * MB:(s + 1) * MB] = self._table_row(e.cache, g, MB)
             row += n
             query_start[s + 1] = row
             batch.host_new_tokens.append(n)
-            batch.host_context_lens.append(e.start + n)
+            batch.host_context_lens.append(start + n)
             batch.host_state_slots.append(e.cache.state_slot)
 
         dev_t[:offset].copy_(host_t[:offset], non_blocking=True)
