@@ -151,6 +151,54 @@ def test_requests_batched_together_generate_what_each_generates_alone(model_fold
         assert alone.generate(prompt, params) == together.sequence(sid).generated, f"request {sid}"
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_crowded_engine_finishes_everything_twice_the_same_way(model_folders, model_folders_bf16, dtype):
+    """Thirty requests of mixed lengths and sampling through a small pool: chunked prompts, decode steps
+    replayed from recorded graphs, preemption and recomputation. Everything finishes with the right
+    number of tokens, every page comes back, and a second engine fed the same way produces the same
+    tokens (the same batches run the same kernels in the same order: nothing depends on timing)."""
+    import random
+
+    import tie_amd
+
+    folder, cfg = (model_folders_bf16 if dtype == "bfloat16" else model_folders)["B"]
+    rng = random.Random(12)
+    reqs = []
+    for i in range(30):
+        prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(rng.choice([1, 3, 17, 40, 75]))]
+        kind = i % 3
+        params = tie_amd.SamplingParams(max_tokens=rng.choice([1, 5, 24]), seed=i,
+                                        temperature=0.0 if kind == 0 else 0.8,
+                                        top_k=0 if kind < 2 else 10, top_p=1.0 if kind < 2 else 0.9)
+        reqs.append((prompt, params))
+
+    def run():
+        engine = make_engine(folder, 16, dtype=dtype, kv_blocks=14, max_seqs=6, max_tokens_per_step=48,
+                             prefill_chunk=32, policy="fcfs", watermark_blocks=0)
+        pending = list(reqs)
+        ids = []
+        steps = 0
+        while pending or engine.has_work():
+            for _ in range(2):                                # requests keep arriving while others run
+                if pending:
+                    ids.append(engine.add_request(*pending.pop(0)))
+            engine.step()
+            steps += 1
+            engine.cache.audit([engine.sequence(i).cache for i in ids if engine.sequence(i).cache is not None])
+            assert steps < 3000, "the engine does not finish"
+        assert engine.cache.num_free() == 14
+        out = [engine.sequence(i).generated for i in ids]
+        for (prompt, params), tokens in zip(reqs, out):
+            assert len(tokens) == params.max_tokens
+            assert all(0 <= t < cfg["vocab_size"] for t in tokens)
+        return out, engine.stats()
+
+    first, stats = run()
+    assert stats.preemptions > 0 and stats.seqs_scheduled > 2 * stats.steps
+    second, _ = run()
+    assert first == second
+
+
 def test_a_failing_step_is_rolled_back_and_offered_again(model_folders):
     import tie_amd
 
