@@ -35,6 +35,7 @@ SHAPES = {
     "dh24_generic_attention": (config(2, 48, 4, 4, 24, 40, 77, tied=True), 4, [4, 31, 64, 90]),
     "dh256": (config(1, 64, 2, 1, 256, 96, 130), 32, [1, 50, 64, 140]),
     "dh96_dh112": (config(1, 88, 6, 3, 96, 104, 211), 8, [7, 70, 129]),
+    "block_of_12": (config(1, 64, 4, 2, 32, 72, 90), 12, [5, 40, 100]),       # no power of two: generic attention
 }
 
 

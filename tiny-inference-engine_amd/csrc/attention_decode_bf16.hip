@@ -93,8 +93,8 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
   // Positions are clamped into [start, pos] for addresses only (pages outside that range may be gone or
   // never have been there); what lies outside is masked in the softmax.
-  auto page_of = [&](int kp) { return block_shift >= 0 ? kp >> block_shift : kp / block_size; };
-  auto offset_of = [&](int kp) { return block_shift >= 0 ? kp & (block_size - 1) : kp % block_size; };
+  auto page_of = [&](int kp) { return kp >> block_shift; };          // block sizes are powers of two here
+  auto offset_of = [&](int kp) { return kp & (block_size - 1); };
   // This lane's keys of a tile: rows of the two sub-tiles, and the runs of values it reads.
   const int krow0 = (col >> 2) * 8 + (col & 3);        // sub-tile 1: + 4
   constexpr int VG = WIDE ? 8 : 4;
@@ -282,12 +282,13 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
                                          int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
                                          int window, int nsplit, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
-      block_size <= 0 || block_size % 4 != 0 || max_blocks <= 0 || nsplit <= 0 || nsplit > MERGE_MAX_SPLITS ||
+      block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
+      nsplit > MERGE_MAX_SPLITS ||
       !(scale > 0.f))   // the running maximum is kept on unscaled scores
     return TIE_BAD_ARGUMENT;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr)) return TIE_BAD_ARGUMENT;
   const dim3 grid(nsplit, KVH, num_seqs);
-  const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
 #define LAUNCH(WIDE)                                                                                            \
   attention_decode_kernel<WIDE><<<grid, TIE_WAVE, 0, stream>>>(                                                  \

@@ -63,8 +63,8 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 // calling kernel. Key positions are clamped into [first, last]: pages before or after the range this
 // workgroup may touch are never addressed (their table entries need not be valid); clamped keys are
 // masked by position later. A macro, so that the register arrays are plain locals of the kernel.
-#define PAGE_OF(kp) (block_shift >= 0 ? (kp) >> block_shift : (kp) / block_size)
-#define OFFSET_OF(kp) (block_shift >= 0 ? (kp) & (block_size - 1) : (kp) % block_size)
+#define PAGE_OF(kp) ((kp) >> block_shift)
+#define OFFSET_OF(kp) ((kp) & (block_size - 1))
 // LOAD_PAGES looks up the pages of every piece of a tile this thread copies; LOAD_TILE then reads the
 // pieces. Two steps, so that all lookups are in flight together and no data load waits for one:
 // the pages of tile t + 2 are looked up while the data of tile t + 1 is on its way.
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
-    int max_blocks, float scale_log2e, int window, int block_shift) {
+    int max_blocks, float scale_log2e, int window, int block_shift, int flip_from) {
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -156,7 +156,10 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
   const int r32 = lane & 31;
   const int hi = lane >> 5;
   const int hc = wave / QC, qc = wave % QC;
-  const int item = num_items - 1 - blockIdx.x;   // long rows (late in a prompt) first
+  // Long rows (late in a prompt) first. Where the whole grid is resident at once (two workgroups a CU),
+  // the second half of it runs short rows first instead, so that a CU's two workgroups add up alike.
+  const bool flipped = static_cast<int>(blockIdx.y + blockIdx.z * gridDim.y) >= flip_from;
+  const int item = flipped ? static_cast<int>(blockIdx.x) : num_items - 1 - static_cast<int>(blockIdx.x);
   const int s = items[item * 2];
   const int row0 = items[item * 2 + 1];
   const int kvh = blockIdx.y;
@@ -315,6 +318,18 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
     }
 }
 
+static int compute_units() {
+  static int cached = 0;
+  if (cached == 0) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      count = 256;
+    cached = count;
+  }
+  return cached;
+}
+
 static void shape_for_group(int G, int* hc, int* qc) {
   *hc = G >= 4 ? 4 : G;
   *qc = *hc == 4 || *hc == 3 ? 1 : (*hc == 2 ? 2 : 4);
@@ -332,7 +347,10 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
                           int max_blocks, float scale_log2e, int window) {
-  const int block_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  const int block_shift = __builtin_ctz(block_size);   // block sizes are powers of two here
+  // One resident round (at most two workgroups on each of the compute units): see the kernel's item order.
+  const long planes = static_cast<long>(grid.y) * grid.z;
+  const int flip_from = (planes >= 2 && planes * grid.x <= 2L * compute_units()) ? static_cast<int>(planes / 2) : 0x7fffffff;
   constexpr size_t lds_bytes = 2 * static_cast<size_t>(LDS_TILE) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
@@ -343,7 +361,7 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   }
   attention_prefill_kernel<HC, QC, WIDE><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, window, block_shift);
+      max_blocks, scale_log2e, window, block_shift, flip_from);
   return tie_launch_status();
 }
 
@@ -351,8 +369,8 @@ extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, co
                                           const int* query_start, const int* context_lens, const int* block_tables,
                                           const int* items, int num_items, int H, int KVH, int block_size,
                                           int max_blocks, float scale, int window, hipStream_t stream) {
-  if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size <= 0 || block_size % 4 != 0 ||
-      max_blocks <= 0 || !(scale > 0.f))   // the running maximum is kept on unscaled scores
+  if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size < 4 ||
+      (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f))   // the running maximum is kept on unscaled scores
     return TIE_BAD_ARGUMENT;
   const int G = H / KVH;
   int hc, qc;

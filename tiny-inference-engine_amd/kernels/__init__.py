@@ -529,6 +529,11 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
                                           out.data_ptr(), R, V, _stream()), "sample")
 
 
+def mfma_block_size(block_size: int) -> bool:
+    """Block sizes the matrix-core attention kernels take: powers of two from 4 (others go to the generic kernel)."""
+    return block_size >= 4 and block_size & (block_size - 1) == 0
+
+
 def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
     """How many ways the keys of each sequence are split so that a decode step fills the GPU."""
     target_waves = 2048
@@ -554,9 +559,9 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         raise InvalidArgument("attention_decode_bf16 takes bfloat16 queries, cache and output")
     if q.shape[1] != H * Dh or out.shape != q.shape:
         raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
-    if Dh not in MFMA_HEAD_DIMS or H % KVH or H // KVH > 16 or bs % 4:
+    if Dh not in MFMA_HEAD_DIMS or H % KVH or H // KVH > 16 or not mfma_block_size(bs):
         raise InvalidArgument(f"attention_decode_bf16 takes head sizes in steps of 16 up to 256, at most 16 query heads "
-                              f"a KV head and block sizes in steps of 4; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+                              f"a KV head and block sizes 4, 8, 16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
     _i32(query_start, "query_start")
     _i32(context_lens, "context_lens")
     _i32(block_tables, "block tables")
@@ -604,9 +609,9 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         raise InvalidArgument("attention_prefill_bf16 takes bfloat16 queries, cache and output")
     if q.shape[1] != H * Dh or out.shape != q.shape:
         raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
-    if Dh not in MFMA_HEAD_DIMS or H % KVH or bs % 4:
-        raise InvalidArgument(f"attention_prefill_bf16 takes head sizes in steps of 16 up to 256 and block sizes in "
-                              f"steps of 4; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+    if Dh not in MFMA_HEAD_DIMS or H % KVH or not mfma_block_size(bs):
+        raise InvalidArgument(f"attention_prefill_bf16 takes head sizes in steps of 16 up to 256 and block sizes 4, 8, "
+                              f"16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
     _i32(query_start, "query_start")
     _i32(context_lens, "context_lens")
     _i32(block_tables, "block tables")
@@ -630,7 +635,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """
     NB, KVH, bs, Dh = k_cache.shape
     fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
-            and num_heads % KVH == 0 and bs % 4 == 0 and scratch is not None)
+            and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
         nsplit = decode_splits(S, KVH, batch.plan_context)
