@@ -647,13 +647,33 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                               S, num_heads, scale, window, nsplit, part_o, part_ml)
         return
     if fast:
-        key = ("prefill_items", num_heads // KVH)
-        items = batch.memo.get(key)
-        if items is None:          # the same for every layer of the step: built once
-            host = torch.tensor(prefill_items(batch.host_new_tokens, num_heads // KVH), dtype=torch.int32)
-            items = batch.memo[key] = host.to(q.device)
-        attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                               items, num_heads, scale, window)
+        # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
+        # split over many waves), the prompt portions to the prefill kernel. Built once a step.
+        G = num_heads // KVH
+        key = ("attention_work", G)
+        work = batch.memo.get(key)
+        if work is None:
+            new = batch.host_new_tokens
+            single = [s for s, n in enumerate(new) if n == 1] if G <= 16 else []
+            if len(single) == len(new):
+                single = []                                   # nothing but single rows and yet not a decode step
+            taken = set(single)
+            items = [it for it in prefill_items(new, G) if it[0] not in taken]
+            work = batch.memo[key] = (
+                torch.tensor(single, dtype=torch.int32).to(q.device) if single else None, len(single),
+                torch.tensor(items, dtype=torch.int32).to(q.device) if items else None)
+        seq_ids, num_single, items = work
+        if num_single:
+            nsplit = decode_splits(num_single, KVH, batch.plan_context)
+            part_o = part_ml = None
+            if nsplit > 1:
+                part_o = scratch("attention.split_o", (num_single * num_heads * nsplit * Dh,), torch.float32)
+                part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
+            attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
+                                  num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids)
+        if items is not None:
+            attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens,
+                                   step.block_tables, items, num_heads, scale, window)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window)
