@@ -381,14 +381,21 @@ def test_attention_decode_bf16_window_edges(window):
 
 
 
-def run_prefill(case, H, KVH, lens_new, window=None):
+def run_prefill(case, H, KVH, lens_new, window=None, nsplit=1):
     from tie_amd import kernels
 
     q = case["q"]
     out = torch.full_like(q, float("nan"))
+    Dh = q.shape[1] // H
     items = torch.tensor(kernels.prefill_items(lens_new, H // KVH), dtype=torch.int32).cuda()
+    extra = {}
+    if nsplit > 1:          # the keys of every item in shares, merged by a second kernel
+        rows = q.shape[0]
+        extra = dict(nsplit=nsplit, merge_rows=i32(list(range(rows))),
+                     part_o=torch.full((rows * H * nsplit * Dh,), float("nan"), dtype=torch.float32, device="cuda"),
+                     part_ml=torch.full((rows * H * nsplit * 2,), float("nan"), dtype=torch.float32, device="cuda"))
     kernels.attention_prefill_bf16(q, case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
-                                   case["tables"], items, H, (q.shape[1] // H) ** -0.5, window)
+                                   case["tables"], items, H, Dh ** -0.5, window, **extra)
     return out
 
 
@@ -403,12 +410,14 @@ def test_attention_prefill_bf16_mixed_batch(H, KVH, Dh, bs):
 
 
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(8, 2, 128, 16), (2, 2, 64, 8), (6, 3, 32, 4)])
-def test_attention_prefill_bf16_long_portions(H, KVH, Dh, bs):
-    # several key tiles per workgroup, row tiles that end inside a tile, a long cached prefix
+@pytest.mark.parametrize("nsplit", [1, 3, 8])
+def test_attention_prefill_bf16_long_portions(H, KVH, Dh, bs, nsplit):
+    # several key tiles per workgroup, row tiles that end inside a tile, a long cached prefix; with nsplit > 1
+    # every item's keys are cut into shares (short items leave some of them empty) and merged
     lens_new, lens_ctx = [300, 130, 64, 33], [300, 1000, 64, 129]
     case, S = attention_case(H, KVH, Dh, bs, lens_new=lens_new, lens_ctx=lens_ctx, seed=24, dtype=torch.bfloat16)
-    out = run_prefill(case, H, KVH, lens_new)
-    close(out, case["want"], 1e-2, f"prefill attention, long portions, H={H} KVH={KVH} Dh={Dh} bs={bs}")
+    out = run_prefill(case, H, KVH, lens_new, nsplit=nsplit)
+    close(out, case["want"], 1e-2, f"prefill attention, long portions, H={H} KVH={KVH} Dh={Dh} bs={bs} splits={nsplit}")
 
 
 @pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "tile_edge_64", "far", "last"])
@@ -426,8 +435,9 @@ def test_attention_prefill_bf16_finds_one_far_key(where):
 def test_attention_prefill_bf16_window_edges(window):
     lens_new, lens_ctx = [9, 1, 20, 50], [30, 41, 20, 200]
     case, S = attention_case(4, 2, 32, 4, lens_new=lens_new, lens_ctx=lens_ctx, seed=27, dtype=torch.bfloat16, window=window)
-    out = run_prefill(case, 4, 2, lens_new, window=window)
-    close(out, case["want"], 1e-2, f"prefill window {window}")
+    for nsplit in (1, 4):
+        out = run_prefill(case, 4, 2, lens_new, window=window, nsplit=nsplit)
+        close(out, case["want"], 1e-2, f"prefill window {window} splits {nsplit}")
 
 
 def test_argmax_and_sample_kernels():

@@ -148,7 +148,8 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
-    int max_blocks, float scale_log2e, int window, int block_shift, int flip_from) {
+    int max_blocks, float scale_log2e, int window, int block_shift, int flip_from, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -159,7 +160,10 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
   // Long rows (late in a prompt) first. Where the whole grid is resident at once (two workgroups a CU),
   // the second half of it runs short rows first instead, so that a CU's two workgroups add up alike.
   const bool flipped = static_cast<int>(blockIdx.y + blockIdx.z * gridDim.y) >= flip_from;
-  const int item = flipped ? static_cast<int>(blockIdx.x) : num_items - 1 - static_cast<int>(blockIdx.x);
+  // With nsplit > 1 a workgroup walks only its share of the item's key tiles and leaves partial results.
+  const int bx = static_cast<int>(blockIdx.x) / nsplit;
+  const int split = static_cast<int>(blockIdx.x) % nsplit;
+  const int item = flipped ? bx : num_items - 1 - bx;
   const int s = items[item * 2];
   const int row0 = items[item * 2 + 1];
   const int kvh = blockIdx.y;
@@ -202,16 +206,24 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
     for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  const int tile_begin = wg_first / KT, tile_end = wg_last / KT;
+  int tile_begin = wg_first / KT, tile_end = wg_last / KT;       // inclusive
+  if (nsplit > 1) {
+    const int per = (tile_end - tile_begin + nsplit) / nsplit;   // ceil(count / nsplit)
+    tile_begin += split * per;
+    tile_end = min(tile_end, tile_begin + per - 1);
+  }
+  const bool empty = tile_begin > tile_end;                      // uniform: a short row range has fewer tiles than splits
   const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
   const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
   constexpr int VG = WIDE ? 8 : 4;   // keys of one value dimension read in one piece
   u32x4_t kreg[K_PER_THREAD], vreg[V_PER_THREAD];
   int kpage[K_PER_THREAD], vpage[V_PER_THREAD][WIDE ? 1 : 2];
-  LOAD_PAGES(tile_begin);
-  LOAD_TILE(tile_begin);
-  if (tile_begin < tile_end) LOAD_PAGES(tile_begin + 1);
-  STORE_TILE(lds, lds + KT * KROW);
+  if (!empty) {
+    LOAD_PAGES(tile_begin);
+    LOAD_TILE(tile_begin);
+    if (tile_begin < tile_end) LOAD_PAGES(tile_begin + 1);
+    STORE_TILE(lds, lds + KT * KROW);
+  }
   __syncthreads();
 
   for (int tile = tile_begin; tile <= tile_end; ++tile) {
@@ -304,9 +316,27 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
 
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (!valid) return;
+  // Element v of acc[dt] is dimension dt*32 + 8*(v/4) + hi*4 + v%4.
+  if (nsplit > 1) {   // partial results of this share of the keys, merged by a second kernel
+    const size_t slot = (static_cast<size_t>(qs + i) * H + head0 + hc) * nsplit + split;
+    float* po = part_o + slot * DH;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        const int d0 = dt * 32 + 8 * vq + hi * 4;
+        if (DH % 32 != 0 && d0 >= DH) continue;
+        *reinterpret_cast<float4*>(po + d0) =
+            make_float4(acc[dt][vq * 4], acc[dt][vq * 4 + 1], acc[dt][vq * 4 + 2], acc[dt][vq * 4 + 3]);
+      }
+    if (hi == 0) {
+      part_ml[slot * 2] = m * scale_log2e;     // the merge works in the exponent's units (base 2); -inf if empty
+      part_ml[slot * 2 + 1] = l;
+    }
+    return;
+  }
   const float inv = 1.0f / l;
   bf16_t* o = out + (static_cast<size_t>(qs + i) * H + head0 + hc) * DH;
-  // Element v of acc[dt] is dimension dt*32 + 8*(v/4) + hi*4 + v%4.
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -317,6 +347,8 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
                                                      pack2(acc[dt][vq * 4 + 2] * inv, acc[dt][vq * 4 + 3] * inv));
     }
 }
+
+#include "attention_merge.h"
 
 static int compute_units() {
   static int cached = 0;
@@ -346,11 +378,12 @@ template <int HC, int QC, bool WIDE>
 static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
-                          int max_blocks, float scale_log2e, int window) {
+                          int max_blocks, float scale_log2e, int window, int nsplit, float* part_o, float* part_ml) {
   const int block_shift = __builtin_ctz(block_size);   // block sizes are powers of two here
   // One resident round (at most two workgroups on each of the compute units): see the kernel's item order.
   const long planes = static_cast<long>(grid.y) * grid.z;
-  const int flip_from = (planes >= 2 && planes * grid.x <= 2L * compute_units()) ? static_cast<int>(planes / 2) : 0x7fffffff;
+  const int flip_from = (nsplit == 1 && planes >= 2 && planes * grid.x <= 2L * compute_units())
+                            ? static_cast<int>(planes / 2) : 0x7fffffff;
   constexpr size_t lds_bytes = 2 * static_cast<size_t>(LDS_TILE) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
@@ -361,32 +394,47 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   }
   attention_prefill_kernel<HC, QC, WIDE><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, window, block_shift, flip_from);
+      max_blocks, scale_log2e, window, block_shift, flip_from, nsplit, part_o, part_ml);
   return tie_launch_status();
 }
 
+// nsplit > 1: every item's keys are cut into nsplit shares, one workgroup each; part_o
+// [rows][H][nsplit][DH] and part_ml [rows][H][nsplit][2] (rows = all rows of the step) take the
+// partial results and a second kernel merges them into out for the num_rows rows of the step.
 extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
                                           const int* query_start, const int* context_lens, const int* block_tables,
                                           const int* items, int num_items, int H, int KVH, int block_size,
-                                          int max_blocks, float scale, int window, hipStream_t stream) {
+                                          int max_blocks, float scale, int window, int nsplit, float* part_o,
+                                          float* part_ml, const int* merge_rows, int num_merge_rows,
+                                          hipStream_t stream) {
   if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size < 4 ||
-      (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f))   // the running maximum is kept on unscaled scores
+      (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f) || nsplit < 1 ||
+      nsplit > MERGE_MAX_SPLITS)   // the running maximum is kept on unscaled scores
+    return TIE_BAD_ARGUMENT;
+  if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr || merge_rows == nullptr || num_merge_rows <= 0 ||
+                     num_merge_rows > 65535))
     return TIE_BAD_ARGUMENT;
   const int G = H / KVH;
   int hc, qc;
   shape_for_group(G, &hc, &qc);
   const int passes = (G + hc - 1) / hc;
   if (passes > 65535) return TIE_BAD_ARGUMENT;
-  const dim3 grid(num_items, KVH, passes);
+  const dim3 grid(num_items * nsplit, KVH, passes);
   const float scale_log2e = scale * 1.44269504088896340736f;
+  int status;
 #define LAUNCH(HC, QC)                                                                                            \
-  return (block_size % 8 == 0 ? launch_prefill<HC, QC, true> : launch_prefill<HC, QC, false>)(                    \
+  status = (block_size % 8 == 0 ? launch_prefill<HC, QC, true> : launch_prefill<HC, QC, false>)(                  \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, window)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, window, nsplit, part_o, part_ml)
   if (hc == 4) LAUNCH(4, 1);
-  if (hc == 3) LAUNCH(3, 1);
-  if (hc == 2) LAUNCH(2, 2);
-  LAUNCH(1, 4);
+  else if (hc == 3) LAUNCH(3, 1);
+  else if (hc == 2) LAUNCH(2, 2);
+  else LAUNCH(1, 4);
 #undef LAUNCH
+  if (status != TIE_OK || nsplit == 1) return status;
+  const int merge_threads = (nsplit > DH ? nsplit : DH) <= 64 ? 64 : ((nsplit > DH ? nsplit : DH) <= 128 ? 128 : 256);
+  attention_merge_rows_kernel<<<dim3(H, num_merge_rows), merge_threads, 0, stream>>>(
+      part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, H, nsplit);
+  return tie_launch_status();
 }

@@ -74,7 +74,8 @@ _SIGNATURES = {
     "attention_prefill_bf16": {
         "tie_attention_prefill_rows_per_item": [_c_int],
         "tie_attention_prefill_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int,
-                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+                                       _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void, _c_void,
+                                       _c_void, _c_int, _c_void],
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
@@ -596,8 +597,16 @@ def prefill_items(new_tokens, group_size: int) -> "list":
 
 def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                            query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
-                           items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None) -> None:
-    """Causal attention of the new rows of the sequences ``items`` names over their cached keys."""
+                           items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None,
+                           nsplit: int = 1, part_o: Optional[torch.Tensor] = None,
+                           part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None) -> None:
+    """Causal attention of the new rows of the sequences ``items`` names over their cached keys.
+
+    ``nsplit`` > 1 cuts every item's keys into that many shares (one workgroup each) for steps with few
+    items and long contexts; ``part_o`` / ``part_ml`` (float32, ``rows * H * nsplit * Dh`` and ``* 2``
+    with rows = all rows of the step) take the partial results and ``merge_rows`` lists the rows
+    that the items cover, which a second kernel then merges.
+    """
     _gpu(q, "queries")
     _gpu(out, "attention output")
     _gpu(k_cache, "k cache")
@@ -618,11 +627,32 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     _i32(items, "work items")
     if items.dim() != 2 or items.shape[1] != 2 or items.shape[0] == 0:
         raise InvalidArgument("work items must be a non-empty [n, 2] tensor")
+    num_merge = 0
+    if nsplit > 1:
+        _f32(part_o, "split accumulators")
+        _f32(part_ml, "split maxima and sums")
+        _i32(merge_rows, "rows to merge")
+        rows = q.shape[0]
+        num_merge = merge_rows.numel()
+        if part_o.numel() < rows * H * nsplit * Dh or part_ml.numel() < rows * H * nsplit * 2 or not 0 < num_merge <= 65535:
+            raise InvalidArgument("the buffers for the splits are too small, or no (or too many) rows to merge")
     lib = _lib("attention_prefill_bf16", Dh)
     _check(lib.tie_attention_prefill_bf16(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), _stream()), "attention_prefill_bf16")
+        block_tables.shape[1], float(scale), int(window or 0), int(nsplit), _ptr(part_o), _ptr(part_ml),
+        _ptr(merge_rows), num_merge, _stream()), "attention_prefill_bf16")
+
+
+def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:
+    """Shares the keys of every prefill item are cut into: more than one only where the items alone leave CUs idle."""
+    passes = -(-group_size // min(group_size, 4))
+    workgroups = num_items * num_kv_heads * passes
+    if workgroups >= 256 or num_rows > 65535:
+        return 1
+    by_fill = 512 // max(1, workgroups)
+    by_length = max(1, -(-max_context // 64) // 4)          # at least four 64-key tiles a share
+    return max(1, min(8, by_fill, by_length))
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
@@ -659,10 +689,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 single = []                                   # nothing but single rows and yet not a decode step
             taken = set(single)
             items = [it for it in prefill_items(new, G) if it[0] not in taken]
+            starts = [0]
+            for n in new:
+                starts.append(starts[-1] + n)
+            merge_rows = [starts[s] + r for s in sorted({it[0] for it in items}) for r in range(new[s])]
             work = batch.memo[key] = (
                 torch.tensor(single, dtype=torch.int32).to(q.device) if single else None, len(single),
-                torch.tensor(items, dtype=torch.int32).to(q.device) if items else None)
-        seq_ids, num_single, items = work
+                torch.tensor(items, dtype=torch.int32).to(q.device) if items else None, len(items),
+                torch.tensor(merge_rows, dtype=torch.int32).to(q.device) if items else None)
+        seq_ids, num_single, items, num_items, merge_rows = work
         if num_single:
             nsplit = decode_splits(num_single, KVH, batch.plan_context)
             part_o = part_ml = None
@@ -672,8 +707,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids)
         if items is not None:
+            rows = q.shape[0]
+            nsplit = prefill_splits(num_items, KVH, G, batch.plan_context, rows)
+            part_o = part_ml = None
+            if nsplit > 1:
+                part_o = scratch("attention.prefill_split_o", (rows * num_heads * nsplit * Dh,), torch.float32)
+                part_ml = scratch("attention.prefill_split_ml", (rows * num_heads * nsplit * 2,), torch.float32)
             attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens,
-                                   step.block_tables, items, num_heads, scale, window)
+                                   step.block_tables, items, num_heads, scale, window, nsplit, part_o, part_ml,
+                                   merge_rows if nsplit > 1 else None)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window)
