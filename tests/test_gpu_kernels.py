@@ -323,6 +323,60 @@ def test_gemm_bf16(M, N, K, tile):
     assert torch.equal(few, out[:3])
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 72, 96), (100, 384, 224), (300, 200, 4096), (2048, 256, 512), (257, 132, 1024),
+                                   (513, 516, 352), (1, 64, 128)])
+@pytest.mark.parametrize("tile", [4, 5])
+def test_gemm_bf16_loaded_straight_into_lds(M, N, K, tile):
+    """The tiles whose operand slices bypass registers: ragged M and N, short and long K, every epilogue."""
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=36, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=37, scale=0.1, dtype=torch.bfloat16).cuda()
+    want = plain.linear(x.cpu(), w.cpu())
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    kernels.gemm_bf16(x, w, out, tile=tile)
+    close(out, want, 1e-5, f"gemm {M}x{N}x{K} tile {tile}")
+    base = rnd(M, N, seed=38).cuda()
+    acc = base.clone()
+    kernels.gemm_bf16(x, w, acc, accumulate=True, tile=tile)
+    close(acc, want + base.cpu().to(F64), 1e-5, "gemm accumulate")
+    half = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    kernels.gemm_bf16(x, w, half, tile=tile)
+    close(half, want, 5e-3, "gemm bfloat16 output")
+    few = torch.empty(min(M, 3), N, dtype=torch.float32, device="cuda")
+    kernels.gemm_bf16(x[:3].contiguous(), w, few, tile=tile)
+    assert torch.equal(few, out[:3])                   # a row's result does not depend on the other rows
+    if K // 32 >= 6:
+        planes = torch.full((2, M, N), float("nan"), dtype=torch.float32, device="cuda")
+        kernels.gemm_bf16(x, w, planes, tile=tile, splits=2)
+        close(planes.cpu().to(F64).sum(0), want, 1e-5, "gemm in two planes")
+    if N % 16 == 0:
+        gate, up = w[: N // 2], w[N // 2:]
+        if (N // 2) % 8 == 0:
+            gated = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device="cuda")
+            kernels.gemm_bf16(x, kernels.interleave_gate_up(gate.contiguous(), up.contiguous()), gated, tile=tile, gated=True)
+            g, u = plain.linear(x.cpu(), gate.cpu()), plain.linear(x.cpu(), up.cpu())
+            close(gated, g / (1 + torch.exp(-g)) * u, 8e-3, "gated product")
+
+
+def test_gemm_bf16_straight_into_lds_refuses_what_it_cannot_take():
+    from tie_amd import kernels
+    from tie_amd.kernels import InvalidArgument
+
+    x = torch.zeros(8, 72, dtype=torch.bfloat16, device="cuda")          # K % 32 != 0
+    with pytest.raises(InvalidArgument):
+        kernels.gemm_bf16(x, torch.zeros(16, 72, dtype=torch.bfloat16, device="cuda"),
+                          torch.zeros(8, 16, device="cuda"), tile=4)
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")          # two slices only
+    with pytest.raises(InvalidArgument):
+        kernels.gemm_bf16(x, torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda"),
+                          torch.zeros(8, 16, device="cuda"), tile=5)
+    # left to choose, the same operands go to a kernel that takes them
+    out = torch.full((8, 16), float("nan"), device="cuda")
+    kernels.gemm_bf16(x, torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda"), out)
+    assert torch.equal(out, torch.zeros_like(out))
+
+
 @pytest.mark.parametrize("M,N,K,splits", [(65, 70, 1024, 2), (100, 384, 4096, 8), (300, 200, 1536, 3), (128, 128, 520, 2)])
 def test_gemm_bf16_in_planes(M, N, K, splits):
     """K cut into ranges: one plane of partial sums a range, which add up to the product."""
@@ -333,8 +387,10 @@ def test_gemm_bf16_in_planes(M, N, K, splits):
     planes = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device="cuda")
     kernels.gemm_bf16(x, w, planes, splits=splits)
     close(planes.cpu().to(F64).sum(0), plain.linear(x.cpu(), w.cpu()), 1e-5, f"gemm {M}x{N}x{K} in {splits} planes")
-    assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(512, 4096, 4096) == 2
+    assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(512, 4096, 4096) == 4
     assert kernels.gemm_splits(2048, 4096, 4096) == 1 and kernels.gemm_splits(128, 4096, 256) == 1
+    assert kernels.gemm_splits(2048, 4096, 12288) == 2 and kernels.gemm_splits(1024, 4096, 12288) == 4
+    assert kernels.gemm_splits(2048, 24576, 4096) == 1 and kernels.gemm_splits(300, 200, 1000) == 2
 
 
 def run_decode(case, S, H, Dh, nsplit, window=None):

@@ -21,6 +21,7 @@
 // contiguous band of the output and walks it column-tile by column-tile: the weights of a column
 // tile are fetched into that L2 once and reused by the row tiles.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
@@ -283,9 +284,292 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
   return tie_launch_status();
 }
 
-// Ranges of K that a product of M rows over w[N, K] is best cut into when its caller adds planes of
-// partial sums: few rows over a narrow weight give too few workgroups otherwise.
-extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
+// ---------------------------------------------------------------------------------------------
+// The same product with operand slices going global memory -> LDS directly (buffer loads with the
+// lds flag: no registers, no LDS write instructions), for K % 32 == 0 and N % 4 == 0.
+//
+// A workgroup of four waves (one per SIMD, 512 registers each) owns a 256 x BN tile, BN = 256 or 128; a wave owns
+// 128 x BN/2 of it, so that every byte read from LDS feeds twice the flops it does with the 64-wide
+// wave tiles above. k advances in slices of 32 through a ring of four LDS stages: while slice t is
+// multiplied, slices t+1 and t+2 are landing or landed and the loads of t+2 (its w rows) and t+3 (its x rows) are
+// issued, a few between the matrix instructions of each half slice so that neither the texture
+// path nor the in-order instruction stream of the one wave backs up. One barrier a slice: it sits
+// after the first half's matrix instructions, when the fragments of the second half are in
+// registers already, so that the stage is free and the next slice's first fragments can be read
+// while the second half multiplies.
+//
+// A staged row is 64 bytes, unpadded; 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 3), which
+// spreads the 32 rows a fragment read touches over the banks. The loads are bounds-checked by the
+// buffer descriptor: rows beyond M or N are not read (whatever the stage holds there lands in
+// output rows or columns that are never stored).
+//
+// The matrix instructions take w's fragment as their first operand: the tile comes out transposed,
+// a lane holding 4 consecutive columns of one output row, which it stores as one 8- or 16-byte piece.
+typedef __attribute__((ext_vector_type(4))) float floatx4_t;
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+#define GD_BM 256
+#define GD_BK 32
+#define GD_STAGES 4
+
+template <int BN, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x_all,
+                                                            const bf16_t* __restrict__ w_all,
+                                                            void* __restrict__ out_all, int M, int N, int K,
+                                                            int tiles_m, int tiles_n, int slices_per_split) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int BM = GD_BM, BK = GD_BK;
+  constexpr int TN = BN / 64;                   // 32-column MFMA tiles of a wave
+  constexpr int PB = BN / 64;                   // wave instructions that stage w's rows (16 rows each, 4 waves)
+  constexpr int BUF = (BM + BN) * BK;           // elements of one stage
+  extern __shared__ bf16_t lds[];
+
+  const int total = tiles_m * tiles_n;
+  int id = blockIdx.x;
+  {
+    const int per_xcd = (total + GB_XCDS - 1) / GB_XCDS;
+    const int remapped = (id % GB_XCDS) * per_xcd + id / GB_XCDS;
+    id = (total % GB_XCDS == 0) ? remapped : id;
+  }
+  const int tile_n = id / tiles_m;
+  const int tile_m = id % tiles_m;
+  const int row0 = tile_m * BM;
+  const int col0 = tile_n * BN;
+  const int k_begin = blockIdx.y * slices_per_split;                        // in slices
+  const int k_tiles = min(slices_per_split, K / BK - k_begin);
+  void* outp = EPI == 0 ? static_cast<void*>(static_cast<float*>(out_all) + static_cast<size_t>(blockIdx.y) * M * N)
+                        : out_all;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int fr = lane & 31;
+  const int fk = lane >> 5;
+
+  // One wave instruction fills 16 rows of 64 bytes: pass p of wave v covers rows 64 p + 16 v + lane / 4.
+  const int lr = wave * 16 + (lane >> 2);
+  const int lchunk = (lane & 3) ^ ((lr >> 1) & 3);
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2;
+  const unsigned loff = static_cast<unsigned>(lr) * row_bytes + lchunk * 16;
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(x_all + static_cast<size_t>(row0) * K + static_cast<size_t>(k_begin) * BK), 0,
+      static_cast<int>(min(BM, M - row0) * row_bytes - k_begin * BK * 2), 0x27000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(w_all + static_cast<size_t>(col0) * K + static_cast<size_t>(k_begin) * BK), 0,
+      static_cast<int>(min(BN, N - col0) * row_bytes - k_begin * BK * 2), 0x27000);
+  unsigned a_off[4], b_off[PB];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) a_off[p] = loff + p * 64 * row_bytes;
+#pragma unroll
+  for (int p = 0; p < PB; ++p) b_off[p] = loff + p * 64 * row_bytes;
+
+  auto stage = [&](int kt) { return lds + (kt & (GD_STAGES - 1)) * BUF; };
+  auto issue_x = [&](int kt) {
+    bf16_t* buf = stage(kt);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_void_t*)(buf + (p * 64 + wave * 16) * BK), 16, a_off[p],
+                                               kt * BK * 2, 0, 0);
+  };
+  auto issue_w = [&](int kt) {
+    bf16_t* buf = stage(kt);
+#pragma unroll
+    for (int p = 0; p < PB; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_void_t*)(buf + (BM + p * 64 + wave * 16) * BK), 16,
+                                               b_off[p], kt * BK * 2, 0, 0);
+  };
+
+  floatx16 acc[4][TN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int sw = (fr >> 1) & 3;
+  const int koff0 = ((0 + fk) ^ sw) * 8, koff1 = ((2 + fk) ^ sw) * 8;
+  const int a_row = (wm * 128 + fr) * BK;
+  const int b_row = (BM + wn * (BN / 2) + fr) * BK;
+
+  bf16x8_t fa[2][4], fb[2][TN];
+  auto load_frags = [&](const bf16_t* buf, int ks, int set) {
+    const int koff = ks ? koff1 : koff0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[set][i] = *reinterpret_cast<const bf16x8_t*>(buf + a_row + i * 32 * BK + koff);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[set][j] = *reinterpret_cast<const bf16x8_t*>(buf + b_row + j * 32 * BK + koff);
+  };
+  auto mfma_step = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+  };
+
+  // Slice j's x rows are issued after the barrier of slice j - 3 and its w rows before the barrier of
+  // slice j - 2; the first slices here. The host gives every range of K at least three slices.
+  issue_x(0);
+  issue_w(0);
+  issue_x(1);
+  issue_w(1);
+  issue_x(2);
+  if (PB == 4) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(10)\n\ts_barrier" ::: "memory");
+  load_frags(stage(0), 0, 0);
+
+  // One slice; its first fragments are in set 0 already. STEADY: slices up to kt + 3 exist, so the loads
+  // sit in straight-line code and exactly those of slice kt + 2 may still be in flight at the barrier.
+  auto slice = [&](int kt, auto steady_tag) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    load_frags(stage(kt), 1, 1);
+    if (STEADY || kt + 2 < k_tiles) issue_w(kt + 2);
+    mfma_step(0);
+    if (STEADY) {
+#pragma unroll
+      for (int q = 0; q < (4 + TN) / 2; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, TN / 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+#pragma unroll
+      for (int q = 0; q < PB; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // My share of slice kt + 1 has landed and my reads of this stage are in registers; after the
+    // barrier that holds for every wave.
+    if (STEADY) {
+      if (PB == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else if (kt + 2 < k_tiles) {
+      if (PB == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (STEADY || kt + 1 < k_tiles) load_frags(stage(kt + 1), 0, 0);
+    if (STEADY || kt + 3 < k_tiles) issue_x(kt + 3);
+    mfma_step(1);
+    if (STEADY) {
+#pragma unroll
+      for (int q = 0; q < (4 + TN) / 2; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, TN / 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int kt = 0;
+  for (; kt + 7 < k_tiles; kt += 4) {
+    slice(kt, std::true_type{});
+    slice(kt + 1, std::true_type{});
+    slice(kt + 2, std::true_type{});
+    slice(kt + 3, std::true_type{});
+  }
+  for (; kt < k_tiles; ++kt) slice(kt, std::false_type{});
+
+  const bool gated_n = EPI == 3;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = row0 + wm * 128 + i * 32 + fr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = col0 + wn * (BN / 2) + j * 32 + 8 * g + 4 * fk;
+        if (m >= M || n >= N) continue;
+        const float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2],
+                    v3 = acc[i][j][4 * g + 3];
+        if (gated_n) {
+          // Columns 16 b .. 16 b + 7 are gates and 16 b + 8 .. 16 b + 15 the ups of outputs 8 b .. 8 b + 7:
+          // register groups g and g + 1 of one lane.
+          if (g & 1) continue;
+          const float u0 = acc[i][j][4 * g + 4], u1 = acc[i][j][4 * g + 5], u2 = acc[i][j][4 * g + 6],
+                      u3 = acc[i][j][4 * g + 7];
+          const int out_col = (n >> 4) * 8 + 4 * fk;
+          uint2 pk;
+          pk.x = pack_bf16x2(v0 / (1.0f + __expf(-v0)) * u0, v1 / (1.0f + __expf(-v1)) * u1);
+          pk.y = pack_bf16x2(v2 / (1.0f + __expf(-v2)) * u2, v3 / (1.0f + __expf(-v3)) * u3);
+          *reinterpret_cast<uint2*>(static_cast<bf16_t*>(outp) + static_cast<size_t>(m) * (N / 2) + out_col) = pk;
+          continue;
+        }
+        const size_t o = static_cast<size_t>(m) * N + n;
+        if (EPI == 0) {
+          const floatx4_t r = {v0, v1, v2, v3};
+          *reinterpret_cast<floatx4_t*>(static_cast<float*>(outp) + o) = r;
+        } else if (EPI == 1) {
+          uint2 pk;
+          pk.x = pack_bf16x2(v0, v1);
+          pk.y = pack_bf16x2(v2, v3);
+          *reinterpret_cast<uint2*>(static_cast<bf16_t*>(outp) + o) = pk;
+        } else {
+          floatx4_t r = *reinterpret_cast<floatx4_t*>(static_cast<float*>(outp) + o);
+          r[0] += v0; r[1] += v1; r[2] += v2; r[3] += v3;
+          *reinterpret_cast<floatx4_t*>(static_cast<float*>(outp) + o) = r;
+        }
+      }
+    }
+  }
+#endif
+}
+
+template <int BN>
+static int launch_gemm_dma(const void* x, const void* w, void* out, int epi, int M, int N, int K, int splits,
+                           hipStream_t stream) {
+  const int tiles_m = (M + GD_BM - 1) / GD_BM, tiles_n = (N + BN - 1) / BN;
+  const int k_slices = K / GD_BK;
+  const int per_split = (k_slices + splits - 1) / splits;
+  if (k_slices - per_split * (splits - 1) < 3) return TIE_BAD_ARGUMENT;   // the last range would be too short
+  const size_t shared = sizeof(bf16_t) * GD_STAGES * (GD_BM + BN) * GD_BK;
+  const dim3 grid(tiles_m * tiles_n, splits);
+#define LAUNCH(EPI)                                                                                          \
+  {                                                                                                          \
+    static bool raised = false;                                                                              \
+    if (!raised) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_dma_kernel<BN, EPI>),      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared)); \
+      if (e != hipSuccess) return static_cast<int>(e);                                                       \
+      raised = true;                                                                                         \
+    }                                                                                                        \
+    gemm_bf16_dma_kernel<BN, EPI><<<grid, 256, shared, stream>>>(static_cast<const bf16_t*>(x),              \
+                                                                 static_cast<const bf16_t*>(w), out, M, N, K, \
+                                                                 tiles_m, tiles_n, per_split);               \
+  }
+  if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
+#undef LAUNCH
+  return tie_launch_status();
+}
+
+// Whether the direct-to-LDS kernel takes this product: whole slices of 32, at least three per range of K,
+// 16-byte aligned rows and 4-column output pieces, and row offsets within a tile that fit 32 bits.
+static bool gemm_dma_takes(const void* x, const void* w, const void* out, int N, int K, int splits) {
+  if (K % GD_BK != 0 || N % 4 != 0 || K > (1 << 22)) return false;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(w) % 16 ||
+      reinterpret_cast<uintptr_t>(out) % 16)
+    return false;
+  const int k_slices = K / GD_BK;
+  const int per_split = (k_slices + splits - 1) / splits;
+  return k_slices - per_split * (splits - 1) >= 3;
+}
+
+// Which tile, and how many ranges of K (planes of partial sums that the caller adds), a product takes when
+// left to choose. Measured on the four weight shapes of an 8B model for 128 to 2048 rows: the 256 x 256
+// tile wherever it gives most CUs a workgroup by itself; else enough ranges of K to get there - with
+// the 256 x 256 tile over a long K, with 256 x 128 over a short one, each range at least 1024 long;
+// few rows (one row tile, half empty) stay on the 128 x 128 tile with up to 8 ranges.
+struct GemmPlan { int tile, splits; };
+
+static int legacy_splits(int M, int N, int K) {
   const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
   if (tiles >= 256) return 1;
   const int k_slices = (K + 63) / 64;
@@ -299,12 +583,41 @@ extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
   return 1;
 }
 
+static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_split) {
+  const long rows256 = (M + 255) / 256;
+  const long t256 = rows256 * ((N + 255) / 256), t128 = rows256 * ((N + 127) / 128);
+  if (straight_to_lds && M >= 256) {
+    if (t256 >= 160) return {4, 1};
+    if (!may_split) return {t128 >= 128 ? 5 : 1, 1};
+    auto ranges = [&](long tiles, long want) {
+      for (int r = 1; r <= 8; r *= 2)
+        if (tiles * r >= want && K / r >= 1024) return r;
+      return 0;
+    };
+    const int r256 = ranges(t256, 160), r128 = ranges(t128, 192);
+    if (K >= 8192 && r256) return {4, r256};
+    if (r128) return {5, r128};
+    if (r256) return {4, r256};
+  }
+  if (may_split) return {1, legacy_splits(M, N, K)};
+  return {t256 >= 160 ? 2 : (t128 >= 192 ? 3 : 1), 1};
+}
+
+static bool straight_to_lds_shape(int N, int K) { return K % GD_BK == 0 && N % 4 == 0 && K <= (1 << 22) && K >= 3 * GD_BK; }
+
+// Ranges of K that a product of M rows over w[N, K] is best cut into when its caller adds planes of
+// partial sums: few rows over a narrow weight give too few workgroups otherwise.
+extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
+  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), true).splits;
+}
+
 // out_dtype: TIE_F32 or TIE_BF16; accumulate adds into a float32 output; gated (bfloat16 output of N / 2
 // columns, N % 16 == 0) applies silu(gate) * up to interleaved column blocks.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K
 // (128x128 tiles; neither accumulate nor gated).
 // tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
-//       3 = 256x128 (eight waves of 64x64).
+//       3 = 256x128 (eight waves of 64x64), 4 = 256x256 and 5 = 256x128 loaded straight into LDS (four
+//       waves of 128x128 or 128x64; K % 32 == 0, N % 4 == 0, 16-byte aligned operands, else refused).
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
                              int N, int K, int tile, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1) return TIE_BAD_ARGUMENT;
@@ -313,14 +626,23 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   if (gated && (accumulate || out_dtype != TIE_BF16 || N % 16 != 0)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
-  if (splits > 1) tile = 1;
-  if (tile == 0) {
-    // Larger tiles need fewer operand bytes per flop; take the largest that still gives most CUs a tile.
-    const long rows256 = (M + 255) / 256;
-    if (rows256 * ((N + 255) / 256) >= 160) tile = 2;
-    else if (rows256 * ((N + 127) / 128) >= 192) tile = 3;
-    else tile = 1;
+  if (tile == 4 || tile == 5) {
+    if (!gemm_dma_takes(x, w, out, N, K, splits)) return TIE_BAD_ARGUMENT;
+    return tile == 4 ? launch_gemm_dma<256>(x, w, out, epi, M, N, K, splits, stream)
+                     : launch_gemm_dma<128>(x, w, out, epi, M, N, K, splits, stream);
   }
+  if (tile == 0) {
+    const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
+    if (splits > 1) {
+      const GemmPlan plan = gemm_plan(M, N, K, straight, true);
+      tile = plan.splits == splits ? plan.tile : 1;
+    } else {
+      tile = gemm_plan(M, N, K, straight, false).tile;
+    }
+    if (tile == 4) return launch_gemm_dma<256>(x, w, out, epi, M, N, K, splits, stream);
+    if (tile == 5) return launch_gemm_dma<128>(x, w, out, epi, M, N, K, splits, stream);
+  }
+  if (splits > 1) tile = 1;
   if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, splits, stream);
   if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, splits, stream);
   return launch_gemm<128, 128, 64, 2, 2>(x, w, out, epi, M, N, K, splits, stream);
