@@ -359,6 +359,60 @@ def test_gemm_bf16_loaded_straight_into_lds(M, N, K, tile):
             close(gated, g / (1 + torch.exp(-g)) * u, 8e-3, "gated product")
 
 
+@pytest.mark.parametrize("N,K", [(16, 96), (48, 128), (208, 4096), (1024, 352)])
+def test_packed_weight_feeds_both_products_the_same_numbers(N, K):
+    """The blocked weight layout changes where bytes lie, not one sum: results equal the row-major ones bit for bit."""
+    from tie_amd import kernels
+
+    w = rnd(N, K, seed=51, scale=0.1, dtype=torch.bfloat16).cuda()
+    packed = kernels.pack_weight(w)
+    assert packed.shape == (N, K) and torch.equal(packed.unpacked(), w)
+    # block (t, b): rows 16 t.., k 32 b..; the 8 elements of (row r, chunk c) at (16 c + r) * 8
+    blocks = packed.blocks.view(-1)
+    t, b, r, c = N // 16 - 1, K // 32 - 1, 5, 2
+    at = ((t * (K // 32) + b) * 64 + 16 * c + r) * 8
+    assert torch.equal(blocks[at:at + 8], w[16 * t + r, 32 * b + 8 * c:32 * b + 8 * c + 8])
+    for M in (1, 8, 40, 64):
+        x = rnd(M, K, seed=52 + M, dtype=torch.bfloat16).cuda()
+        for splits in (1, 2):
+            shape = (M, N) if splits == 1 else (splits, M, N)
+            a = torch.full(shape, float("nan"), dtype=torch.float32, device="cuda")
+            b_ = torch.full(shape, float("nan"), dtype=torch.float32, device="cuda")
+            kernels.skinny_gemm_bf16(x, w, a, splits=splits)
+            kernels.skinny_gemm_bf16(x, packed, b_, splits=splits)
+            assert torch.equal(a, b_), f"decode product M={M} splits={splits}"
+        if N % 16 == 0:
+            a = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device="cuda")
+            b_ = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device="cuda")
+            kernels.skinny_gemm_bf16(x, w, a, gated=True)
+            kernels.skinny_gemm_bf16(x, packed, b_, gated=True)
+            assert torch.equal(a, b_)
+    for M in (65, 300, 513):
+        x = rnd(M, K, seed=60 + M, dtype=torch.bfloat16).cuda()
+        want = plain.linear(x.cpu(), w.cpu())
+        for tile in (4, 5):
+            a = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            b_ = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            kernels.gemm_bf16(x, w, a, tile=tile)
+            kernels.gemm_bf16(x, packed, b_, tile=tile)
+            assert torch.equal(a, b_), f"tiled product M={M} tile={tile}"
+            close(b_, want, 1e-5, "tiled product over a packed weight")
+        out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        kernels.linear(x, packed, out)                       # left to choose
+        close(out, want, 1e-5, "linear over a packed weight")
+        s = kernels.gemm_splits(M, N, K, packed=True)
+        if s > 1:
+            planes = torch.full((s, M, N), float("nan"), dtype=torch.float32, device="cuda")
+            kernels.gemm_bf16(x, packed, planes, splits=s)
+            close(planes.cpu().to(F64).sum(0), want, 1e-5, f"packed weight in {s} planes")
+    with pytest.raises(kernels.InvalidArgument):
+        kernels.gemm_bf16(rnd(65, K, seed=1, dtype=torch.bfloat16).cuda(), packed,
+                          torch.zeros(65, N, device="cuda"), tile=1)          # only tiles 4 and 5 read the layout
+    with pytest.raises(kernels.InvalidArgument):
+        kernels.linear(torch.zeros(2, K, device="cuda"), packed, torch.zeros(2, N, device="cuda"))   # float32 input
+    assert not kernels.packable(w[:, :64].contiguous()) and not kernels.packable(w.float())
+
+
 def test_gemm_bf16_straight_into_lds_refuses_what_it_cannot_take():
     from tie_amd import kernels
     from tie_amd.kernels import InvalidArgument

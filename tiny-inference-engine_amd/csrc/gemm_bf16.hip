@@ -312,7 +312,7 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 #define GD_BK 32
 #define GD_STAGES 4
 
-template <int BN, int EPI>
+template <int BN, int EPI, bool PW>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x_all,
                                                             const bf16_t* __restrict__ w_all,
                                                             void* __restrict__ out_all, int M, int N, int K,
@@ -347,21 +347,32 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   const int fk = lane >> 5;
 
   // One wave instruction fills 16 rows of 64 bytes: pass p of wave v covers rows 64 p + 16 v + lane / 4.
+  // Rows beyond the matrix are clamped to its last one (their products are never stored).
   const int lr = wave * 16 + (lane >> 2);
   const int lchunk = (lane & 3) ^ ((lr >> 1) & 3);
   const unsigned row_bytes = static_cast<unsigned>(K) * 2;
-  const unsigned loff = static_cast<unsigned>(lr) * row_bytes + lchunk * 16;
+  const int kblocks = K / BK;
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<bf16_t*>(x_all + static_cast<size_t>(row0) * K + static_cast<size_t>(k_begin) * BK), 0,
       static_cast<int>(min(BM, M - row0) * row_bytes - k_begin * BK * 2), 0x27000);
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<bf16_t*>(w_all + static_cast<size_t>(col0) * K + static_cast<size_t>(k_begin) * BK), 0,
-      static_cast<int>(min(BN, N - col0) * row_bytes - k_begin * BK * 2), 0x27000);
   unsigned a_off[4], b_off[PB];
 #pragma unroll
-  for (int p = 0; p < 4; ++p) a_off[p] = loff + p * 64 * row_bytes;
+  for (int p = 0; p < 4; ++p) a_off[p] = min(lr + p * 64, M - 1 - row0) * row_bytes + lchunk * 16;
+  // w: rows like x's, or (PW) the packed layout, where the 16 rows x 32 k that one wave instruction
+  // stages are one block of 1 KB: block (tile, k-block) at ((tile * kblocks) + k-block) * 1 KB.
+  const int tile0 = col0 / 16, last_tile = (N - 1) / 16;
+  const bf16_t* b_base = PW ? w_all + (static_cast<size_t>(tile0) * kblocks + k_begin) * 512
+                            : w_all + static_cast<size_t>(col0) * K + static_cast<size_t>(k_begin) * BK;
+  const unsigned b_bytes = PW ? static_cast<unsigned>(min(BN / 16, last_tile + 1 - tile0)) * kblocks * 1024 - k_begin * 1024
+                              : min(BN, N - col0) * row_bytes - k_begin * BK * 2;
+  const __amdgpu_buffer_rsrc_t b_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(b_base), 0, static_cast<int>(b_bytes), 0x27000);
+  unsigned b_tile_off[PB];   // PW: wave-uniform byte offset of this wave's block row
 #pragma unroll
-  for (int p = 0; p < PB; ++p) b_off[p] = loff + p * 64 * row_bytes;
+  for (int p = 0; p < PB; ++p) {
+    b_off[p] = PW ? lane * 16 : min(lr + p * 64, N - 1 - col0) * row_bytes + lchunk * 16;
+    b_tile_off[p] = PW ? static_cast<unsigned>(min(p * 4 + wave, last_tile - tile0)) * kblocks * 1024 : 0;
+  }
 
   auto stage = [&](int kt) { return lds + (kt & (GD_STAGES - 1)) * BUF; };
   auto issue_x = [&](int kt) {
@@ -376,7 +387,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #pragma unroll
     for (int p = 0; p < PB; ++p)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_void_t*)(buf + (BM + p * 64 + wave * 16) * BK), 16,
-                                               b_off[p], kt * BK * 2, 0, 0);
+                                               b_off[p], PW ? b_tile_off[p] + kt * 1024 : kt * BK * 2, 0, 0);
   };
 
   floatx16 acc[4][TN];
@@ -387,18 +398,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+  // Fragment addresses. x's stage rows are swizzled (above); w's are too unless packed, where the
+  // 16-byte piece of (row r of block t, k-chunk c) sits at t * 1 KB + (16 c + r) * 16 bytes: the 16 lanes
+  // that one LDS cycle serves read 256 consecutive bytes.
   const int sw = (fr >> 1) & 3;
   const int koff0 = ((0 + fk) ^ sw) * 8, koff1 = ((2 + fk) ^ sw) * 8;
   const int a_row = (wm * 128 + fr) * BK;
-  const int b_row = (BM + wn * (BN / 2) + fr) * BK;
+  const int b_row = PW ? BM * BK + (wn * (BN / 32) + (fr >> 4)) * 512 + (fr & 15) * 8
+                       : (BM + wn * (BN / 2) + fr) * BK;
 
   bf16x8_t fa[2][4], fb[2][TN];
   auto load_frags = [&](const bf16_t* buf, int ks, int set) {
     const int koff = ks ? koff1 : koff0;
+    const int koff_w = PW ? (ks * 2 + fk) * 128 : koff;
 #pragma unroll
     for (int i = 0; i < 4; ++i) fa[set][i] = *reinterpret_cast<const bf16x8_t*>(buf + a_row + i * 32 * BK + koff);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[set][j] = *reinterpret_cast<const bf16x8_t*>(buf + b_row + j * 32 * BK + koff);
+    for (int j = 0; j < TN; ++j) fb[set][j] = *reinterpret_cast<const bf16x8_t*>(buf + b_row + j * 32 * BK + koff_w);
   };
   auto mfma_step = [&](int set) {
 #pragma unroll
@@ -523,7 +539,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #endif
 }
 
-template <int BN>
+template <int BN, bool PW>
 static int launch_gemm_dma(const void* x, const void* w, void* out, int epi, int M, int N, int K, int splits,
                            hipStream_t stream) {
   const int tiles_m = (M + GD_BM - 1) / GD_BM, tiles_n = (N + BN - 1) / BN;
@@ -536,14 +552,13 @@ static int launch_gemm_dma(const void* x, const void* w, void* out, int epi, int
   {                                                                                                          \
     static bool raised = false;                                                                              \
     if (!raised) {                                                                                           \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_dma_kernel<BN, EPI>),      \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_dma_kernel<BN, EPI, PW>),      \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared)); \
       if (e != hipSuccess) return static_cast<int>(e);                                                       \
       raised = true;                                                                                         \
     }                                                                                                        \
-    gemm_bf16_dma_kernel<BN, EPI><<<grid, 256, shared, stream>>>(static_cast<const bf16_t*>(x),              \
-                                                                 static_cast<const bf16_t*>(w), out, M, N, K, \
-                                                                 tiles_m, tiles_n, per_split);               \
+    gemm_bf16_dma_kernel<BN, EPI, PW><<<grid, 256, shared, stream>>>(                                        \
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n, per_split); \
   }
   if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
 #undef LAUNCH
@@ -583,21 +598,30 @@ static int legacy_splits(int M, int N, int K) {
   return 1;
 }
 
-static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_split) {
+static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_split, bool packed) {
   const long rows256 = (M + 255) / 256;
   const long t256 = rows256 * ((N + 255) / 256), t128 = rows256 * ((N + 127) / 128);
+  auto ranges = [&](long tiles, long want, int shortest) {
+    for (int r = 1; r <= 8; r *= 2)
+      if (tiles * r >= want && K / r >= shortest) return r;
+    return 0;
+  };
   if (straight_to_lds && M >= 256) {
     if (t256 >= 160) return {4, 1};
-    if (!may_split) return {t128 >= 128 ? 5 : 1, 1};
-    auto ranges = [&](long tiles, long want) {
-      for (int r = 1; r <= 8; r *= 2)
-        if (tiles * r >= want && K / r >= 1024) return r;
-      return 0;
-    };
-    const int r256 = ranges(t256, 160), r128 = ranges(t128, 192);
+    if (!may_split) return {t128 >= 128 || packed ? 5 : 1, 1};
+    const int r256 = ranges(t256, 160, 1024), r128 = ranges(t128, 192, 1024);
     if (K >= 8192 && r256) return {4, r256};
     if (r128) return {5, r128};
     if (r256) return {4, r256};
+  }
+  if (packed) {
+    // Only the tiles that load straight into LDS read the packed layout: 256 x 128, with as many
+    // ranges of K (512 or longer) as it takes to give most CUs a workgroup, at most 8.
+    if (!may_split) return {5, 1};
+    int r = ranges(t128, 192, 512);
+    if (r == 0)
+      for (r = 8; r > 1 && K / r < 512; r /= 2) {}
+    return {5, r};
   }
   if (may_split) return {1, legacy_splits(M, N, K)};
   return {t256 >= 160 ? 2 : (t128 >= 192 ? 3 : 1), 1};
@@ -607,8 +631,9 @@ static bool straight_to_lds_shape(int N, int K) { return K % GD_BK == 0 && N % 4
 
 // Ranges of K that a product of M rows over w[N, K] is best cut into when its caller adds planes of
 // partial sums: few rows over a narrow weight give too few workgroups otherwise.
-extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
-  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), true).splits;
+extern "C" int tie_gemm_bf16_splits(int M, int N, int K, int packed) {
+  if (packed && !straight_to_lds_shape(N, K)) return 1;
+  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), true, packed != 0).splits;
 }
 
 // out_dtype: TIE_F32 or TIE_BF16; accumulate adds into a float32 output; gated (bfloat16 output of N / 2
@@ -618,31 +643,36 @@ extern "C" int tie_gemm_bf16_splits(int M, int N, int K) {
 // tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
 //       3 = 256x128 (eight waves of 64x64), 4 = 256x256 and 5 = 256x128 loaded straight into LDS (four
 //       waves of 128x128 or 128x64; K % 32 == 0, N % 4 == 0, 16-byte aligned operands, else refused).
+// packed: w is stored in blocks of 16 rows x 32 k, 1 KB each, in the matrix cores' operand order (as the
+//       decode product reads it); N % 16 == 0, and only tiles 4 and 5 read it.
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
-                             int N, int K, int tile, int splits, hipStream_t stream) {
+                             int N, int K, int tile, int splits, int packed, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1) return TIE_BAD_ARGUMENT;
   if (accumulate && out_dtype != TIE_F32) return TIE_BAD_ARGUMENT;
   if (out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || out_dtype != TIE_BF16 || N % 16 != 0)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
-  if (tile == 4 || tile == 5) {
-    if (!gemm_dma_takes(x, w, out, N, K, splits)) return TIE_BAD_ARGUMENT;
-    return tile == 4 ? launch_gemm_dma<256>(x, w, out, epi, M, N, K, splits, stream)
-                     : launch_gemm_dma<128>(x, w, out, epi, M, N, K, splits, stream);
-  }
+  const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
+  if (packed && (N % 16 != 0 || !straight || (tile != 0 && tile != 4 && tile != 5))) return TIE_BAD_ARGUMENT;
   if (tile == 0) {
-    const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
     if (splits > 1) {
-      const GemmPlan plan = gemm_plan(M, N, K, straight, true);
-      tile = plan.splits == splits ? plan.tile : 1;
+      const GemmPlan plan = gemm_plan(M, N, K, straight, true, packed != 0);
+      tile = plan.splits == splits ? plan.tile : (packed ? 5 : 1);
     } else {
-      tile = gemm_plan(M, N, K, straight, false).tile;
+      tile = gemm_plan(M, N, K, straight, false, packed != 0).tile;
     }
-    if (tile == 4) return launch_gemm_dma<256>(x, w, out, epi, M, N, K, splits, stream);
-    if (tile == 5) return launch_gemm_dma<128>(x, w, out, epi, M, N, K, splits, stream);
+  } else if (tile < 4 && splits > 1) {
+    tile = 1;
   }
-  if (splits > 1) tile = 1;
+  if (tile == 4 || tile == 5) {
+    if (!straight) return TIE_BAD_ARGUMENT;
+    if (tile == 4)
+      return packed ? launch_gemm_dma<256, true>(x, w, out, epi, M, N, K, splits, stream)
+                    : launch_gemm_dma<256, false>(x, w, out, epi, M, N, K, splits, stream);
+    return packed ? launch_gemm_dma<128, true>(x, w, out, epi, M, N, K, splits, stream)
+                  : launch_gemm_dma<128, false>(x, w, out, epi, M, N, K, splits, stream);
+  }
   if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, splits, stream);
   if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, splits, stream);
   return launch_gemm<128, 128, 64, 2, 2>(x, w, out, epi, M, N, K, splits, stream);

@@ -17,6 +17,12 @@
 // the same order whatever else is in the batch.
 //
 // Requires K % 8 == 0 (16-byte loads); other shapes go to the generic kernel.
+//
+// PACKED: w is stored as [N/16][K/32] blocks of 1 KB, block (t, b) holding rows 16 t .. 16 t + 15 over
+// k = 32 b .. 32 b + 31 in the order the matrix core takes them: lane l's 16 bytes (row l % 16, k-chunk
+// l / 16) at byte 16 l. A wave's load is then 1 KB of consecutive memory and its stream through K one
+// contiguous run, which the memory system serves measurably faster than 16 rows' 64-byte pieces
+// (6.1 against 5.1 TB/s on a 201 MB weight); read once, the stream is loaded non-temporally.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -29,13 +35,24 @@ __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
+typedef __attribute__((ext_vector_type(4))) unsigned int sk_u32x4_t;
+
+template <bool PACKED>
+__device__ __forceinline__ bf16x8_t load_weight_frag(const bf16_t* p) {
+  if (PACKED) {
+    const sk_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const sk_u32x4_t*>(p));
+    return *reinterpret_cast<const bf16x8_t*>(&v);
+  }
+  return load_frag(p);
+}
+
 __device__ __forceinline__ bf16x8_t zero_frag() {
   const uint4 v = make_uint4(0, 0, 0, 0);
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
 // MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 loaded ahead of the MFMAs.
-template <int MT, int RT, int U, typename TO>
+template <int MT, int RT, int U, typename TO, bool PACKED>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
@@ -47,10 +64,15 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   const int g = lane >> 4;   // which 8-element chunk of the 32-wide k block
   const int n0 = blockIdx.x * 16 * RT;
 
-  // Rows beyond N are clamped for the loads; their columns are dropped at the store.
+  // Rows beyond N are clamped for the loads; their columns are dropped at the store. wp[t] points at
+  // this lane's 16 bytes of k-block 0; a k-block further on is KB_STRIDE elements further on.
+  constexpr int KB_STRIDE = PACKED ? 512 : 32;
   const bf16_t* wp[RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t) wp[t] = w + static_cast<size_t>(min(n0 + t * 16 + r, N - 1)) * K;
+  for (int t = 0; t < RT; ++t) {
+    if (PACKED) wp[t] = w + static_cast<size_t>(min(n0 / 16 + t, (N - 1) / 16)) * (K / 32) * 512 + lane * 8;
+    else wp[t] = w + static_cast<size_t>(min(n0 + t * 16 + r, N - 1)) * K + g * 8;
+  }
   const bf16_t* xp[MT];
   bool xvalid[MT];
 #pragma unroll
@@ -80,7 +102,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     for (int u = 0; u < U; ++u) {
       const int k = (kb + u) * 32 + g * 8;
 #pragma unroll
-      for (int t = 0; t < RT; ++t) b[t][u] = load_frag(wp[t] + k);
+      for (int t = 0; t < RT; ++t) b[t][u] = load_weight_frag<PACKED>(wp[t] + static_cast<size_t>(kb + u) * KB_STRIDE);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) a[mt][u] = xvalid[mt] ? load_frag(xp[mt] + k) : zero_frag();
     }
@@ -101,7 +123,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     for (int mt = 0; mt < MT; ++mt) a[mt] = (kvalid && xvalid[mt]) ? load_frag(xp[mt] + k) : zero_frag();
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-      const bf16x8_t b = kvalid ? load_frag(wp[t] + k) : zero_frag();
+      const bf16x8_t b = kvalid ? load_weight_frag<PACKED>(wp[t] + static_cast<size_t>(kb) * KB_STRIDE) : zero_frag();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], b, acc[mt][t], 0, 0, 0);
     }
@@ -182,9 +204,11 @@ extern "C" int tie_skinny_gemm_splits(int N, int K) { return (N < 8192 && K >= 5
 // gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
 // and receives silu(gate) * up.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
+// packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
 extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
-                                    int M, int N, int K, int splits, hipStream_t stream) {
+                                    int M, int N, int K, int splits, int packed, hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1 || splits > 64) return TIE_BAD_ARGUMENT;
+  if (packed && (N % 16 != 0 || K % 32 != 0)) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || N % 16 != 0 || splits != 1)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
@@ -192,14 +216,19 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
   const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
   const int kblocks = (K + 31) / 32;
   const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
-#define LAUNCH(MT, RT, U, TO)                                                                                \
-  skinny_gemm_kernel<MT, RT, U, TO><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                                \
+#define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
+  skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                             \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
       gated, per_wave)
+#define LAUNCH(MT, RT, U, TO)                  \
+  {                                            \
+    if (packed) LAUNCH_P(MT, RT, U, TO, true); \
+    else LAUNCH_P(MT, RT, U, TO, false);       \
+  }
 #define LAUNCH_RT(MT, TO)                                  \
-  if (rt == 1) LAUNCH(MT, 1, 4, TO);                       \
-  else if (rt == 2) LAUNCH(MT, 2, 4, TO);                  \
-  else if (rt == 3) LAUNCH(MT, 3, 2, TO);                  \
+  if (rt == 1) LAUNCH(MT, 1, 4, TO)                        \
+  else if (rt == 2) LAUNCH(MT, 2, 4, TO)                   \
+  else if (rt == 3) LAUNCH(MT, 3, 2, TO)                   \
   else LAUNCH(MT, 4, 2, TO)
 #define LAUNCH_MT(TO)                                      \
   if (mt == 1) { LAUNCH_RT(1, TO); }                       \
@@ -211,5 +240,6 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
 #undef LAUNCH_MT
 #undef LAUNCH_RT
 #undef LAUNCH
+#undef LAUNCH_P
   return tie_launch_status();
 }

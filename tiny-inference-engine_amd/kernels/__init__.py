@@ -64,12 +64,12 @@ _SIGNATURES = {
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                 _c_void],
+                                 _c_int, _c_void],
     },
     "gemm_bf16": {
-        "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int],
+        "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
         "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                          _c_void],
+                          _c_int, _c_void],
     },
     "attention_prefill_bf16": {
         "tie_attention_prefill_rows_per_item": [_c_int],
@@ -284,9 +284,55 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate
         _code(out, "matmul output"), int(accumulate), T, N, K, _stream()), "gemm_generic")
 
 
+class PackedWeight:
+    """A bfloat16 ``[N, K]`` weight stored as ``[N/16][K/32]`` blocks of 1 KB in the matrix cores' operand order.
+
+    Block (t, b) holds rows 16 t .. 16 t + 15 over k = 32 b .. 32 b + 31; within it the 8 elements of
+    (row r, k-chunk c) lie at element (16 c + r) * 8. A wave of the decode product then loads 1 KB of
+    consecutive memory per matrix instruction and walks K as one contiguous run, and the tiled product
+    stages one block per load. Built once at load time by ``pack_weight``; only the bfloat16 products
+    read it (``N % 16 == 0`` and ``K % 32 == 0``).
+    """
+
+    __slots__ = ("blocks", "shape")
+    dtype = torch.bfloat16
+
+    def __init__(self, blocks: torch.Tensor, shape):
+        self.blocks = blocks
+        self.shape = tuple(shape)
+
+    def data_ptr(self) -> int:
+        return self.blocks.data_ptr()
+
+    @property
+    def device(self):
+        return self.blocks.device
+
+    def unpacked(self) -> torch.Tensor:
+        """The ``[N, K]`` row-major matrix again (a copy)."""
+        N, K = self.shape
+        return self.blocks.view(N // 16, K // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(N, K).contiguous()
+
+
+def packable(w) -> bool:
+    """Whether ``pack_weight`` takes this matrix: bfloat16, on the GPU, rows in steps of 16 and K in steps of 32."""
+    return isinstance(w, torch.Tensor) and w.is_cuda and w.dim() == 2 and w.dtype == torch.bfloat16 and \
+        w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0 and w.shape[1] >= 96
+
+
+def pack_weight(w: torch.Tensor) -> PackedWeight:
+    """The matrix in the blocked layout of ``PackedWeight`` (a copy; the row-major tensor can be dropped)."""
+    if not packable(w):
+        raise InvalidArgument(f"pack_weight takes a bfloat16 GPU matrix [N % 16 == 0, K % 32 == 0, K >= 96], got "
+                              f"{list(w.shape)} {w.dtype}")
+    N, K = w.shape
+    blocks = w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+    return PackedWeight(blocks, (N, K))
+
+
 def _bf16_product_operands(x, w, out, gated, what):
     _gpu(x, "matmul input")
-    _gpu(w, "matmul weight")
+    _gpu(w.blocks if isinstance(w, PackedWeight) else w, "matmul weight")
     _gpu(out, "matmul output")
     M, K = x.shape
     N, K2 = w.shape
@@ -328,12 +374,12 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
         raise InvalidArgument("a gated product does not accumulate")
     _check(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16(
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
-        int(splits), _stream()), "skinny_gemm_bf16")
+        int(splits), int(isinstance(w, PackedWeight)), _stream()), "skinny_gemm_bf16")
 
 
-def gemm_splits(M: int, N: int, K: int) -> int:
+def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
     """Ranges of K a product of M > 64 rows over a ``[N, K]`` weight is best cut into when its caller adds partial sums."""
-    return int(_lib("gemm_bf16").tie_gemm_bf16_splits(M, N, K))
+    return int(_lib("gemm_bf16").tie_gemm_bf16_splits(M, N, K, int(packed)))
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0,
@@ -354,7 +400,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     if accumulate and (gated or out.dtype != torch.float32):
         raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only, and not in a gated product")
     _check(_lib("gemm_bf16").tie_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
-                                           int(accumulate), int(gated), M, N, K, tile, int(splits), _stream()),
+                                           int(accumulate), int(gated), M, N, K, tile, int(splits),
+                                           int(isinstance(w, PackedWeight)), _stream()),
            "gemm_bf16")
 
 
@@ -374,14 +421,17 @@ def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tenso
         gemm_bf16(x, w_interleaved, out, gated=True)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out (+)= x @ w.T, on the fastest kernel that takes these operands."""
+def linear(x: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out (+)= x @ w.T, on the fastest kernel that takes these operands (w a matrix or a ``PackedWeight``)."""
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and \
             not (accumulate and out.dtype != torch.float32):
         if x.shape[0] <= 64:
             skinny_gemm_bf16(x, w, out, accumulate)
         else:
             gemm_bf16(x, w, out, accumulate)
+    elif isinstance(w, PackedWeight):
+        raise InvalidArgument(f"a packed weight is read by the bfloat16 products only: input {x.dtype}, output "
+                              f"{out.dtype}, accumulate={accumulate}")
     else:
         gemm_generic(x, w, out, accumulate)
 

@@ -40,7 +40,7 @@ class SwiGLU(FeedForward):
         self.fused = gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and \
             self.intermediate % 8 == 0 and self.hidden % 8 == 0
         if self.fused:
-            self.gate_up.weight = kernels.interleave_gate_up(gate, up)
+            self.gate_up.set_weight(kernels.interleave_gate_up(gate, up))
         else:
             self.gate_up.load(fetch)
 

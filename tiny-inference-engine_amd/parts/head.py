@@ -40,7 +40,9 @@ class LmHead(Head):
         return [TensorSpec(self.weight_name, shape, "matrix", ("normal", 0.02))]
 
     def load(self, fetch, mode, device) -> None:
-        self.weight = fetch(self.tied_to or self.weight_name, "matrix")
+        w = fetch(self.tied_to or self.weight_name, "matrix")
+        # The blocked copy is the head's own: a tied embedding table keeps its rows for the gather.
+        self.weight = kernels.pack_weight(w) if kernels.packable(w) else w
 
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
         last = self.norm.forward(ctx, x, rows=rows, out_name="head.norm")

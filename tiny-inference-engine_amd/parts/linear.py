@@ -41,12 +41,16 @@ class Linear:
     def load(self, fetch) -> None:
         parts = [fetch(n, "matrix") for n in self.names]
         if len(parts) == 1:
-            self.weight = parts[0]
+            self.set_weight(parts[0])
             return
         dtypes = {p.dtype for p in parts}
         if len(dtypes) > 1:  # stored in different widths: the wider one decides
             parts = [p.to(torch.float32) for p in parts]
-        self.weight = torch.cat(parts, dim=0).contiguous()
+        self.set_weight(torch.cat(parts, dim=0).contiguous())
+
+    def set_weight(self, w: torch.Tensor) -> None:
+        """Keeps ``w`` (``[out, in]``), in the matrix cores' blocked layout where the bfloat16 products can read that."""
+        self.weight = kernels.pack_weight(w) if kernels.packable(w) else w
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ctx=None) -> torch.Tensor:
         """out (+)= x @ W^T. With ``ctx`` an accumulating product may leave its addition owed to ``out``.
@@ -80,7 +84,7 @@ class Linear:
         else:
             splits = self._tiled_splits.get(M)
             if splits is None:
-                splits = self._tiled_splits[M] = kernels.gemm_splits(M, w.shape[0], K)
+                splits = self._tiled_splits[M] = kernels.gemm_splits(M, w.shape[0], K, isinstance(w, kernels.PackedWeight))
         if splits <= 1:
             return None
         planes = ctx.scratch(name, (splits, M, w.shape[0]), torch.float32)
