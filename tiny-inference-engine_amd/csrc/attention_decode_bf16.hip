@@ -117,7 +117,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st) {
         const int d = st * 32 + quad * 8;
-        kf[u][st] = d < DH ? *reinterpret_cast<const u32x4_t*>(kr + d) : u32x4_t{0, 0, 0, 0};
+        kf[u][st] = d < DH ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kr + d)) : u32x4_t{0, 0, 0, 0};
       }
     }
   };
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     for (int dt = 0; dt < DTILES; ++dt) {
       const size_t d_off = static_cast<size_t>(dt * 16 + col) * block_size;
       if (WIDE) {
-        vf[dt] = *reinterpret_cast<const u32x4_t*>(vp[0] + d_off);
+        vf[dt] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vp[0] + d_off));
       } else {
         const u32x2_t h0 = *reinterpret_cast<const u32x2_t*>(vp[0] + d_off);
         const u32x2_t h1 = *reinterpret_cast<const u32x2_t*>(vp[WIDE ? 0 : 1] + d_off);
