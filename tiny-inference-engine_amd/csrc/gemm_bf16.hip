@@ -1,6 +1,11 @@
 // The prefill-time matrix product for gfx950: out[M, N] (+)= x[M, K] . w[N, K]^T with bfloat16
 // operands and float32 accumulation on v_mfma_f32_32x32x16_bf16.
 //
+// Two kernels. The one described first stages operand slices through registers and takes every shape
+// with K % 8 == 0; the second (further down, gemm_bf16_dma_kernel) loads them from global memory
+// straight into LDS, needs K % 32 == 0 and N % 4 == 0, also reads weights in packed blocks, and is
+// the one the prefill step runs on. gemm_plan picks between their tiles.
+//
 // Both operands are K-contiguous, which is the order the matrix cores consume: a lane's fragment
 // is 8 consecutive k of one row (16 bytes). A workgroup of four or eight waves owns a BM x BN tile of
 // the output; k advances in slices of BK (32 or 64). Each slice of x and w goes global memory -> registers ->
@@ -299,9 +304,11 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
 // while the second half multiplies.
 //
 // A staged row is 64 bytes, unpadded; 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 3), which
-// spreads the 32 rows a fragment read touches over the banks. The loads are bounds-checked by the
-// buffer descriptor: rows beyond M or N are not read (whatever the stage holds there lands in
-// output rows or columns that are never stored).
+// spreads the 32 rows a fragment read touches over the banks. Rows beyond M or N are clamped to the
+// last row (their products land in output rows or columns that are never stored). With PW the weight
+// comes in packed blocks of 16 rows x 32 k (1 KB in the matrix cores' operand order, as the decode
+// product reads it): one load instruction stages one block, and the 16 lanes that LDS serves in a
+// cycle read 256 consecutive bytes of it.
 //
 // The matrix instructions take w's fragment as their first operand: the tile comes out transposed,
 // a lane holding 4 consecutive columns of one output row, which it stores as one 8- or 16-byte piece.
