@@ -147,6 +147,31 @@ def test_recorded_decode_steps_replay_to_the_eager_result(folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_more_sequences_decode_together_than_the_decode_product_takes(folders, dtype):
+    """Eighty requests decode side by side: above 64 rows a step's products run on the tiled kernels
+    (over packed weights, in ranges of K), also inside the recorded graphs that later steps replay."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders[dtype]["B"]
+    requests = th.make_requests(cfg["vocab_size"], [9 + i % 7 for i in range(80)], seed=77)
+    want = reference_logits(folder, cfg, requests)
+    tail = 6
+    steps = []
+    ids = list(requests)
+    for at in range(0, len(ids), 16):                     # prompts, sixteen requests a step
+        steps.append({"step": len(steps), "end": [], "entries": [
+            {"id": r, "tokens": requests[r][:-tail], "want": list(range(len(requests[r]) - tail))} for r in ids[at:at + 16]]})
+    for t in range(tail, 0, -1):                          # then one token each, all eighty together
+        steps.append({"step": len(steps), "end": ids if t == 1 else [], "entries": [
+            {"id": r, "tokens": [requests[r][-t]], "want": [0]} for r in ids]})
+    replayer = TraceReplayer.from_folder(folder, dtype, 80 * 64, block_size=16)
+    got = th.collect(replayer, steps)
+    check(got, want, dtype, f"B/{dtype}/eighty together")
+    if dtype == "bfloat16":
+        assert replayer.runner.graph_replays >= tail - 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """A short prompt, then every further token one by one, up to the model's context."""
     from tie_amd.engine.replay import TraceReplayer
