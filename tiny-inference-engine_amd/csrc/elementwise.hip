@@ -373,6 +373,118 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   }
 }
 
+// The same for head sizes of 32, 64, 128, 256 or 512: a lane takes 4 consecutive elements of a head's
+// first half and the 4 they pair with in the second (16-byte loads and stores where the old kernel's were
+// 4 and 2 bytes), head_dim / 8 lanes share a head, four waves of heads a workgroup. The sums of squares
+// meet by shuffles inside the lanes of a head.
+typedef __attribute__((ext_vector_type(4))) float qk_f4_t;
+
+template <typename T>
+__device__ __forceinline__ qk_f4_t load4(const T* p);
+template <>
+__device__ __forceinline__ qk_f4_t load4<float>(const float* p) { return *reinterpret_cast<const qk_f4_t*>(p); }
+template <>
+__device__ __forceinline__ qk_f4_t load4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return qk_f4_t{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                 __uint_as_float(v.y & 0xffff0000u)};
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, qk_f4_t v);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, qk_f4_t v) { *reinterpret_cast<qk_f4_t*>(p) = v; }
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, qk_f4_t v) {
+  uint2 o;
+  o.x = pack_bf16x2(v[0], v[1]);
+  o.y = pack_bf16x2(v[2], v[3]);
+  *reinterpret_cast<uint2*>(p) = o;
+}
+
+template <typename TX>
+__device__ __forceinline__ qk_f4_t load4_planes(const TX* p, size_t plane_stride, int planes) {
+  qk_f4_t v = load4(p);
+  if (planes == 2) return v + load4(p + plane_stride);
+  for (int s = 1; s < planes; ++s) v += load4(p + static_cast<size_t>(s) * plane_stride);
+  return v;
+}
+
+#define QK4_THREADS 256
+
+template <typename TX, typename TQ, typename TC, int LPH>   // LPH: lanes per head = head_dim / 8
+__global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
+    const TX* qkv, TQ* q_out, const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
+    const float* __restrict__ inv_freq, const float* __restrict__ angles, const int* __restrict__ positions,
+    const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H, int KVH,
+    int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads) {
+  constexpr int Dh = LPH * 8, half = LPH * 4;
+  const int t = blockIdx.y;
+  const int slot_index = blockIdx.x * (QK4_THREADS / LPH) + threadIdx.x / LPH;
+  const int p0 = (threadIdx.x % LPH) * 4;
+  if (slot_index >= heads) return;             // whole heads leave: the shuffles below stay inside a head
+  const TX* in = qkv + static_cast<size_t>(t) * in_row + static_cast<size_t>(slot_index) * Dh;
+  const bool is_q = slot_index < H;
+  const bool is_k = !is_q && slot_index < H + KVH;
+  if (!is_q && !is_k) {
+    // Value head: into the cache, transposed inside the page. Neighbouring lanes take neighbouring
+    // dimensions, which lie block_size elements apart there: the closest the stores of one token get.
+    const int slot = slots[t];
+    TC* dst = v_cache + (static_cast<size_t>(slot / block_size) * KVH + (slot_index - H - KVH)) * Dh * block_size +
+              slot % block_size;
+    const int sub = threadIdx.x % LPH;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = load_planes(in + sub + LPH * i, plane_stride, planes);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_from_float(dst + static_cast<size_t>(sub + LPH * i) * block_size, v[i]);
+    return;
+  }
+  qk_f4_t a = load4_planes(in + p0, plane_stride, planes);
+  qk_f4_t b = load4_planes(in + half + p0, plane_stride, planes);
+
+  const float* w = is_q ? q_w : k_w;
+  if (w != nullptr) {
+    float ss = (a[0] * a[0] + b[0] * b[0]) + (a[1] * a[1] + b[1] * b[1]) + (a[2] * a[2] + b[2] * b[2]) +
+               (a[3] * a[3] + b[3] * b[3]);
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, TIE_WAVE);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(Dh) + eps);
+    a = (a * inv) * load4(w + p0);
+    b = (b * inv) * load4(w + half + p0);
+  }
+  qk_f4_t o1 = a, o2 = b;
+  if (angles != nullptr) {
+    const qk_f4_t cs = load4(angles + static_cast<size_t>(t) * Dh + p0);
+    const qk_f4_t sn = load4(angles + static_cast<size_t>(t) * Dh + half + p0);
+    o1 = a * cs - b * sn;
+    o2 = b * cs + a * sn;
+  } else if (inv_freq != nullptr) {
+    const float pos = static_cast<float>(positions[t]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float sn, cs;
+      sincosf(pos * inv_freq[p0 + i], &sn, &cs);
+      o1[i] = a[i] * cs - b[i] * sn;
+      o2[i] = b[i] * cs + a[i] * sn;
+    }
+  }
+  if (is_q) {
+    TQ* dst = q_out + static_cast<size_t>(t) * q_row + static_cast<size_t>(slot_index) * Dh;
+    store4(dst + p0, o1);
+    store4(dst + half + p0, o2);
+  } else if (k_dense != nullptr) {
+    TQ* dst = k_dense + static_cast<size_t>(t) * k_row + static_cast<size_t>(slot_index - H) * Dh;
+    store4(dst + p0, o1);
+    store4(dst + half + p0, o2);
+  } else {
+    const int slot = slots[t];
+    TC* dst = k_cache + ((static_cast<size_t>(slot / block_size) * KVH + (slot_index - H)) * block_size +
+                         slot % block_size) * Dh;
+    store4(dst + p0, o1);
+    store4(dst + half + p0, o2);
+  }
+}
+
 // angles[t, 0:Dh/2] = cos(float(positions[t]) * inv_freq[i]), angles[t, Dh/2:Dh] = sin of the same: what
 // the kernel below would compute per head and layer, once per step instead.
 __global__ void rope_angles_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
@@ -409,6 +521,38 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
     return TIE_BAD_ARGUMENT;
   const int heads = H + ((write_kv || k_dense != nullptr) ? KVH : 0) + (write_kv ? KVH : 0);
   if (in_row < heads * Dh || (k_dense != nullptr && k_row < KVH * Dh)) return TIE_BAD_ARGUMENT;
+  // Head sizes of 32 .. 512 in powers of two, and rows that keep 16-byte pieces aligned: the 4-wide kernel.
+  const bool wide = (Dh == 32 || Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) && in_row % 4 == 0 &&
+                    q_row % 4 == 0 && k_row % 4 == 0 && plane_stride % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(k_dense) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(angles) % 16 == 0 && reinterpret_cast<uintptr_t>(q_w) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(k_w) % 16 == 0;
+  if (wide) {
+    const int lph = Dh / 8;
+    const dim3 grid4((heads + QK4_THREADS / lph - 1) / (QK4_THREADS / lph), T);
+#define LAUNCH4_L(TX, TQ, TC, LPH)                                                                            \
+  qk_norm_rope_kv_write4_kernel<TX, TQ, TC, LPH><<<grid4, QK4_THREADS, 0, stream>>>(                          \
+      static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
+      static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, block_size,   \
+      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads)
+#define LAUNCH4(TX, TQ, TC)                         \
+  {                                                 \
+    if (lph == 4) LAUNCH4_L(TX, TQ, TC, 4);         \
+    else if (lph == 8) LAUNCH4_L(TX, TQ, TC, 8);    \
+    else if (lph == 16) LAUNCH4_L(TX, TQ, TC, 16);  \
+    else if (lph == 32) LAUNCH4_L(TX, TQ, TC, 32);  \
+    else LAUNCH4_L(TX, TQ, TC, 64);                 \
+  }
+    if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH4(float, float, float)
+    else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH4(float, bf16_t, bf16_t)
+    else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH4(bf16_t, bf16_t, bf16_t)
+    else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_BF16) LAUNCH4(float, float, bf16_t)
+    else return TIE_BAD_ARGUMENT;
+#undef LAUNCH4
+#undef LAUNCH4_L
+    return tie_launch_status();
+  }
   const dim3 grid(heads, T);
 #define LAUNCH(TX, TQ, TC)                                                                                   \
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
