@@ -530,6 +530,18 @@ def test_attention_prefill_bf16_long_portions(H, KVH, Dh, bs, nsplit):
     close(out, case["want"], 1e-2, f"prefill attention, long portions, H={H} KVH={KVH} Dh={Dh} bs={bs} splits={nsplit}")
 
 
+def test_prefill_items_cover_the_rows_the_kernel_takes_per_item():
+    """The item list is built on the host, the rows an item covers are the kernel's: the two must agree, or
+    items overlap (and with key shares two workgroups then write one row's partial results)."""
+    from tie_amd import kernels
+
+    lib = kernels._lib("attention_prefill_bf16", 64)
+    for group in (1, 2, 3, 4, 5, 8, 16):
+        rows = int(lib.tie_attention_prefill_rows_per_item(group))
+        items = kernels.prefill_items([rows * 2 + 5], group)
+        assert [first for _, first in items] == [0, rows, 2 * rows], f"group of {group}"
+
+
 @pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "tile_edge_64", "far", "last"])
 def test_attention_prefill_bf16_finds_one_far_key(where):
     spike = {"first": lambda ctx: 0, "page_edge": lambda ctx: 16 * 3 - 1, "tile_edge": lambda ctx: 32 * 7,
