@@ -318,6 +318,9 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 #define GD_BM 256
 #define GD_BK 32
 #define GD_STAGES 4
+// Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
+// selects x, y, z, w; no swizzle, no stride (the compiler's own default for raw buffers on this target).
+#define GD_RSRC_FLAGS 0x27000
 
 template <int BN, int EPI, bool PW>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x_all,
@@ -361,7 +364,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   const int kblocks = K / BK;
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<bf16_t*>(x_all + static_cast<size_t>(row0) * K + static_cast<size_t>(k_begin) * BK), 0,
-      static_cast<int>(min(BM, M - row0) * row_bytes - k_begin * BK * 2), 0x27000);
+      static_cast<int>(min(BM, M - row0) * row_bytes - k_begin * BK * 2), GD_RSRC_FLAGS);
   unsigned a_off[4], b_off[PB];
 #pragma unroll
   for (int p = 0; p < 4; ++p) a_off[p] = min(lr + p * 64, M - 1 - row0) * row_bytes + lchunk * 16;
@@ -373,7 +376,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   const unsigned b_bytes = PW ? static_cast<unsigned>(min(BN / 16, last_tile + 1 - tile0)) * kblocks * 1024 - k_begin * 1024
                               : min(BN, N - col0) * row_bytes - k_begin * BK * 2;
   const __amdgpu_buffer_rsrc_t b_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(b_base), 0, static_cast<int>(b_bytes), 0x27000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(b_base), 0, static_cast<int>(b_bytes), GD_RSRC_FLAGS);
   unsigned b_tile_off[PB];   // PW: wave-uniform byte offset of this wave's block row
 #pragma unroll
   for (int p = 0; p < PB; ++p) {
