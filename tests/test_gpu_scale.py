@@ -40,6 +40,17 @@ def test_serving_widths_bfloat16_against_float32():
         torch.cuda.empty_cache()
         return got
 
+    # one prompt of the size the prefill is measured at, ragged against every tile (2100 = 8 x 256 + 52 rows):
+    # a few of its positions are compared, the last among them
+    long_prompt = th.make_requests(WIDE["vocab_size"], [2100], seed=4)["r0"]
+    long_steps = [{"step": 0, "entries": [{"id": "long", "tokens": long_prompt, "want": [0, 255, 256, 1023, 2047, 2099]}],
+                   "end": ["long"]}]
+    want_long = run("float32", long_steps, th.round64(2100))["long"]
+    got_long = run("bfloat16", long_steps, th.round64(2100))["long"]
+    for position, ref in want_long.items():
+        err = float((got_long[position] - ref).abs().max() / ref.abs().max())
+        assert torch.isfinite(got_long[position]).all() and err < 3e-2, f"long prompt, position {position}: {err:.3e}"
+
     biggest = max(th.round64(len(t)) for t in requests.values())
     want = run("float32", th.whole(requests), biggest)
     steps, peak = th.mixed(requests, max_live=4, seed=5, tail=40)     # long runs of decoded tokens, portions beside them
