@@ -315,9 +315,13 @@ class PackedWeight:
 
 
 def packable(w) -> bool:
-    """Whether ``pack_weight`` takes this matrix: bfloat16, on the GPU, rows in steps of 16 and K in steps of 32."""
+    """Whether ``pack_weight`` takes this matrix: bfloat16, on the GPU, rows in steps of 16 and K in steps of 32.
+
+    K between 96 and 2^22 is what the tiled product's packed path takes (at least three slices of 32; the
+    row offsets of a tile within 32 bits).
+    """
     return isinstance(w, torch.Tensor) and w.is_cuda and w.dim() == 2 and w.dtype == torch.bfloat16 and \
-        w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0 and w.shape[1] >= 96
+        w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0 and 96 <= w.shape[1] <= (1 << 22)
 
 
 def pack_weight(w: torch.Tensor) -> PackedWeight:
