@@ -215,8 +215,9 @@ def test_run_orders_shared_caches_and_windows(tmp_path, order, window, dtype, to
 
 # ------------------------------------------------------------------ toy parts, defined and registered here
 def register_toy_parts():
+    from tie_amd import kernels
     from tie_amd.cache.spec import FixedState
-    from tie_amd.parts import Mixer, Position, TensorSpec, register_part
+    from tie_amd.parts import FeedForward, Mixer, Position, TensorSpec, register_part
 
     @register_part("mixer", "toy_decay")
     class ToyDecayMixer(Mixer):
@@ -246,6 +247,45 @@ def register_toy_parts():
                     state.mul_(self.decay).add_(u[t])
                     residual[t] += state @ self.w_out.float().T
                 row += n
+
+    @register_part("feed_forward", "toy_routed")
+    class ToyRoutedFeedForward(FeedForward):
+        """Router logits in float32, the top k experts per token, softmax over the chosen, ReLU experts."""
+
+        def __init__(self, params):
+            super().__init__(params)
+            self.hidden, self.width = params["hidden"], params["width"]
+            self.experts, self.top_k, self.names = params["experts"], params["top_k"], params["names"]
+
+        def tensors(self):
+            specs = [TensorSpec(self.names["router"], (self.experts, self.hidden), "matrix", ("normal", 0.5))]
+            for e in range(self.experts):                      # expert weights: ordinary tensors with an index in the name
+                specs.append(TensorSpec(self.names["w1"].format(e=e), (self.width, self.hidden), "matrix", ("normal", 0.2)))
+                specs.append(TensorSpec(self.names["w2"].format(e=e), (self.hidden, self.width), "matrix", ("normal", 0.2)))
+            return specs
+
+        def load(self, fetch, mode, device):
+            self.router = fetch(self.names["router"], "matrix")
+            self.w1 = [fetch(self.names["w1"].format(e=e), "matrix") for e in range(self.experts)]
+            self.w2 = [fetch(self.names["w2"].format(e=e), "matrix") for e in range(self.experts)]
+
+        def forward(self, ctx, h, residual):
+            T = h.shape[0]
+            logits = ctx.scratch("toy_routed.logits", (T, self.experts), torch.float32)
+            kernels.linear(h, self.router, logits)                                  # the framework's own product
+            top, chosen = torch.topk(logits, self.top_k, dim=1)
+            gate = torch.softmax(top, dim=1)
+            for e in range(self.experts):
+                rows, slot = (chosen == e).nonzero(as_tuple=True)
+                if rows.numel() == 0:
+                    continue
+                x = h[rows].contiguous()
+                mid = torch.empty(rows.numel(), self.width, dtype=h.dtype, device=h.device)
+                kernels.linear(x, self.w1[e], mid)
+                mid.clamp_(min=0)
+                out = torch.empty(rows.numel(), self.hidden, dtype=torch.float32, device=h.device)
+                kernels.linear(mid, self.w2[e], out)
+                residual.index_add_(0, rows, out * gate[rows, slot][:, None])
 
     @register_part("position", "toy_shift")
     class ToyShiftPosition(Position):
@@ -279,8 +319,14 @@ def toy_spec(cfg):
                 "scale": cfg["head_dim"] ** -0.5, "window": None, "qk_norm": None,
                 "position": PartSpec("toy_shift", {"slope": cfg["slope"]}),
                 "names": {"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}})
-        ffn = PartSpec("swiglu", {"hidden": D, "intermediate": cfg["intermediate"],
-                                  "names": {"gate": p + "gate", "up": p + "up", "down": p + "down"}})
+        if cfg["feed_forwards"][l] == "routed":
+            ffn = PartSpec("toy_routed", {"hidden": D, "width": cfg["expert_width"], "experts": cfg["experts"],
+                                          "top_k": cfg["top_k"],
+                                          "names": {"router": p + "router", "w1": p + "experts.{e}.w1",
+                                                    "w2": p + "experts.{e}.w2"}})
+        else:
+            ffn = PartSpec("swiglu", {"hidden": D, "intermediate": cfg["intermediate"],
+                                      "names": {"gate": p + "gate", "up": p + "up", "down": p + "down"}})
         layers.append(LayerSpec(PartSpec("pre_norm"), mixer, ffn,
                                 {"pre_mixer": norm(p + "n1"), "pre_feed_forward": norm(p + "n2")}))
     return ModelSpec("ToyStateLM", cfg["vocab_size"], D, cfg["max_positions"],
@@ -315,7 +361,19 @@ def toy_plain(weights, cfg, tokens):
             a = plain.causal_attention(q, k, v, Dh ** -0.5).reshape(T, H * Dh)
             x = x + plain.linear(a, weights[p + "o"])
         h = plain.rms_norm(x, weights[p + "n2"], cfg["eps"])
-        x = x + plain.swiglu(h, weights[p + "gate"], weights[p + "up"], weights[p + "down"])
+        if cfg["feed_forwards"][l] == "routed":
+            logits = plain.linear(h, weights[p + "router"])
+            top, chosen = torch.topk(logits, cfg["top_k"], dim=1)
+            gate = torch.softmax(top, dim=1)
+            out = torch.zeros_like(x)
+            for t in range(T):
+                for j in range(cfg["top_k"]):
+                    e = int(chosen[t, j])
+                    mid = plain.linear(h[t:t + 1], weights[p + f"experts.{e}.w1"]).clamp(min=0)
+                    out[t] += gate[t, j] * plain.linear(mid, weights[p + f"experts.{e}.w2"])[0]
+            x = x + out
+        else:
+            x = x + plain.swiglu(h, weights[p + "gate"], weights[p + "up"], weights[p + "down"])
     return plain.linear(plain.rms_norm(x, weights["final_norm"], cfg["eps"]), weights["embed"])
 
 
@@ -331,7 +389,8 @@ def test_a_toy_architecture_registered_from_outside_runs_through_the_step_functi
     try:
         cfg = {"architectures": ["ToyStateLM"], "vocab_size": 90, "hidden_size": 48, "intermediate": 72,
                "heads": 3, "kv_heads": 1, "head_dim": 16, "state_width": 20, "decay": 0.8, "slope": 0.01,
-               "eps": 1e-5, "max_positions": 256, "mixers": ["decay", "attention", "decay"]}
+               "eps": 1e-5, "max_positions": 256, "mixers": ["decay", "attention", "decay"],
+               "feed_forwards": ["dense", "routed", "routed"], "experts": 5, "top_k": 2, "expert_width": 24}
         folder = write_random_model(tmp_path / "toy", cfg, seed=4, dtype="float32")   # the parts' TensorSpecs drive it
         replayer = TraceReplayer.from_folder(folder, "float32", 192, block_size=4)    # config.json names the class
         plan = replayer.model.cache_plan
@@ -357,4 +416,5 @@ def test_a_toy_architecture_registered_from_outside_runs_through_the_step_functi
     finally:
         unregister_architecture("ToyStateLM")
         unregister_part("mixer", "toy_decay")
+        unregister_part("feed_forward", "toy_routed")
         unregister_part("position", "toy_shift")
