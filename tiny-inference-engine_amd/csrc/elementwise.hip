@@ -3,8 +3,12 @@
 // sampling kernels (argmax, temperature). All arithmetic is float32; only
 // loads and stores convert. One C entry point per operation.
 #include "common.h"
+#include "argmax_static.h"
 
 #include <math.h>
+#include <stdio.h>
+
+#include <mutex>
 
 // ---------------------------------------------------------------- embedding
 // out[t, :] = float(table[ids[t], :]). Reference: src/backend/cpu/cpu_backend.cpp:51-76.
@@ -656,6 +660,47 @@ extern "C" int tie_argmax(const float* logits, int* out, float* max_out, float* 
   if (status != TIE_OK) return status;
   argmax_final_kernel<<<R, TIE_WAVE, 0, stream>>>(part_v, part_i, out, max_out);
   return tie_launch_status();
+}
+
+// The same two stages with the candidates in a file-scope array instead of a caller's workspace,
+// for callers that cannot allocate (declared and described in argmax_static.h). In host code the
+// array's name is only a stand-in: its address on a device comes from hipGetSymbolAddress, once per
+// device with that device current, and that pointer is what the kernels receive.
+// The array carries no `used` attribute: its use by host code below is what makes the compiler export
+// the device symbol, which the runtime looks up by name; marked `used` it stays a local symbol and
+// loading the library aborts.
+#define ARGMAX_STATIC_DEVICES 64
+static __device__ __align__(256) unsigned char argmax_static_scratch[TIE_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS *
+                                                                      (sizeof(float) + sizeof(int))];
+static void* argmax_static_ptr[ARGMAX_STATIC_DEVICES];   // per device: where its copy of the array lies
+static std::mutex argmax_static_mutex;
+
+extern "C" int tie_argmax_static(const float* logits, int* out, float* max_out, int R, int V, hipStream_t stream) {
+  if (R <= 0 || V <= 0 || logits == nullptr || out == nullptr) return TIE_BAD_ARGUMENT;
+  if (R > TIE_ARGMAX_STATIC_MAX_ROWS) {
+    fprintf(stderr, "tie_argmax_static: %d rows exceed the %d rows its static scratch array holds\n", R,
+            TIE_ARGMAX_STATIC_MAX_ROWS);
+    return TIE_EXCEEDS_STATIC_SCRATCH;
+  }
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (device < 0 || device >= ARGMAX_STATIC_DEVICES) return TIE_BAD_ARGUMENT;
+  void* base;
+  {
+    std::lock_guard<std::mutex> lock(argmax_static_mutex);
+    if (argmax_static_ptr[device] == nullptr) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_static_scratch));
+      if (e != hipSuccess) return static_cast<int>(e);
+      if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+      argmax_static_ptr[device] = p;
+    }
+    base = argmax_static_ptr[device];
+  }
+  float* part_v = static_cast<float*>(base);
+  int* part_i = reinterpret_cast<int*>(part_v + static_cast<size_t>(TIE_ARGMAX_STATIC_MAX_ROWS) * ARGMAX_CHUNKS);
+  return tie_argmax(logits, out, max_out, part_v, part_i, R, V, stream);
 }
 
 // ------------------------------------------------------ temperature sampling

@@ -51,6 +51,7 @@ _SIGNATURES = {
                                       _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_argmax_static": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
         "tie_gemm_generic": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -569,6 +570,28 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor, max_out: Optional[torch
                                        torch.empty(rows * 64, dtype=torch.int32, device=logits.device))
     _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), _ptr(max_out), ws[0].data_ptr(),
                                           ws[1].data_ptr(), R, V, _stream()), "argmax")
+
+
+ARGMAX_STATIC_MAX_ROWS = 1024     # TIE_ARGMAX_STATIC_MAX_ROWS of csrc/argmax_static.h
+
+
+def argmax_rows_static(logits: torch.Tensor, out: torch.Tensor, max_out: Optional[torch.Tensor] = None) -> None:
+    """``argmax_rows`` without any allocation: the candidates between its two stages live in a static device array.
+
+    For callers that cannot allocate (stream capture, loops that must stay off the allocator). At most
+    ``ARGMAX_STATIC_MAX_ROWS`` rows; calls that may overlap on one GPU race on the shared array.
+    """
+    _f32(logits, "logits")
+    R, V = logits.shape
+    _i32(out, "argmax output", R)
+    if max_out is not None:
+        _f32(max_out, "row maxima", (R,))
+    if R > ARGMAX_STATIC_MAX_ROWS:
+        raise InvalidArgument(f"argmax_rows_static takes at most {ARGMAX_STATIC_MAX_ROWS} rows (the size of its static "
+                              f"scratch array), got {R}")
+    with torch.cuda.device(logits.device):
+        _check(_lib("elementwise").tie_argmax_static(logits.data_ptr(), out.data_ptr(), _ptr(max_out), R, V,
+                                                     _stream()), "argmax_static")
 
 
 def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
