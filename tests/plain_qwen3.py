@@ -95,6 +95,29 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     return out
 
 
+def causal_attention_tail(q_tail: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                          window: Optional[int] = None) -> torch.Tensor:
+    """The last ``n`` rows of ``causal_attention`` when only their queries are at hand.
+
+    q_tail [n, H, Dh] are the queries at positions T-n .. T-1 of a sequence whose keys and values
+    k, v [T, KVH, Dh] are all given: the same formula (src/backend/cpu/cpu_backend.cpp:261-319), without
+    the T x T score matrix, so that a context of tens of thousands of keys stays affordable.
+    """
+    q_tail, k, v = q_tail.to(F64), k.to(F64), v.to(F64)
+    n, H, Dh = q_tail.shape
+    T, KVH = k.shape[0], k.shape[1]
+    group = H // KVH
+    out = torch.zeros_like(q_tail)
+    for r in range(n):
+        pos = T - n + r
+        first = 0 if window is None else max(0, pos - window + 1)
+        for h in range(H):
+            kvh = h // group
+            scores = scale * (k[first:pos + 1, kvh, :] @ q_tail[r, h, :])
+            out[r, h, :] = torch.softmax(scores, dim=0) @ v[first:pos + 1, kvh, :]
+    return out
+
+
 def swiglu(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
     """down(gate / (1 + exp(-gate)) * up). src/model/qwen3.cpp:235-238; src/backend/cpu/cpu_backend.cpp:195-207."""
     g = linear(h, w_gate)

@@ -153,6 +153,59 @@ def test_qk_norm_rope_kv_write(H, KVH, Dh, bs):
                                   Dh, bs, planes=3, plane_stride=planes.stride(0))
     assert torch.equal(q1, q3) and torch.equal(kc1, kc3) and torch.equal(vc1, vc3)
 
+def rotate_pairs(x, positions, inv_freq, rotary_dim, pairing):
+    """The first ``rotary_dim`` dimensions of x [T, heads, Dh] rotated as pairs (i, i + rotary_dim/2)
+    ("rotate_half") or (2i, 2i + 1) ("interleaved") by position * inv_freq[i]; the rest unchanged."""
+    x = x.to(F64)
+    out = x.clone()
+    half = rotary_dim // 2
+    angle = torch.tensor(positions, dtype=torch.float32)[:, None] * inv_freq[None, :]      # float32 angles
+    cos, sin = torch.cos(angle.to(F64))[:, None, :], torch.sin(angle.to(F64))[:, None, :]
+    if pairing == "rotate_half":
+        a, b = x[..., :half], x[..., half:rotary_dim]
+        out[..., :half], out[..., half:rotary_dim] = a * cos - b * sin, b * cos + a * sin
+    else:
+        a, b = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+        out[..., 0:rotary_dim:2], out[..., 1:rotary_dim:2] = a * cos - b * sin, b * cos + a * sin
+    return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,rotary_dim,bs", [(4, 2, 16, 8, 4), (6, 2, 32, 32, 16), (3, 1, 48, 20, 8),
+                                                    (8, 2, 128, 64, 16), (2, 1, 256, 0, 4), (2, 2, 80, 78, 2)])
+@pytest.mark.parametrize("pairing", ["rotate_half", "interleaved"])
+def test_qk_norm_rope_rotates_part_of_a_head_and_neighbouring_pairs(H, KVH, Dh, rotary_dim, bs, pairing):
+    """What the position interface may return beside Qwen3's whole-head halves: a rotation of the first
+    rotary_dim dimensions only, and pairs of neighbours; with and without the per-step table of angles."""
+    from tie_amd import kernels
+
+    T, eps = 5, 1e-5
+    qkv = rnd(T, (H + 2 * KVH) * Dh, seed=18, scale=2.0).cuda()
+    qw, kw = (1 + 0.1 * rnd(Dh, seed=19)).cuda(), (1 + 0.1 * rnd(Dh, seed=20)).cuda()
+    positions, slots = [0, 3, 77, 300, 4095], [9, 2, 31, 4, 17]
+    inv_freq = torch.from_numpy(plain.rope_inv_freq(1e4, max(rotary_dim, 2)))[:rotary_dim // 2].contiguous()
+    NB = 32 // bs + 1
+    x = qkv.cpu()
+    q_in = x[:, :H * Dh].view(T, H, Dh)
+    k_in = x[:, H * Dh:(H + KVH) * Dh].view(T, KVH, Dh)
+    q_want = rotate_pairs(plain.rms_norm(q_in, qw.cpu(), eps), positions, inv_freq, rotary_dim, pairing)
+    k_want = rotate_pairs(plain.rms_norm(k_in, kw.cpu(), eps), positions, inv_freq, rotary_dim, pairing)
+    if rotary_dim == Dh and pairing == "rotate_half":
+        close(q_want, plain.rope_neox(plain.rms_norm(q_in, qw.cpu(), eps), positions, 1e4), 1e-12, "the test's own rotation")
+    table = None
+    if rotary_dim:
+        table = torch.empty(T, rotary_dim, device="cuda")
+        kernels.rope_angles(i32(positions), inv_freq.cuda(), table)
+    for angles in (None, table):
+        kc = torch.zeros(NB, KVH, bs, Dh, device="cuda")
+        vc = torch.zeros(NB, KVH, Dh, bs, device="cuda")
+        q = torch.empty(T, H * Dh, device="cuda")
+        kernels.qk_norm_rope_kv_write(qkv, q, qw, kw, eps, inv_freq.cuda() if rotary_dim else None, i32(positions),
+                                      i32(slots), kc, vc, H, KVH, Dh, bs, angles=angles, rotary_dim=rotary_dim,
+                                      pairing=pairing)
+        close(q.view(T, H, Dh), q_want, 2e-6, f"q, rotary_dim {rotary_dim}, {pairing}")
+        for t, slot in enumerate(slots):
+            close(kc[slot // bs, :, slot % bs], k_want[t], 2e-6, f"k of token {t}, rotary_dim {rotary_dim}, {pairing}")
+
 
 def attention_case(H, KVH, Dh, bs, lens_new, lens_ctx, seed, dtype=torch.float32, window=None, spike=None):
     """Builds a batch of sequences with scattered, unordered block tables; returns kernel inputs and the plain result."""
@@ -488,6 +541,68 @@ def test_attention_decode_bf16_window_edges(window):
     for nsplit in (1, 4):
         out = run_decode(case, S, 4, 32, nsplit, window=window)
         close(out, case["want"], 1e-2, f"decode window {window} splits {nsplit}")
+
+
+def long_decode_case(H, KVH, Dh, bs, lens_ctx, seed, spike_back):
+    """Decode rows over long contexts (vectorised filling, the plain result for the last row only).
+
+    Key ``ctx - spike_back`` of every sequence is made to stand out for the last query, with a value of 5
+    in every dimension: a share of keys that is dropped, read twice or merged with a wrong weight shows."""
+    rng = np.random.RandomState(seed)
+    S = len(lens_ctx)
+    MB = max(math.ceil(c / bs) for c in lens_ctx) + 1
+    NB = sum(math.ceil(c / bs) for c in lens_ctx) + 3
+    pages = torch.from_numpy(rng.permutation(NB).astype(np.int64))
+    kc = torch.full((NB, KVH, bs, Dh), 1e30, dtype=torch.bfloat16)          # unused slots hold garbage
+    vc = torch.full((NB, KVH, Dh, bs), 1e30, dtype=torch.bfloat16)
+    tables = np.zeros((S, MB), dtype=np.int32)
+    q_rows, want_rows, used = [], [], 0
+    for s, ctx in enumerate(lens_ctx):
+        q = rnd(1, H, Dh, seed=seed * 100 + s)
+        k = rnd(ctx, KVH, Dh, seed=seed * 100 + s + 50)
+        v = rnd(ctx, KVH, Dh, seed=seed * 100 + s + 70)
+        j = ctx - spike_back
+        k[j] = 0
+        k[j, :, 0] = 30.0
+        q[0] = 0
+        q[0, :, 0] = 30.0
+        v[j] = 5.0
+        q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+        n_pages = math.ceil(ctx / bs)
+        table = pages[used:used + n_pages]
+        used += n_pages
+        tables[s, :n_pages] = table.numpy()
+        pos = torch.arange(ctx)
+        kc[table[pos // bs], :, pos % bs] = k
+        vc[table[pos // bs], :, :, pos % bs] = v
+        q_rows.append(q.reshape(1, H * Dh))
+        want_rows.append(plain.causal_attention_tail(q, k, v, Dh ** -0.5).reshape(1, H * Dh))
+    return dict(q=torch.cat(q_rows).cuda().contiguous(), kc=kc.cuda(), vc=vc.cuda(), tables=torch.from_numpy(tables).cuda(),
+                query_start=i32(list(range(S + 1))), context_lens=i32(lens_ctx), want=torch.cat(want_rows)), S
+
+
+@pytest.mark.parametrize("nsplit", [32, 64, 129, 256])
+def test_attention_decode_bf16_many_key_shares(nsplit):
+    """The numbers of shares that serving contexts get (32 at 4096 keys, up to 256): every merge width."""
+    H, KVH, Dh = 8, 2, 128
+    case, S = long_decode_case(H, KVH, Dh, 16, [8200, 16001, 12288], seed=31, spike_back=7000)
+    out = run_decode(case, S, H, Dh, nsplit)
+    close(out, case["want"], 1e-2, f"decode attention over long contexts, {nsplit} shares")
+    assert float(out.float().min()) > 4.9
+
+
+@pytest.mark.parametrize("H,KVH", [(4, 1), (8, 2), (16, 4)])
+def test_attention_decode_bf16_one_sequence_past_32k(H, KVH):
+    """One sequence alone at 40 000 keys with few KV heads: the plan asks for as many shares as it may."""
+    from tie_amd import kernels
+
+    Dh, ctx = 64, 40000
+    nsplit = kernels.decode_splits(1, KVH, 65536)
+    assert nsplit == kernels.MAX_KEY_SPLITS or KVH > 8
+    case, S = long_decode_case(H, KVH, Dh, 16, [ctx], seed=33, spike_back=39000)
+    out = run_decode(case, S, H, Dh, nsplit)
+    close(out, case["want"], 1e-2, f"decode attention, one sequence of {ctx} keys, {nsplit} shares")
+    assert float(out.float().min()) > 4.9
 
 
 

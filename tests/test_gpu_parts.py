@@ -127,6 +127,32 @@ def test_sums_a_product_leaves_owed_reach_the_stream_through_the_norm_or_settle(
     assert ctx._owed is None and torch.equal(residual2, residual)
 
 
+@pytest.mark.parametrize("T", [4, 200])
+def test_two_products_in_a_row_that_leave_their_sums_owed(T):
+    """Two accumulating projections into one stream with no norm between them (a parallel residual, shared
+    beside routed experts): the first one's planes must reach the stream before the second reuses their buffer."""
+    from tie_amd.parts.linear import Linear
+
+    g = torch.Generator().manual_seed(5)
+    D, K = 256, 1024
+    w = {"a": (torch.randn(D, K, generator=g) * 0.05).to(torch.bfloat16),
+         "b": (torch.randn(D, K, generator=g) * 0.05).to(torch.bfloat16)}
+    fetch = fetcher(w, "bfloat16")
+    first, second = Linear(["a"], [D], K), Linear(["b"], [D], K)
+    first.load(fetch)
+    second.load(fetch)
+    x1, x2 = torch.randn(T, K, generator=g).to(torch.bfloat16), torch.randn(T, K, generator=g).to(torch.bfloat16)
+    stream = torch.randn(T, D, generator=g)
+    want = stream.to(F64) + plain.linear(x1.to(F64), w["a"].to(F64)) + plain.linear(x2.to(F64), w["b"].to(F64))
+    ctx = make_ctx(T, "bfloat16")
+    residual = stream.cuda().clone()
+    first(x1.cuda(), residual, accumulate=True, ctx=ctx)
+    assert ctx._owed is not None, "a product over 1024 of K at this size is expected to leave its sum owed"
+    second(x2.cuda(), residual, accumulate=True, ctx=ctx)
+    ctx.settle()
+    close(residual, want, 2e-3, "stream after two owed products")
+
+
 def test_position_part_holds_the_reference_frequencies():
     from tie_amd.parts import PartSpec, build_part
 
@@ -221,7 +247,11 @@ def register_toy_parts():
 
     @register_part("mixer", "toy_decay")
     class ToyDecayMixer(Mixer):
-        """s_t = decay * s_{t-1} + W_in h_t ; out_t = W_out s_t, with s kept per request in a state slot."""
+        """s_t = decay * s_{t-1} + W_in h_t ; out_t = W_out s_t, with s kept per request in a state slot.
+
+        It walks the step's sequences on the host, so a recording of it would hold one step's slots for good."""
+
+        capturable = False
 
         def __init__(self, params):
             super().__init__(params)
@@ -248,9 +278,29 @@ def register_toy_parts():
                     residual[t] += state @ self.w_out.float().T
                 row += n
 
+    @register_part("mixer", "toy_decay_on_device")
+    class ToyDecayMixerOnDevice(ToyDecayMixer):
+        """The same mixer written so that decode-only steps may be recorded: there, one row a sequence, the
+        states are gathered and scattered by the step's slot array ON THE DEVICE, and nothing of the step is
+        read on the host. (Steps with prompt portions are never recorded and take the loop above.)"""
+
+        capturable = True
+
+        def forward(self, ctx, h, cache, residual):
+            if not ctx.batch.all_decode:
+                return super().forward(ctx, h, cache, residual)
+            slots = cache.state_slots.long()
+            state = cache.state.index_select(0, slots) * self.decay + h.float() @ self.w_in.float().T
+            cache.state.index_copy_(0, slots, state)
+            residual += state @ self.w_out.float().T
+
     @register_part("feed_forward", "toy_routed")
     class ToyRoutedFeedForward(FeedForward):
-        """Router logits in float32, the top k experts per token, softmax over the chosen, ReLU experts."""
+        """Router logits in float32, the top k experts per token, softmax over the chosen, ReLU experts.
+
+        ``nonzero`` waits for the GPU, so a model with this part runs every step eagerly."""
+
+        capturable = False
 
         def __init__(self, params):
             super().__init__(params)
@@ -301,6 +351,15 @@ def register_toy_parts():
             k[:, :, 0] += shift[:, None]
 
 
+def unregister_toy_parts():
+    from tie_amd.parts import unregister_part
+
+    unregister_part("mixer", "toy_decay")
+    unregister_part("mixer", "toy_decay_on_device")
+    unregister_part("feed_forward", "toy_routed")
+    unregister_part("position", "toy_shift")
+
+
 def toy_spec(cfg):
     from tie_amd.models import LayerCall, LayerSpec, ModelSpec
     from tie_amd.parts import PartSpec
@@ -310,8 +369,8 @@ def toy_spec(cfg):
     layers = []
     for l, kind in enumerate(cfg["mixers"]):
         p = f"layers.{l}."
-        if kind == "decay":
-            mixer = PartSpec("toy_decay", {"hidden": D, "width": cfg["state_width"], "decay": cfg["decay"],
+        if kind in ("decay", "decay_on_device"):
+            mixer = PartSpec("toy_" + kind, {"hidden": D, "width": cfg["state_width"], "decay": cfg["decay"],
                                            "names": {"in": p + "mix.in", "out": p + "mix.out"}})
         else:
             mixer = PartSpec("paged_attention", {
@@ -342,7 +401,7 @@ def toy_plain(weights, cfg, tokens):
     for l, kind in enumerate(cfg["mixers"]):
         p = f"layers.{l}."
         h = plain.rms_norm(x, weights[p + "n1"], cfg["eps"])
-        if kind == "decay":
+        if kind in ("decay", "decay_on_device"):
             u = plain.linear(h, weights[p + "mix.in"])
             s = torch.zeros(cfg["state_width"], dtype=F64)
             out = []
@@ -381,7 +440,6 @@ def test_a_toy_architecture_registered_from_outside_runs_through_the_step_functi
     from tie_amd.cache.spec import FixedState, PagedKV
     from tie_amd.config.registry import register_architecture, unregister_architecture
     from tie_amd.engine.replay import TraceReplayer
-    from tie_amd.parts import unregister_part
     from tie_amd.weights.random_init import write_random_model
 
     register_toy_parts()
@@ -415,6 +473,75 @@ def test_a_toy_architecture_registered_from_outside_runs_through_the_step_functi
             tokens.append(t)
     finally:
         unregister_architecture("ToyStateLM")
-        unregister_part("mixer", "toy_decay")
-        unregister_part("feed_forward", "toy_routed")
-        unregister_part("position", "toy_shift")
+        unregister_toy_parts()
+
+
+def changing_live_sets(requests, head, subsets):
+    """A trace: every request's first ``head[id]`` tokens in one mixed step, then decode-only steps over the
+    live subsets named in turn (so equal step shapes meet different requests and state slots), then the rest."""
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": requests[r][:head[r]], "want": list(range(head[r]))}
+                                      for r in requests], "end": []}]
+    pos = dict(head)
+    k = 0
+    while any(pos[r] < len(requests[r]) for r in requests):
+        chosen = [r for r in subsets[k % len(subsets)] if pos[r] < len(requests[r])]
+        k += 1
+        if not chosen:
+            continue
+        entries = [{"id": r, "tokens": [requests[r][pos[r]]], "want": [0]} for r in chosen]
+        for r in chosen:
+            pos[r] += 1
+        steps.append({"step": len(steps), "entries": entries, "end": [r for r in chosen if pos[r] == len(requests[r])]})
+    return steps
+
+
+@pytest.mark.parametrize("kind", ["recorded", "eager"])
+def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, kind):
+    """The serving precision, where decode-only steps are recorded and replayed. A model whose parts all read
+    the step on the device is recorded, and replays must follow the step's slots as the live set changes; a
+    model with one part that reads the step on the host (or waits for the GPU) must not be recorded at all."""
+    import tie_amd
+    from tie_amd.config.registry import register_architecture, unregister_architecture
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.weights.random_init import write_random_model
+
+    register_toy_parts()
+    register_architecture("ToyStateLM", lambda values: dict(values), toy_spec, model_types=("toy_state",))
+    try:
+        cfg = {"architectures": ["ToyStateLM"], "vocab_size": 90, "hidden_size": 48, "intermediate": 72,
+               "heads": 3, "kv_heads": 1, "head_dim": 16, "state_width": 20, "decay": 0.8, "slope": 0.01,
+               "eps": 1e-5, "max_positions": 256, "experts": 5, "top_k": 2, "expert_width": 24}
+        if kind == "recorded":
+            cfg.update(mixers=["decay_on_device", "attention", "decay_on_device"], feed_forwards=["dense"] * 3)
+        else:
+            cfg.update(mixers=["decay", "attention", "decay_on_device"], feed_forwards=["dense", "routed", "dense"])
+        folder = write_random_model(tmp_path / "toy", cfg, seed=4, dtype="bfloat16")
+        replayer = TraceReplayer.from_folder(folder, "bfloat16", 256, block_size=4)
+        assert replayer.runner.use_graphs == (kind == "recorded")
+        weights = load_plain_weights(folder)
+        requests = th.make_requests(cfg["vocab_size"], [40, 52, 31, 44], seed=6)
+        want = {rid: toy_plain(weights, cfg, toks).float() for rid, toks in requests.items()}
+        head = {"r0": 20, "r1": 30, "r2": 12, "r3": 25}
+        subsets = [("r0", "r1"), ("r2", "r3"), ("r1", "r2"), ("r3", "r0"), ("r0", "r1", "r2"), ("r3", "r2", "r1"),
+                   ("r2",), ("r0",), ("r0", "r1", "r2", "r3"), ("r3", "r1", "r0", "r2")]
+        got = th.collect(replayer, changing_live_sets(requests, head, subsets))
+        for rid, ref in want.items():
+            mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
+            close(mine, ref, 3e-2, f"toy model in bfloat16 ({kind}), request {rid}")
+        assert replayer.cache.num_free_state_slots == replayer.cache.max_state_slots
+        assert (replayer.runner.graph_replays > 20) == (kind == "recorded")
+        # and through the engine, whose scheduler hands the slots out; recording can also be switched off there
+        for use_graphs in (None, False):
+            engine = tie_amd.create_engine(replayer.model, kv_blocks=64, block_size=4, max_seqs=2,
+                                           max_tokens_per_step=16, use_graphs=use_graphs)
+            assert engine.runner.use_graphs == (kind == "recorded" and use_graphs is None)
+            prompt = requests["r2"]
+            out = engine.generate(prompt, tie_amd.SamplingParams(max_tokens=6))
+            tokens = list(prompt)
+            for t in out:
+                row = toy_plain(weights, cfg, tokens)[-1]
+                assert float(row.max() - row[t]) <= 3e-2 * float(row.abs().max()), "a token the plain logits do not favour"
+                tokens.append(t)
+    finally:
+        unregister_architecture("ToyStateLM")
+        unregister_toy_parts()

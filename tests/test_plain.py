@@ -110,6 +110,15 @@ def test_attention_window_limits_the_keys():
     assert torch.allclose(plain.causal_attention(q, k, v, 0.5, window=T), plain.causal_attention(q, k, v, 0.5))
 
 
+@pytest.mark.parametrize("window", [None, 1, 4, 9])
+def test_attention_tail_is_the_last_rows_of_the_whole(window):
+    T, H, KVH, Dh, n = 23, 6, 2, 8, 5
+    q, k, v = rand(T, H, Dh, seed=31), rand(T, KVH, Dh, seed=32), rand(T, KVH, Dh, seed=33)
+    whole = plain.causal_attention(q, k, v, 0.4, window)
+    assert torch.allclose(plain.causal_attention_tail(q[-n:], k, v, 0.4, window), whole[-n:], atol=1e-12)
+    assert torch.allclose(plain.causal_attention_tail(q[-1:], k, v, 0.4, window), whole[-1:], atol=1e-12)
+
+
 def test_swiglu_is_silu_times_up():
     h = rand(3, 16, seed=16)
     wg, wu, wd = rand(24, 16, seed=17), rand(24, 16, seed=18), rand(16, 24, seed=19)

@@ -19,15 +19,18 @@ from .models.builder import Model, load_model
 from .sampling.params import SamplingParams
 from .weights.binder import FLOAT32, normalize_mode
 
-DEFAULT_KV_BYTES = 4 << 30  # the reference's default KV budget (src/cli/args.h:241)
+DEFAULT_KV_BYTES = 4 << 30  # the reference's default KV budget (src/cli/args.h:24)
 
 
 def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, kv_blocks: Optional[int] = None,
                   block_size: int = 16, max_seqs: int = 64, max_tokens_per_step: int = 512, prefill_chunk: int = 0,
                   policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1,
                   stop_tokens: Sequence[int] = (), max_seq_len: Optional[int] = None,
-                  device: str = "cuda:0") -> Engine:
-    """``model`` is a folder (config.json + safetensors) or a Model that is already loaded."""
+                  device: str = "cuda:0", use_graphs: Optional[bool] = None) -> Engine:
+    """``model`` is a folder (config.json + safetensors) or a Model that is already loaded.
+
+    ``use_graphs`` False runs every step eagerly; None (the default) records decode-only steps into HIP
+    graphs in bfloat16 mode when every part of the model allows it."""
     if not isinstance(model, Model):
         model = load_model(model, normalize_mode(dtype), device)
     cache_dtype = "float32" if model.mode == FLOAT32 else "bfloat16"
@@ -39,7 +42,8 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
     serving = ServingConfig(max_tokens_per_step=max_tokens_per_step, max_seqs=max_seqs, prefill_chunk=prefill_chunk)
     scheduler = BatchScheduler(cache, SchedulerConfig(serving=serving, policy=policy, aging=aging,
                                                       watermark_blocks=watermark_blocks))
-    return Engine(model, cache, scheduler, serving, stop_tokens=stop_tokens, max_seq_len=max_seq_len)
+    return Engine(model, cache, scheduler, serving, stop_tokens=stop_tokens, max_seq_len=max_seq_len,
+                  use_graphs=use_graphs)
 
 
 def generate(model, prompt: Sequence[int], params: Optional[SamplingParams] = None, **engine_options) -> List[int]:

@@ -36,7 +36,8 @@ from ..errors import CapacityError, InvalidArgument
 from .block_pool import BlockPool
 from .spec import CachePlan, FixedState, PagedKV
 
-_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}       # what the kernels read and write
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
 _INT32_MAX = 2 ** 31 - 1
 FREED = -1  # table entry of a page that a window has passed and that was given back
 
@@ -104,10 +105,11 @@ class CacheManager:
                         (group.num_planes, 2, self.num_blocks, need.num_kv_heads, block_size, need.head_dim),
                         dtype=_DTYPES[dtype], device=device)
                 else:
-                    if need.dtype not in _DTYPES:
-                        raise InvalidArgument(f"state dtype must be one of {', '.join(_DTYPES)}, got '{need.dtype}'")
+                    if need.dtype not in _STATE_DTYPES:
+                        raise InvalidArgument(
+                            f"state dtype must be one of {', '.join(_STATE_DTYPES)}, got '{need.dtype}'")
                     self.state[g] = torch.zeros((group.num_planes, max_state_slots) + tuple(need.shape),
-                                                dtype=_DTYPES[need.dtype], device=device)
+                                                dtype=_STATE_DTYPES[need.dtype], device=device)
 
     # ----------------------------------------------------------------- sizes
     def blocks_for(self, tokens: int) -> int:

@@ -241,6 +241,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 #include "attention_merge.h"
 
 extern "C" int tie_attention_decode_head_dim() { return DH; }
+extern "C" int tie_attention_max_splits() { return MERGE_MAX_SPLITS; }
 
 extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
                                          float* part_o, float* part_ml, const int* query_start,
@@ -265,8 +266,7 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
 #undef LAUNCH
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
-  const int merge_threads = (nsplit > DH ? nsplit : DH) <= 64 ? 64 : ((nsplit > DH ? nsplit : DH) <= 128 ? 128 : 256);
-  attention_merge_kernel<<<dim3(H, num_seqs), merge_threads, 0, stream>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), query_start, seq_ids, H, nsplit);
+  attention_merge_kernel<<<dim3(H, num_seqs), attention_merge_threads(nsplit), 0, stream>>>(
+      part_o, part_ml, static_cast<bf16_t*>(out), nullptr, query_start, seq_ids, H, nsplit);
   return tie_launch_status();
 }

@@ -433,8 +433,7 @@ extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, co
   else LAUNCH(1, 4);
 #undef LAUNCH
   if (status != TIE_OK || nsplit == 1) return status;
-  const int merge_threads = (nsplit > DH ? nsplit : DH) <= 64 ? 64 : ((nsplit > DH ? nsplit : DH) <= 128 ? 128 : 256);
-  attention_merge_rows_kernel<<<dim3(H, num_merge_rows), merge_threads, 0, stream>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, H, nsplit);
+  attention_merge_kernel<<<dim3(H, num_merge_rows), attention_merge_threads(nsplit), 0, stream>>>(
+      part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, nullptr, nullptr, H, nsplit);
   return tie_launch_status();
 }

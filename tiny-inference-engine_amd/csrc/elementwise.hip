@@ -267,6 +267,8 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
 //   q, k: per-head RMSNorm over Dh with one weight vector shared by all heads,
 //         THEN rotate-half rotary: pairs (i, i + Dh/2), angle = float(pos) * inv_freq[i]
 //         (reference: src/model/qwen3.cpp:222-225, cpu_backend.cpp:161-193, backend/rope.h:9-13).
+//         More generally the first rotary_dim <= Dh dimensions of a head are rotated, as pairs
+//         (i, i + rotary_dim/2) or, interleaved, (2i, 2i + 1); the rest only passes the norm.
 //   q goes to q_out[t * q_row + h*Dh + d]; k (after norm and rotation) and raw v go to the paged
 //   cache with page = slot / block_size, offset = slot % block_size (cpu_backend.cpp:235-259):
 //   keys at ((page*KVH + h)*block_size + offset)*Dh + d, one row per position; values transposed
@@ -295,11 +297,18 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
                                              const int* __restrict__ positions, const int* __restrict__ slots,
                                              TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H,
                                              int KVH, int Dh, int block_size, int in_row, int q_row, int k_row,
-                                             size_t plane_stride, int planes) {
+                                             size_t plane_stride, int planes, int rotary_dim, int interleaved) {
   const int t = blockIdx.y;
   const int slot_index = blockIdx.x;
   const int lane = threadIdx.x;
   const int half = Dh / 2;
+  // Pair p < Dh/2 of a head is the elements (e1(p), e2(p)): the rotated pairs first, then the
+  // dimensions beyond rotary_dim in two runs (they are not rotated, so how they pair does not matter).
+  const int rhalf = rotary_dim / 2;
+  auto e1 = [&](int p) { return p < rhalf ? (interleaved ? 2 * p : p) : rotary_dim + (p - rhalf); };
+  auto e2 = [&](int p) {
+    return p < rhalf ? (interleaved ? 2 * p + 1 : p + rhalf) : rotary_dim + (half - rhalf) + (p - rhalf);
+  };
   const TX* in = qkv + static_cast<size_t>(t) * in_row + static_cast<size_t>(slot_index) * Dh;
 
   const bool is_q = slot_index < H;
@@ -321,8 +330,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
     x1[i] = 0.f;
     x2[i] = 0.f;
     if (p < half) {
-      x1[i] = load_planes(in + p, plane_stride, planes);
-      x2[i] = load_planes(in + p + half, plane_stride, planes);
+      x1[i] = load_planes(in + e1(p), plane_stride, planes);
+      x2[i] = load_planes(in + e2(p), plane_stride, planes);
       ss += x1[i] * x1[i] + x2[i] * x2[i];
     }
   }
@@ -349,15 +358,18 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   for (int i = 0; i < TIE_MAX_PAIRS; ++i) {
     const int p = lane + i * TIE_WAVE;
     if (p >= half) continue;
+    const int d1 = e1(p), d2 = e2(p);
     float a = x1[i], b = x2[i];
     if (w != nullptr) {
-      a = (a * inv) * w[p];
-      b = (b * inv) * w[p + half];
+      a = (a * inv) * w[d1];
+      b = (b * inv) * w[d2];
     }
     float o1 = a, o2 = b;
-    if (angles != nullptr) {   // cos and sin of this token's angles, computed once for all heads and layers
-      const float cs = angles[static_cast<size_t>(t) * Dh + p];
-      const float sn = angles[static_cast<size_t>(t) * Dh + half + p];
+    if (p >= rhalf) {
+      // beyond the rotated dimensions
+    } else if (angles != nullptr) {   // cos and sin of this token's angles, computed once for all heads and layers
+      const float cs = angles[static_cast<size_t>(t) * rotary_dim + p];
+      const float sn = angles[static_cast<size_t>(t) * rotary_dim + rhalf + p];
       o1 = a * cs - b * sn;
       o2 = b * cs + a * sn;
     } else if (inv_freq != nullptr) {
@@ -368,19 +380,19 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
       o2 = b * cs + a * sn;
     }
     if (dense_dst != nullptr) {
-      store_from_float(dense_dst + p, o1);
-      store_from_float(dense_dst + p + half, o2);
+      store_from_float(dense_dst + d1, o1);
+      store_from_float(dense_dst + d2, o2);
     } else {
-      store_from_float(cache_dst + p, o1);
-      store_from_float(cache_dst + p + half, o2);
+      store_from_float(cache_dst + d1, o1);
+      store_from_float(cache_dst + d2, o2);
     }
   }
 }
 
 // The same for head sizes of 32, 64, 128, 256 or 512: a lane takes 4 consecutive elements of a head's
-// first half and the 4 they pair with in the second (16-byte loads and stores where the old kernel's were
-// 4 and 2 bytes), head_dim / 8 lanes share a head, four waves of heads a workgroup. The sums of squares
-// meet by shuffles inside the lanes of a head.
+// first half and the 4 they pair with in the second (16-byte loads and stores where the one-wave-a-head
+// kernel above moves 4 and 2 bytes), head_dim / 8 lanes share a head, four waves of heads a workgroup.
+// The sums of squares meet by shuffles inside the lanes of a head. Whole heads rotated as halves only.
 typedef __attribute__((ext_vector_type(4))) float qk_f4_t;
 
 template <typename T>
@@ -510,13 +522,21 @@ extern "C" int tie_rope_angles(const int* positions, const float* inv_freq, floa
   return tie_launch_status();
 }
 
-// angles (optional): the table of tie_rope_angles for these positions; then inv_freq is not read.
+// angles (optional): the table of tie_rope_angles for these positions ([T, rotary_dim]); then inv_freq is not read.
+// rotary_dim: how many leading dimensions of a head are rotated (inv_freq holds rotary_dim / 2 values);
+// interleaved: pairs (2i, 2i + 1) instead of (i, i + rotary_dim / 2).
 extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int q_dtype,
                                          const float* q_w, const float* k_w, float eps, const float* inv_freq,
                                          const float* angles, const int* positions, const int* slots, void* k_cache, void* v_cache,
                                          int cache_dtype, int write_kv, void* k_dense, int T, int H, int KVH,
                                          int Dh, int block_size, int in_row, int q_row, int k_row,
-                                         long plane_stride, int planes, hipStream_t stream) {
+                                         long plane_stride, int planes, int rotary_dim, int interleaved,
+                                         hipStream_t stream) {
+  if (rotary_dim < 0 || rotary_dim > Dh || rotary_dim % 2 != 0) return TIE_BAD_ARGUMENT;
+  if (inv_freq == nullptr && angles == nullptr) {   // no rotation at all
+    rotary_dim = 0;
+    interleaved = 0;
+  }
   if (planes < 1 || (planes > 1 && plane_stride < static_cast<long>(T) * in_row)) return TIE_BAD_ARGUMENT;
   if (T <= 0 || H <= 0 || KVH <= 0 || Dh <= 0 || Dh % 2 != 0 || Dh > 2 * TIE_MAX_PAIRS * TIE_WAVE ||
       block_size <= 0 || T > 65535 || q_row < H * Dh)
@@ -526,7 +546,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   const int heads = H + ((write_kv || k_dense != nullptr) ? KVH : 0) + (write_kv ? KVH : 0);
   if (in_row < heads * Dh || (k_dense != nullptr && k_row < KVH * Dh)) return TIE_BAD_ARGUMENT;
   // Head sizes of 32 .. 512 in powers of two, and rows that keep 16-byte pieces aligned: the 4-wide kernel.
-  const bool wide = (Dh == 32 || Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) && in_row % 4 == 0 &&
+  const bool wide = (rotary_dim == 0 || (rotary_dim == Dh && !interleaved)) && (Dh == 32 || Dh == 64 || Dh == 128 || Dh == 256 || Dh == 512) && in_row % 4 == 0 &&
                     q_row % 4 == 0 && k_row % 4 == 0 && plane_stride % 4 == 0 &&
                     reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(k_dense) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
@@ -562,7 +582,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   qk_norm_rope_kv_write_kernel<TX, TQ, TC><<<grid, TIE_WAVE, 0, stream>>>(                                    \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, Dh,           \
-      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes)
+      block_size, in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, rotary_dim, interleaved)
   if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);

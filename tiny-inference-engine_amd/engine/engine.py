@@ -47,14 +47,14 @@ class EngineStats:
 
 class Engine:
     def __init__(self, model: Model, cache: CacheManager, scheduler=None, serving: Optional[ServingConfig] = None,
-                 stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None):
+                 stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None, use_graphs: Optional[bool] = None):
         self.model = model
         self.cache = cache
         self.serving = serving or ServingConfig()
         self.serving.validate()
         self.scheduler = scheduler or BatchScheduler(cache, SchedulerConfig(serving=self.serving))
         self.stop_tokens = set(int(t) for t in stop_tokens)
-        self.runner = ModelRunner(model, cache, max_seq_len)
+        self.runner = ModelRunner(model, cache, max_seq_len, use_graphs=use_graphs)
         self.sampler = DeviceSampler(model.device)
         self.sequences: Dict[int, Sequence] = {}
         self.on_token: Optional[Callable[[int, int], None]] = None

@@ -22,8 +22,9 @@ from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
+from .. import kernels
 from ..cache.manager import CacheManager
-from ..errors import InvalidArgument
+from ..errors import CapacityError, InvalidArgument
 from ..models.builder import Model
 from ..parts.base import StepContext, Workspace
 from ..weights.binder import BFLOAT16
@@ -53,9 +54,10 @@ class ModelRunner:
         self.max_blocks_per_seq = cache.blocks_for(self.max_seq_len)
         self.builder = BatchBuilder(cache, model.spec.vocab_size, self.max_blocks_per_seq, self.device)
         self.workspace = Workspace(self.device)
-        if use_graphs is None:
-            use_graphs = model.mode == BFLOAT16 and self.device.type == "cuda"
-        self.use_graphs = use_graphs
+        # Recording needs every part's consent: one part that reads the step's host-side values would
+        # bake them into the recording (see Part.capturable). ``use_graphs`` can only switch it off.
+        wanted = (model.mode == BFLOAT16) if use_graphs is None else bool(use_graphs)
+        self.use_graphs = wanted and self.device.type == "cuda" and model.capturable()
         self._recorded: Dict[Tuple[int, int, int], _RecordedStep] = {}
         self.graph_replays = 0
 
@@ -68,10 +70,15 @@ class ModelRunner:
 
         The returned tensor is scratch memory of the runner: it is valid until the next step.
         """
+        total = 0
         for e in entries:
             if e.start + len(e.tokens) > self.max_seq_len:
                 raise InvalidArgument(
                     f"a request would reach {e.start + len(e.tokens)} tokens; the limit is {self.max_seq_len}")
+            total += len(e.tokens)
+        if total > kernels.MAX_STEP_TOKENS:
+            raise CapacityError(f"a step of {total} tokens exceeds the {kernels.MAX_STEP_TOKENS} the kernels take; "
+                                f"cut the prompt into portions")
         batch = self.builder.build(entries)
         if not (self.use_graphs and batch.all_decode and self.model.layer_hook is None):
             return self._forward(batch)

@@ -36,6 +36,9 @@ _PER_HEAD_DIM = {
     "attention_prefill_bf16": ("tie_attention_prefill_bf16", "attention_prefill_bf16.hip"),
 }
 MFMA_HEAD_DIMS = tuple(range(16, 257, 16))   # head sizes the matrix-core attention kernels are built for
+MAX_KEY_SPLITS = 256      # MERGE_MAX_SPLITS of csrc/attention_merge.h: the most shares one row's keys are cut into
+MAX_HEAD_DIM = 512        # the largest head size any attention kernel takes (the generic ones)
+MAX_STEP_TOKENS = 65535   # rows of one step: a grid dimension of the row-wise kernels
 
 _SIGNATURES = {
     "elementwise": {
@@ -46,7 +49,8 @@ _SIGNATURES = {
         "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_void],
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
+                                      _c_void],
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
                                       _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -80,6 +84,7 @@ _SIGNATURES = {
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
+        "tie_attention_max_splits": [],
         "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                       _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                       _c_void],
@@ -457,8 +462,13 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
                           positions: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                           v_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
                           block_size: int, write_kv: bool = True, k_dense: Optional[torch.Tensor] = None,
-                          planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None) -> None:
+                          planes: int = 1, plane_stride: int = 0, angles: Optional[torch.Tensor] = None,
+                          rotary_dim: Optional[int] = None, pairing: str = "rotate_half") -> None:
     """Per-head RMSNorm of q and k, rotation by position, q to ``q_out``, k and v into the paged cache.
+
+    The first ``rotary_dim`` dimensions of a head (default: all) are rotated, as pairs
+    ``(i, i + rotary_dim / 2)`` (``pairing`` "rotate_half") or ``(2 i, 2 i + 1)`` ("interleaved") by
+    ``position * inv_freq[i]``; ``inv_freq`` holds ``rotary_dim / 2`` values.
 
     ``angles`` (from ``rope_angles`` for the same positions and ``inv_freq``) spares the kernel the
     sines and cosines.
@@ -481,17 +491,22 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         raise InvalidArgument(f"qkv rows hold {in_width} values, {heads * Dh} are needed")
     if tuple(q_out.shape) != (T, H * Dh):
         raise InvalidArgument(f"q output has shape {list(q_out.shape)}, expected {[T, H * Dh]}")
-    if Dh % 2 or Dh > 512:
-        raise InvalidArgument(f"head_dim {Dh} must be even and at most 512")
-    if T > 65535:
-        raise InvalidArgument(f"a step of {T} tokens exceeds the 65535 this kernel takes")
+    if Dh % 2 or Dh > MAX_HEAD_DIM:
+        raise InvalidArgument(f"head_dim {Dh} must be even and at most {MAX_HEAD_DIM}")
+    if T > MAX_STEP_TOKENS:
+        raise InvalidArgument(f"a step of {T} tokens exceeds the {MAX_STEP_TOKENS} this kernel takes")
     for wt, nm in ((q_weight, "q_norm weight"), (k_weight, "k_norm weight")):
         if wt is not None:
             _f32(wt, nm, (Dh,))
+    rotary_dim = Dh if rotary_dim is None else int(rotary_dim)
+    if rotary_dim % 2 or not 0 <= rotary_dim <= Dh:
+        raise InvalidArgument(f"rotary_dim {rotary_dim} must be even and at most head_dim {Dh}")
+    if pairing not in ("rotate_half", "interleaved"):
+        raise InvalidArgument(f"the fused kernel rotates pairs as 'rotate_half' or 'interleaved', not '{pairing}'")
     if inv_freq is not None:
-        _f32(inv_freq, "inv_freq", (Dh // 2,))
+        _f32(inv_freq, "inv_freq", (rotary_dim // 2,))
     if angles is not None:
-        _f32(angles, "rope angles", (T, Dh))
+        _f32(angles, "rope angles", (T, rotary_dim))
     _i32(positions, "positions", T)
     cache_code = _code(q_out, "q output")
     k_row = 0
@@ -514,7 +529,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
-        _stream()), "qk_norm_rope_kv_write")
+        rotary_dim, int(pairing == "interleaved"), _stream()), "qk_norm_rope_kv_write")
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -534,10 +549,10 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
     if H % KVH:
         raise InvalidArgument(f"{H} query heads are not a multiple of {KVH} kv heads")
-    if Dh > 512:
-        raise InvalidArgument(f"head_dim {Dh} exceeds the 512 this kernel takes")
-    if T > 65535:
-        raise InvalidArgument(f"a step of {T} tokens exceeds the 65535 this kernel takes")
+    if Dh > MAX_HEAD_DIM:
+        raise InvalidArgument(f"head_dim {Dh} exceeds the {MAX_HEAD_DIM} this kernel takes")
+    if T > MAX_STEP_TOKENS:
+        raise InvalidArgument(f"a step of {T} tokens exceeds the {MAX_STEP_TOKENS} this kernel takes")
     S = context_lens.numel()
     _i32(query_start, "query_start", S + 1)
     _i32(context_lens, "context_lens")
@@ -614,11 +629,23 @@ def mfma_block_size(block_size: int) -> bool:
 
 
 def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
-    """How many ways the keys of each sequence are split so that a decode step fills the GPU."""
+    """How many ways the keys of each sequence are split so that a decode step fills the GPU.
+
+    Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take.
+    """
     target_waves = 2048
     by_occupancy = -(-target_waves // max(1, num_seqs * num_kv_heads))
     by_length = max(1, max_context // 128)          # at least four 32-key tiles a split
-    return max(1, min(by_occupancy, by_length))
+    return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
+
+
+def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+    """Refuses, when a model is built, head geometries that no attention kernel here takes."""
+    if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+        raise InvalidArgument(f"{num_heads} query heads are not a positive multiple of {num_kv_heads} kv heads")
+    if head_dim <= 0 or head_dim % 2 or head_dim > MAX_HEAD_DIM:
+        raise InvalidArgument(f"head_dim {head_dim} must be even and at most {MAX_HEAD_DIM}: no attention kernel of "
+                              f"this engine takes it")
 
 
 def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -646,6 +673,8 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     _i32(block_tables, "block tables")
     if seq_ids is not None:
         _i32(seq_ids, "sequence ids", num_seqs)
+    if not 1 <= nsplit <= MAX_KEY_SPLITS:
+        raise InvalidArgument(f"attention_decode_bf16 cuts the keys into 1 to {MAX_KEY_SPLITS} shares, got {nsplit}")
     if nsplit > 1:
         _f32(part_o, "split accumulators")
         _f32(part_ml, "split maxima and sums")

@@ -2,7 +2,7 @@
 
 Each library is one ``.hip`` source of ``csrc/`` (plus the shared header) built
 with hipcc for gfx950 into ``csrc/_build/<name>-<hash>.so``; the hash covers the
-sources, the defines and the flags, so a stale library is never loaded. A
+source, the headers it includes, the defines and the flags, so a stale library is never loaded. A
 library is compiled the first time it is asked for and found missing - a fresh
 checkout builds what its model needs at its first call, printing a line now
 and then while hipcc runs - and ``build_all`` compiles everything up front.
@@ -16,6 +16,7 @@ import ctypes
 import hashlib
 import os
 import pathlib
+import re
 import shutil
 import subprocess
 import sys
@@ -72,9 +73,25 @@ def _candidates(filename: str):
     yield pathlib.Path(tempfile.gettempdir()) / f"tie_amd_build_{os.getuid()}" / filename
 
 
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"([^"]+)"', re.MULTILINE)
+
+
+def _sources_of(source: str):
+    """The source file and the headers of ``csrc/`` it includes, directly or through other headers."""
+    seen, todo = [], [source]
+    while todo:
+        name = todo.pop()
+        path = CSRC / name
+        if name in seen or not path.exists():
+            continue
+        seen.append(name)
+        todo.extend(_INCLUDE.findall(path.read_text()))
+    return [CSRC / n for n in sorted(seen)]
+
+
 def library_filename(name: str, source: str, defines: Mapping[str, object]) -> str:
     h = hashlib.sha256()
-    for path in sorted(CSRC.glob("*.h")) + [CSRC / source]:
+    for path in _sources_of(source):
         h.update(path.name.encode())
         h.update(path.read_bytes())
     h.update(repr(sorted((k, str(v)) for k, v in defines.items())).encode())

@@ -8,6 +8,7 @@ a step: embedding, the run order, the head on the wanted rows.
 
 from __future__ import annotations
 
+import sys
 from typing import Callable, Dict, List, Optional
 
 import torch
@@ -17,7 +18,7 @@ from ..config.registry import resolve_architecture
 from ..errors import InvalidArgument
 from ..parts import base as parts_base
 from ..parts.base import StepContext, TensorSpec, build_part
-from ..weights.binder import check_tensors, normalize_mode, place_tensor
+from ..weights.binder import BFLOAT16, check_tensors, normalize_mode, place_tensor
 from ..weights.loader import ModelFiles, load_model_folder
 from ..weights.safetensors_io import StoredTensor
 from .spec import ModelSpec
@@ -83,7 +84,18 @@ class Model:
             part.load_all(fetch, mode, device)
         self.mode = mode
         self.device = device
+        wide = sorted(name for (name, role), t in placed.items() if role == "matrix" and t.dtype == torch.float32)
+        if mode == BFLOAT16 and wide:
+            # Stored in 32 bits (or F16, widened): kept so, and every product over them runs on the float32
+            # kernel instead of the matrix cores. Correct, but far slower; say it once, loudly.
+            print(f"[tie_amd] WARNING: {len(wide)} weight matrices are not stored as BF16 (first: {wide[0]}); they "
+                  f"stay 32-bit and their products run on the float32 kernels, roughly ten times slower than the "
+                  f"bfloat16 ones. Convert the checkpoint to BF16 for serving speed.", file=sys.stderr, flush=True)
         return self
+
+    def capturable(self) -> bool:
+        """Whether every part allows its launches to be recorded and replayed (see ``Part.capturable``)."""
+        return all(part.all_capturable() for part in self._all_parts())
 
     # ------------------------------------------------------------------ step
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:

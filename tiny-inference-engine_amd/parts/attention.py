@@ -22,7 +22,6 @@ import torch
 
 from .. import kernels
 from ..cache.spec import PagedKV
-from ..errors import InvalidArgument
 from .base import Mixer, Part, PartSpec, StepContext, TensorSpec, build_part, register_part
 from .linear import Linear
 
@@ -37,8 +36,7 @@ class PagedAttention(Mixer):
         self.head_dim = int(params["head_dim"])
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")
-        if self.num_heads % self.num_kv_heads:
-            raise InvalidArgument(f"num_heads {self.num_heads} is not a multiple of num_kv_heads {self.num_kv_heads}")
+        kernels.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim)
         names = params["names"]
         q_dim, kv_dim = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
         self.q_dim, self.kv_dim = q_dim, kv_dim
@@ -88,12 +86,15 @@ class PagedAttention(Mixer):
             qkv = ctx.scratch("attention.qkv", (T, width), torch.float32)
             self.qkv(h, qkv)
         if table is not None:
-            inv_freq = table[0]
+            inv_freq, rotary_dim, pairing = table
+            if inv_freq is None:                      # an encoding that leaves queries and keys as they are
+                rotary_dim, pairing = None, "rotate_half"
             kernels.qk_norm_rope_kv_write(
                 qkv, q, self.q_norm_weight, self.k_norm_weight, eps, inv_freq, ctx.batch.positions,
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
                 write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
-                angles=self.position.angles(ctx))
+                angles=self.position.angles(ctx) if inv_freq is not None else None,
+                rotary_dim=rotary_dim, pairing=pairing)
         else:
             # A position encoding that is no rotation table: normalise in place, let the part
             # change q and k (float32 views into the projection rows), then convert and store.

@@ -76,7 +76,18 @@ def build_part(family: str, spec: PartSpec, **extra):
 
 
 class Part:
-    """Base of every part: declared tensors, loading, and nothing else."""
+    """Base of every part: declared tensors, loading, and nothing else.
+
+    ``capturable`` says whether the part's ``forward`` may be recorded into a HIP graph and replayed
+    for later steps: true only if everything that differs between steps is read ON THE DEVICE from
+    the step's arrays (``ctx.batch.tokens``, ``positions``, ``state_slots``, a group's block tables:
+    they live at fixed addresses) and the launches themselves depend only on the step's shape. A
+    part that reads host-side values of the step (``ctx.batch.host_*``), loops over them, or calls
+    anything that waits for the GPU (``nonzero``, ``.item()``, ``.cpu()``) sets it to False; a model
+    with one such part runs every step eagerly.
+    """
+
+    capturable = True
 
     def __init__(self, params: Mapping[str, Any]):
         self.params = dict(params)
@@ -100,6 +111,9 @@ class Part:
         self.load(fetch, mode, device)
         for child in self.children():
             child.load_all(fetch, mode, device)
+
+    def all_capturable(self) -> bool:
+        return bool(self.capturable) and all(child.all_capturable() for child in self.children())
 
 
 class Workspace:
@@ -227,7 +241,11 @@ class Position(Part):
 
     ``rotary_table()`` returns ``(inv_freq float32 [rotary_dim/2], rotary_dim,
     pairing)`` when the encoding is a rotation of pairs by position * inv_freq,
-    which the fused kernel applies itself; otherwise it returns None and the
+    which the fused kernel applies itself: the first ``rotary_dim`` (even, at
+    most head_dim) dimensions of every head are rotated, paired as
+    ``(i, i + rotary_dim/2)`` for pairing ``"rotate_half"`` or ``(2i, 2i + 1)``
+    for ``"interleaved"``; the other dimensions pass unchanged. ``inv_freq`` None
+    means no rotation at all. Any other encoding returns None here and the
     mixer calls ``apply(ctx, q, k, positions)`` on float32 tensors
     ``[T, heads, head_dim]`` instead.
     """
@@ -236,7 +254,8 @@ class Position(Part):
         return None
 
     def angles(self, ctx: "StepContext") -> Optional[torch.Tensor]:
-        """Optional: ``[T, rotary_dim]`` float32 cos | sin of this step's positions, for the fused kernel."""
+        """Optional: ``[T, rotary_dim]`` float32, cos of the ``rotary_dim/2`` angles then their sines, of this
+        step's positions, for the fused kernel (which otherwise computes them per head)."""
         return None
 
     def apply(self, ctx: StepContext, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:

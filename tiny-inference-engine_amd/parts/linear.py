@@ -60,6 +60,9 @@ class Linear:
         ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once.
         """
         if ctx is not None and accumulate and out.dtype == torch.float32:
+            # An earlier product's planes may still be owed and live in the buffer the new planes take:
+            # add them before they are overwritten (after a norm that took the debt this does nothing).
+            ctx.settle()
             planes = self.partial_planes(ctx, x, "linear.partials")
             if planes is not None:
                 ctx.defer_add(out, planes)
