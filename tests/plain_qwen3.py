@@ -20,7 +20,7 @@ F64 = torch.float64
 
 def embed(table: torch.Tensor, ids: Sequence[int]) -> torch.Tensor:
     """x[t] = table[ids[t]], no scaling. src/backend/cpu/cpu_backend.cpp:51-76; src/model/qwen3.cpp:213."""
-    return table.to(F64)[torch.as_tensor(list(ids), dtype=torch.long)]
+    return table[torch.as_tensor(list(ids), dtype=torch.long)].to(F64)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -148,11 +148,14 @@ def attention_block(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cf
 
 
 def forward(weights: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int],
-            hidden_states: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+            hidden_states: Optional[List[torch.Tensor]] = None, rows: Optional[Sequence[int]] = None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence. src/model/qwen3.cpp:213-259.
 
     x = embed; per layer: x += attention(norm(x)); x += mlp(norm(x)); logits = norm(x) @ lm_head^T,
     lm_head being the embedding matrix when tie_word_embeddings is set (qwen3.cpp:94-100).
+    ``rows``: the positions whose logits are returned (all by default), as the reference's step
+    returns logits at the requested rows only (qwen3.cpp:249-259). Weights may come in any float
+    type: every product widens its operands to float64 itself.
     """
     cfg = normalized_config(cfg)
     eps = cfg["rms_norm_eps"]
@@ -167,6 +170,8 @@ def forward(weights: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int],
                        weights[p + "mlp.down_proj.weight"])
         if hidden_states is not None:
             hidden_states.append(x.clone())
+    if rows is not None:
+        x = x[torch.as_tensor(list(rows), dtype=torch.long)]
     x = rms_norm(x, weights["model.norm.weight"], eps)
     head = weights["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else weights["lm_head.weight"]
     return linear(x, head)
