@@ -102,11 +102,11 @@ def test_capacity_rejections_and_clamping(model_folders):
 
     folder, cfg = model_folders["A"]                      # context 128
     engine = make_engine(folder, 4, kv_blocks=10)         # the pool holds 40 tokens
-    with pytest.raises(InvalidArgument, match="empty"):
+    with pytest.raises(InvalidArgument, match="at least one prompt token"):
         engine.add_request([])
-    with pytest.raises(InvalidArgument, match="outside vocabulary"):
+    with pytest.raises(InvalidArgument, match="not in the vocabulary"):
         engine.add_request([1, cfg["vocab_size"]])
-    with pytest.raises(CapacityError, match="KV blocks"):
+    with pytest.raises(CapacityError, match="the cache of 10 pages"):
         engine.add_request([1] * 40)
     sid = engine.add_request([1] * 30, tie_amd.SamplingParams(max_tokens=100))
     assert engine.sequence(sid).params.max_tokens == 10   # clamped to the room the pool leaves
@@ -114,7 +114,7 @@ def test_capacity_rejections_and_clamping(model_folders):
         engine.step()
     assert engine.sequence(sid).num_generated == 10 and engine.sequence(sid).finish_reason.value == "length"
     big = make_engine(folder, 4, kv_blocks=64)
-    with pytest.raises(CapacityError, match="context"):
+    with pytest.raises(CapacityError, match="the model's context holds 128"):
         big.add_request([1] * 128)
 
 
@@ -246,14 +246,14 @@ def test_cancel_release_and_callbacks(model_folders):
             engine.step()                                     # but stepping inside a step is refused
 
     engine.on_token = on_token
-    with pytest.raises(InvalidArgument, match="still running"):
+    with pytest.raises(InvalidArgument, match="has not finished"):
         engine.release(a)
     while engine.has_work():
         engine.step()
     assert engine.sequence(a).finish_reason.value == "cancelled" and engine.sequence(a).num_generated == 3
     assert engine.sequence(b).num_generated == 5
     engine.release(a)
-    with pytest.raises(InvalidArgument, match="no sequence"):
+    with pytest.raises(InvalidArgument, match="knows no sequence"):
         engine.sequence(a)
     assert engine.cache.num_free() == engine.cache.num_blocks
 

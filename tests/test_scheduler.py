@@ -345,5 +345,41 @@ def test_randomized_everything_finishes_and_no_page_is_shared_or_lost(seed):
 test_randomized_everything_finishes_and_no_page_is_shared_or_lost.preemptions = 0
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_the_shortcut_for_steady_decoding_plans_what_the_rounds_would(seed):
+    """Two schedulers over equal pools and equal requests, one with the shortcut switched off: equal plans."""
+    rng = random.Random(1000 + seed)
+    blocks, budget = rng.randint(6, 40), rng.randint(4, 32)
+    cfg = lambda: config(budget, rng_seats, FCFS if seed % 2 else SRPT_AGING, 0, 4)
+    rng_seats = rng.randint(1, min(8, budget))
+    fast, slow = Fixture(blocks, cfg()), Fixture(blocks, cfg())
+    slow.sched._steady_decode = lambda plan, budget: False
+    arrivals = sorted((rng.randint(0, 30), rng.randint(1, blocks * 4 - 1)) for _ in range(rng.randint(1, 10)))
+    arrivals = [(at, n, rng.randint(1, blocks * 4 - n)) for at, n in arrivals]
+    step = nxt = 0
+    while step < 3000 and (nxt < len(arrivals) or fast.sched.has_work()):
+        while nxt < len(arrivals) and arrivals[nxt][0] <= step:
+            for f in (fast, slow):
+                f.add(arrivals[nxt][1], arrivals[nxt][2])
+            nxt += 1
+        plans = [f.run() for f in (fast, slow)]
+        assert [(x.seq.id, x.num_tokens) for x in plans[0].seqs] == [(x.seq.id, x.num_tokens) for x in plans[1].seqs]
+        for f in (fast, slow):
+            for s in f.seqs:
+                if s.state == SeqState.DECODING and s.num_generated >= s.params.max_tokens:
+                    f.finish(s)
+        assert fast.cache.num_free() == slow.cache.num_free()
+        step += 1
+    assert not fast.sched.has_work() and not slow.sched.has_work()
+    test_the_shortcut_for_steady_decoding_plans_what_the_rounds_would.taken += fast.sched.steady_steps
+
+
+test_the_shortcut_for_steady_decoding_plans_what_the_rounds_would.taken = 0
+
+
+def test_the_shortcut_was_taken():
+    assert test_the_shortcut_for_steady_decoding_plans_what_the_rounds_would.taken > 100
+
+
 def test_the_randomized_runs_did_preempt():
     assert test_randomized_everything_finishes_and_no_page_is_shared_or_lost.preemptions > 0

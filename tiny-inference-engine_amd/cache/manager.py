@@ -57,6 +57,9 @@ class RequestCache:
     def num_held(self) -> int:
         return sum(1 for table in self.tables for b in table if b != FREED)
 
+    def holds_pages(self) -> bool:
+        return any(b != FREED for table in self.tables for b in table)
+
 
 class CacheManager:
     def __init__(self, plan: CachePlan, block_size: int = 16, num_blocks: Optional[int] = None,
@@ -93,6 +96,7 @@ class CacheManager:
         self.num_blocks = min(num_blocks, _INT32_MAX // block_size)
 
         self.pools: Dict[int, BlockPool] = {g: BlockPool(self.num_blocks) for g in plan.paged_groups}
+        self.has_windows = any(plan.groups[g].need.window is not None for g in plan.paged_groups)
         self._free_state_slots: List[int] = list(range(max_state_slots - 1, -1, -1))
         self._state_slot_used = [False] * max_state_slots
         self.kv: Dict[int, torch.Tensor] = {}
@@ -122,6 +126,14 @@ class CacheManager:
         if not self.pools:
             return self.num_blocks
         return min(p.num_free for p in self.pools.values())
+
+    def has_free_pages(self, count: int) -> bool:
+        """Whether every paged group has ``count`` free pages."""
+        return all(pool.num_free >= count for pool in self.pools.values())
+
+    def holds_pages(self, req: "RequestCache") -> bool:
+        """Whether giving back what ``req`` holds would free at least one page of some group."""
+        return req.holds_pages()
 
     @property
     def num_free_state_slots(self) -> int:
@@ -227,6 +239,8 @@ class CacheManager:
         Their table entries stay (as FREED) so that positions keep their index.
         """
         freed = 0
+        if not self.has_windows:
+            return freed
         for g, pool in self.pools.items():
             window = self.plan.groups[g].need.window
             if window is None:

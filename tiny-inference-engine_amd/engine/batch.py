@@ -23,7 +23,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import FREED, CacheManager, RequestCache
+from ..cache.manager import CacheManager, RequestCache
 from ..errors import CapacityError, InvalidArgument
 
 
@@ -101,34 +101,32 @@ class BatchBuilder:
 
     @staticmethod
     def _table_row(cache, g: int, MB: int) -> np.ndarray:
-        """A request's block table of group ``g`` as a row of ``MB`` page numbers (0 where there is none).
-
-        Kept on the request between steps and rebuilt only when the table has changed."""
+        """A request's block table of group ``g`` as a row of ``MB`` page numbers: 0 where the table has ended,
+        FREED where a window has passed. Kept on the request between steps, rebuilt only when the table changed."""
         memo = cache.rows[g]
         if memo is None or memo[0] != cache.version or memo[1].shape[0] != MB:
             arr = np.zeros(MB, dtype=np.int32)
             table = cache.tables[g][:MB]
             if table:
-                arr[:len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)    # FREED (-1) -> 0
+                arr[:len(table)] = table
             memo = cache.rows[g] = (cache.version, arr)
         return memo[1]
 
-    def build(self, entries: Sequence[StepEntry]) -> StepBatch:
-        if not entries:
-            raise InvalidArgument("a step needs at least one entry")
-        bs = self.cache.block_size
+    def _check(self, entries: Sequence[StepEntry]):
+        """Refuses what must never reach a kernel; returns (rows, wanted rows, whether every entry is one token)."""
         MB = self.max_blocks_per_seq
-        S = len(entries)
+        groups = self.cache.plan.paged_groups
+        needs_slot = bool(self.cache.plan.state_groups)
         seen = set()
-        T = 0
-        R = 0
+        T = R = 0
         for e in entries:
             n = len(e.tokens)
             if n < 1:
                 raise InvalidArgument("an entry of a step needs at least one token")
-            if id(e.cache) in seen:
+            key = id(e.cache)
+            if key in seen:
                 raise InvalidArgument("a request appears twice in one step")
-            seen.add(id(e.cache))
+            seen.add(key)
             if e.start < 0:
                 raise InvalidArgument(f"an entry starts at position {e.start}")
             for w in e.want:
@@ -138,15 +136,97 @@ class BatchBuilder:
             if need > MB:
                 raise CapacityError(
                     f"{e.start + n} tokens need {need} KV blocks but a block-table row holds {MB}")
-            for g in self.cache.plan.paged_groups:
+            for g in groups:
                 if len(e.cache.tables[g]) < need:
                     raise InvalidArgument(
                         f"a request has {len(e.cache.tables[g])} KV blocks reserved; {e.start + n} tokens need {need}")
-            if self.cache.plan.state_groups and e.cache.state_slot < 0:
+            if needs_slot and e.cache.state_slot < 0:
                 raise InvalidArgument("a request of a model with per-request state has no state slot")
             T += n
             R += len(e.want)
+        return T, R, T == len(entries)
 
+    def _bad_token(self, ids) -> InvalidArgument:
+        bad = next(int(t) for t in ids if not 0 <= int(t) < self.vocab_size)
+        return InvalidArgument(f"token id {bad} outside vocabulary of {self.vocab_size}")
+
+    def _fill_decode(self, entries, view, batch: StepBatch) -> None:
+        """Every entry brings one token: the arrays are filled as whole vectors, not entry by entry."""
+        S = len(entries)
+        bs, MB = self.cache.block_size, self.max_blocks_per_seq
+        starts = np.fromiter((e.start for e in entries), dtype=np.int32, count=S)
+        ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=S)
+        if ids.min() < 0 or ids.max() >= self.vocab_size:
+            raise self._bad_token(ids)
+        order = np.arange(S + 1, dtype=np.int32)
+        view("tokens")[:] = ids
+        view("positions")[:] = starts
+        view("seq_of_row")[:] = order[:S]
+        view("query_start")[:] = order
+        view("context_lens")[:] = starts + 1
+        slots = [e.cache.state_slot for e in entries]
+        view("state_slots")[:] = np.maximum(np.asarray(slots, dtype=np.int32), 0)
+        view("logit_rows")[:] = [s for s, e in enumerate(entries) for _ in e.want]     # wanted places are all 0
+        page_of_start = starts // bs
+        for g in self.cache.plan.paged_groups:
+            tables = view(("tables", g)).reshape(S, MB)
+            for s, e in enumerate(entries):
+                tables[s] = self._table_row(e.cache, g, MB)
+            pages = tables[order[:S], page_of_start]
+            if pages.min() < 0:
+                s = int(np.argmin(pages))
+                raise InvalidArgument(f"position {int(starts[s])} lies in a page that was already given back")
+            view(("slots", g))[:] = pages * bs + starts % bs
+            np.maximum(tables, 0, out=tables)        # FREED (-1) -> 0: the kernels never read those entries
+        batch.host_new_tokens = [1] * S
+        batch.host_context_lens = (starts + 1).tolist()
+        batch.host_state_slots = slots
+
+    def _fill_general(self, entries, view, batch: StepBatch) -> None:
+        bs, MB = self.cache.block_size, self.max_blocks_per_seq
+        groups = self.cache.plan.paged_groups
+        tokens, positions, seq_of_row = view("tokens"), view("positions"), view("seq_of_row")
+        query_start, context_lens = view("query_start"), view("context_lens")
+        state_slots, logit_rows = view("state_slots"), view("logit_rows")
+        slot_views = [view(("slots", g)) for g in groups]
+        table_views = [view(("tables", g)) for g in groups]
+        row = r = 0
+        query_start[0] = 0
+        for s, e in enumerate(entries):
+            n = len(e.tokens)
+            start = e.start
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if ids.min() < 0 or ids.max() >= self.vocab_size:
+                raise self._bad_token(ids)
+            where = np.arange(start, start + n, dtype=np.int32)
+            tokens[row:row + n] = ids
+            positions[row:row + n] = where
+            seq_of_row[row:row + n] = s
+            context_lens[s] = start + n
+            state_slots[s] = max(e.cache.state_slot, 0)
+            for w in e.want:
+                logit_rows[r] = row + w
+                r += 1
+            for gi, g in enumerate(groups):
+                table = self._table_row(e.cache, g, MB)
+                pages = table[where // bs]
+                if pages.min() < 0:
+                    gone = int(where[int(np.argmin(pages))])
+                    raise InvalidArgument(f"position {gone} lies in a page that was already given back")
+                slot_views[gi][row:row + n] = pages * bs + where % bs
+                table_views[gi][s * MB:(s + 1) * MB] = np.maximum(table, 0)     # FREED (-1) -> 0: never read
+            row += n
+            query_start[s + 1] = row
+            batch.host_new_tokens.append(n)
+            batch.host_context_lens.append(start + n)
+            batch.host_state_slots.append(e.cache.state_slot)
+
+    def build(self, entries: Sequence[StepEntry]) -> StepBatch:
+        if not entries:
+            raise InvalidArgument("a step needs at least one entry")
+        MB = self.max_blocks_per_seq
+        S = len(entries)
+        T, R, all_single = self._check(entries)
         groups = self.cache.plan.paged_groups
         layout = {}
         offset = 0
@@ -166,53 +246,11 @@ class BatchBuilder:
             o, c = layout[key]
             return host[o:o + c]
 
-        tokens, positions, seq_of_row = view("tokens"), view("positions"), view("seq_of_row")
-        query_start, context_lens = view("query_start"), view("context_lens")
-        state_slots, logit_rows = view("state_slots"), view("logit_rows")
         batch = StepBatch()
-        row = 0
-        r = 0
-        query_start[0] = 0
-        slot_views = [view(("slots", g)) for g in groups]
-        table_views = [view(("tables", g)) for g in groups]
-        for s, e in enumerate(entries):
-            n = len(e.tokens)
-            start = e.start
-            if n == 1:                                  # a decoded token: no arrays needed
-                tok = e.tokens[0]
-                if not 0 <= tok < self.vocab_size:
-                    raise InvalidArgument(f"token id {tok} outside vocabulary of {self.vocab_size}")
-                tokens[row] = tok
-                positions[row] = start
-                seq_of_row[row] = s
-            else:
-                ids = np.asarray(e.tokens, dtype=np.int64)
-                if ids.min() < 0 or ids.max() >= self.vocab_size:
-                    bad = int(ids[(ids < 0) | (ids >= self.vocab_size)][0])
-                    raise InvalidArgument(f"token id {bad} outside vocabulary of {self.vocab_size}")
-                tokens[row:row + n] = ids
-                positions[row:row + n] = np.arange(start, start + n, dtype=np.int32)
-                seq_of_row[row:row + n] = s
-            context_lens[s] = start + n
-            state_slots[s] = max(e.cache.state_slot, 0)
-            for w in e.want:
-                logit_rows[r] = row + w
-                r += 1
-            for gi, g in enumerate(groups):
-                table = e.cache.tables[g]
-                if n == 1:
-                    page = table[start // bs]
-                    if page == FREED:
-                        raise InvalidArgument(f"position {start} lies in a page that was already given back")
-                    slot_views[gi][row] = page * bs + start % bs
-                else:
-                    slot_views[gi][row:row + n] = self.cache.slots(e.cache, g, start, start + n)
-                table_views[gi][s * MB:(s + 1) * MB] = self._table_row(e.cache, g, MB)
-            row += n
-            query_start[s + 1] = row
-            batch.host_new_tokens.append(n)
-            batch.host_context_lens.append(start + n)
-            batch.host_state_slots.append(e.cache.state_slot)
+        if all_single:
+            self._fill_decode(entries, view, batch)
+        else:
+            self._fill_general(entries, view, batch)
 
         dev_t[:offset].copy_(host_t[:offset], non_blocking=True)
         if self.device.type == "cuda":

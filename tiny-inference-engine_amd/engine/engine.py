@@ -1,27 +1,24 @@
 """The engine: requests in, tokens out, one step at a time.
 
-The scheduler picks the work, the engine builds the batch, runs the step
-function, samples, and finishes sequences (``src/engine/engine.cpp:26-235`` of
-the reference, whose behaviour this follows):
+One ``step()`` is: the scheduler plans (which sequence, how many tokens); the plan becomes the
+entries of one batch; the step function runs them; progress is recorded; the sequences whose
+whole input is now cached sample their next token. The behaviour towards the caller is the
+reference engine's (``src/engine/engine.cpp:26-235``):
 
-* ``add_request`` rejects only what can never run - an empty prompt, a token id
-  outside the vocabulary, a prompt that leaves no room for one generated token
-  in the context, the page pool or a block-table row - and clamps ``max_tokens``
-  to the room that is left;
-* a step that fails before progress is recorded gives back the pages reserved
-  for it and is offered again; a failure while sampling finishes the affected
-  sequences with an error and frees what they hold;
-* a sequence samples once all its known tokens are cached; it finishes on a
-  stop token (kept in the output) or at ``max_tokens``.
+* ``add_request`` turns away only what could never run - no tokens, a token id the vocabulary does
+  not have, a prompt that leaves no room for a single generated token in the context, in the page
+  pool or in a block-table row - and shortens ``max_tokens`` to the room there is;
+* a step that fails before its progress is recorded gives its pages back and will be planned
+  again; a failure after that (sampling, a token callback) ends the affected sequences with
+  ``FinishReason.ERROR`` and frees what they hold, since their cache already counts the step;
+* a sequence ends on a stop token (which stays in its output) or after ``max_tokens`` tokens.
 """
 
 from __future__ import annotations
 
 import dataclasses
 import time
-from typing import Callable, Dict, List, Optional, Sequence as Seq
-
-import torch
+from typing import Callable, Dict, List, Optional, Sequence as Seq, Tuple
 
 from ..cache.manager import CacheManager
 from ..errors import CapacityError, InvalidArgument
@@ -30,7 +27,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import DeviceSampler
 from .batch import StepEntry
 from .runner import ModelRunner
-from .scheduler import BatchScheduler, ScheduledBatch, SchedulerConfig
+from .scheduler import BatchScheduler, SchedulerConfig, StepPlan
 from .sequence import FinishReason, SeqState, Sequence
 from .serving import ServingConfig
 
@@ -41,7 +38,7 @@ class EngineStats:
     seqs_scheduled: int = 0      # summed over steps; divided by steps it is the mean batch size
     prefill_tokens: int = 0      # prompt tokens, and tokens recomputed after preemption
     decode_tokens: int = 0
-    step_seconds: float = 0.0    # time in the model's step function
+    step_seconds: float = 0.0    # from handing a batch to the step function until its tokens are read
     preemptions: int = 0
 
 
@@ -53,54 +50,50 @@ class Engine:
         self.serving = serving or ServingConfig()
         self.serving.validate()
         self.scheduler = scheduler or BatchScheduler(cache, SchedulerConfig(serving=self.serving))
-        self.stop_tokens = set(int(t) for t in stop_tokens)
+        self.stop_tokens = frozenset(int(t) for t in stop_tokens)
         self.runner = ModelRunner(model, cache, max_seq_len, use_graphs=use_graphs)
         self.sampler = DeviceSampler(model.device)
         self.sequences: Dict[int, Sequence] = {}
-        self.on_token: Optional[Callable[[int, int], None]] = None
+        self.on_token: Optional[Callable[[int, int], None]] = None     # (sequence id, token), as each token is known
         self._stats = EngineStats()
-        self._next_id = 0
-        self._stepping = False
+        self._ids = 0
+        self._inside_step = False
 
     # -------------------------------------------------------------- requests
+    def _token_limits(self) -> List[Tuple[int, str]]:
+        """The three ceilings on a sequence's length (prompt and generated together), each with its name."""
+        page = self.cache.block_size
+        return [(self.model.spec.max_positions, "the model's context"),
+                (self.cache.num_blocks * page, f"the cache of {self.cache.num_blocks} pages (see --kv-mem)"),
+                (self.runner.max_blocks_per_seq * page, f"a block-table row of {self.runner.max_blocks_per_seq} pages")]
+
     def add_request(self, prompt: Seq[int], params: Optional[SamplingParams] = None) -> int:
         params = dataclasses.replace(params) if params is not None else SamplingParams()
         params.validate()
         prompt = [int(t) for t in prompt]
         if not prompt:
-            raise InvalidArgument("prompt is empty")
+            raise InvalidArgument("a request needs at least one prompt token")
         vocab = self.model.spec.vocab_size
-        for t in prompt:
-            if not 0 <= t < vocab:
-                raise InvalidArgument(f"prompt token {t} outside vocabulary of {vocab}")
-        # Most tokens (prompt included) one sequence can hold: the context, the whole pool, one block-table row.
-        bs = self.cache.block_size
-        context_cap = self.model.spec.max_positions
-        pool_cap = self.cache.num_blocks * bs
-        row_cap = self.runner.max_blocks_per_seq * bs
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            bad = next(t for t in prompt if not 0 <= t < vocab)
+            raise InvalidArgument(f"prompt token {bad} is not in the vocabulary of {vocab}")
         n = len(prompt)
-        if n >= context_cap:
-            raise CapacityError(f"prompt of {n} tokens leaves no room to generate in the model context of {context_cap}")
-        if n >= pool_cap:
-            raise CapacityError(
-                f"prompt of {n} tokens plus one generated token needs {self.cache.blocks_for(n + 1)} KV blocks "
-                f"but the cache holds {self.cache.num_blocks}; raise --kv-mem")
-        if n >= row_cap:
-            raise CapacityError(
-                f"prompt of {n} tokens needs {self.cache.blocks_for(n + 1)} KV blocks but a sequence may hold "
-                f"{self.runner.max_blocks_per_seq}")
-        params.max_tokens = min(params.max_tokens, min(context_cap, pool_cap, row_cap) - n)
-        seq = Sequence(self._next_id, prompt, params, self.cache.new_request())
-        self._next_id += 1
-        self.scheduler.add(seq)
+        ceiling, what = min(self._token_limits(), key=lambda limit: limit[0])    # ties: the first named
+        if n + 1 > ceiling:
+            raise CapacityError(f"a prompt of {n} tokens and one generated token make {n + 1}; {what} holds "
+                                f"{ceiling}")
+        params.max_tokens = min(params.max_tokens, ceiling - n)
+        seq = Sequence(self._ids, prompt, params, self.cache.new_request())
+        self._ids += 1
         self.sequences[seq.id] = seq
+        self.scheduler.add(seq)
         return seq.id
 
     def sequence(self, seq_id: int) -> Sequence:
-        try:
-            return self.sequences[seq_id]
-        except KeyError:
-            raise InvalidArgument(f"no sequence with id {seq_id}") from None
+        seq = self.sequences.get(seq_id)
+        if seq is None:
+            raise InvalidArgument(f"the engine knows no sequence {seq_id}")
+        return seq
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()
@@ -108,150 +101,151 @@ class Engine:
     def cancel(self, seq_id: int) -> None:
         seq = self.sequence(seq_id)
         if seq.state != SeqState.FINISHED:
-            self._finish(seq, FinishReason.CANCELLED)
+            self._end(seq, FinishReason.CANCELLED)
 
     def release(self, seq_id: int) -> None:
-        if self._stepping:
-            raise InvalidArgument(f"cannot release sequence {seq_id} during a step")
+        """Forgets a finished sequence (its tokens with it)."""
+        if self._inside_step:
+            raise InvalidArgument(f"sequence {seq_id} cannot be released from inside a step")
         if self.sequence(seq_id).state != SeqState.FINISHED:
-            raise InvalidArgument(f"sequence {seq_id} is still running")
+            raise InvalidArgument(f"sequence {seq_id} has not finished; cancel it first")
         del self.sequences[seq_id]
 
     def stats(self) -> EngineStats:
-        s = dataclasses.replace(self._stats)
-        s.preemptions = self.scheduler.num_preemptions
-        return s
+        return dataclasses.replace(self._stats, preemptions=self.scheduler.num_preemptions)
 
-    # ------------------------------------------------------------------ step
-    def _check_batch(self, batch: ScheduledBatch) -> None:
-        """A scheduler's mistake must fail loudly before any compute or progress (engine.cpp:65-92)."""
-        if len(batch.seqs) > self.serving.max_seqs:
-            raise InvalidArgument(f"scheduler gave {len(batch.seqs)} sequences; a step allows at most {self.serving.max_seqs}")
-        seen = set()
-        total = 0
-        for s in batch.seqs:
-            seq = s.seq
-            if s.num_tokens <= 0 or s.num_tokens > seq.num_pending:
-                raise InvalidArgument(
-                    f"scheduler gave sequence {seq.id} {s.num_tokens} tokens; it has {seq.num_pending} pending")
-            if id(seq) in seen:
-                raise InvalidArgument(f"scheduler gave sequence {seq.id} twice in one step")
-            seen.add(id(seq))
-            end = seq.num_computed + s.num_tokens
-            need = self.cache.blocks_for(end)
-            for g in self.cache.plan.paged_groups:
-                have = len(seq.cache.tables[g])
-                if have < need or have > self.runner.max_blocks_per_seq:
-                    raise InvalidArgument(
-                        f"sequence {seq.id} has {have} KV blocks reserved; {end} tokens need {need} and a row holds "
-                        f"at most {self.runner.max_blocks_per_seq}")
-            total += s.num_tokens
-        if total > self.serving.max_tokens_per_step:
-            raise InvalidArgument(f"scheduler gave {total} tokens; a step allows at most {self.serving.max_tokens_per_step}")
-
-    def step(self) -> None:
-        if self._stepping:
-            raise InvalidArgument("step() called during a step (e.g. from a token callback)")
-        batch = self.scheduler.schedule()
-        if not batch:
-            return
-        self._stepping = True
-        try:
-            self._run(batch)
-        finally:
-            self._stepping = False
-
-    def _run(self, batch: ScheduledBatch) -> None:
-        sampled: List[Sequence] = []
-        prefill_tokens = decode_tokens = 0
-        try:
-            self._check_batch(batch)
-            entries = []
-            for s in batch.seqs:
-                seq = s.seq
-                begin, end = seq.num_computed, seq.num_computed + s.num_tokens
-                # A decode is the single newest token of a sequence that was already decoding; a prompt
-                # portion, or tokens recomputed after preemption, is prefill (engine.cpp:121-124).
-                if seq.state == SeqState.DECODING and s.num_tokens == 1:
-                    decode_tokens += 1
-                else:
-                    prefill_tokens += s.num_tokens
-                want = ()
-                if end == len(seq.tokens):     # a sequence samples once its whole pending input is cached
-                    want = (s.num_tokens - 1,)
-                    sampled.append(seq)
-                entries.append(StepEntry(seq.cache, begin, seq.tokens[begin:end], want))
-            started = time.perf_counter()
-            logits = self.runner.step(entries)      # queued on the GPU; sampling below is queued right behind it
-            self._stats.steps += 1
-            self._stats.seqs_scheduled += len(batch.seqs)
-            self._stats.prefill_tokens += prefill_tokens
-            self._stats.decode_tokens += decode_tokens
-        except BaseException:
-            # The step never ran: give back what the scheduler reserved for it, and let it be scheduled again.
-            for s in batch.seqs:
-                self.cache.truncate(s.seq.cache, s.seq.num_computed)
-            self.scheduler.abandon(batch)
-            raise
-
-        for s in batch.seqs:
-            s.seq.num_computed += s.num_tokens
-            self.cache.trim(s.seq.cache, s.seq.num_computed)
-        self.scheduler.complete(batch)
-        if not sampled:
-            self._stats.step_seconds += time.perf_counter() - started
-            return
-
-        try:
-            tokens = self.sampler.sample_rows(logits, [q.params for q in sampled], [q.rng for q in sampled])
-        except BaseException:
-            for seq in sampled:
-                if seq.state != SeqState.FINISHED:
-                    self._finish(seq, FinishReason.ERROR)
-            raise
-        self._stats.step_seconds += time.perf_counter() - started   # reading the tokens waited for the GPU
-        for i, seq in enumerate(sampled):
-            if seq.state == SeqState.FINISHED:      # cancelled by an earlier token callback of this step
-                continue
-            token = tokens[i]
-            try:
-                seq.tokens.append(token)
-                seq.state = SeqState.DECODING
-                if self.on_token is not None:
-                    self.on_token(seq.id, token)
-            except BaseException:
-                # Sequences after it already count this step as computed but will never get its token.
-                for later in sampled[i:]:
-                    if later.state != SeqState.FINISHED:
-                        self._finish(later, FinishReason.ERROR)
-                raise
-            if seq.state == SeqState.FINISHED:      # its own callback cancelled it
-                continue
-            if token in self.stop_tokens:
-                self._finish(seq, FinishReason.STOP)
-            elif seq.num_generated >= seq.params.max_tokens:
-                self._finish(seq, FinishReason.LENGTH)
-
-    def _finish(self, seq: Sequence, reason: FinishReason) -> None:
+    def _end(self, seq: Sequence, reason: FinishReason) -> None:
         seq.state = SeqState.FINISHED
         seq.finish_reason = reason
         self.cache.release(seq.cache)
         self.scheduler.finish(seq)
 
+    # ------------------------------------------------------------------ step
+    def step(self) -> None:
+        if self._inside_step:
+            raise InvalidArgument("step() was called from inside a step (a token callback?)")
+        plan = self.scheduler.schedule()
+        if not plan:
+            return
+        self._inside_step = True
+        try:
+            self._carry_out(plan)
+        finally:
+            self._inside_step = False
+
+    def _entries_of(self, plan: StepPlan):
+        """The plan as batch entries, checked on the way: a planner's mistake stops here, before any compute.
+
+        Returns (entries, the sequences that sample after this step, prompt tokens, decoded tokens).
+        """
+        serving = self.serving
+        if len(plan.seqs) > serving.max_seqs or plan.total_tokens > serving.max_tokens_per_step:
+            raise InvalidArgument(f"the plan holds {len(plan.seqs)} sequences and {plan.total_tokens} tokens; a step "
+                                  f"takes {serving.max_seqs} and {serving.max_tokens_per_step}")
+        entries, sampling, seen = [], [], set()
+        prompt_tokens = decoded_tokens = 0
+        groups = self.cache.plan.paged_groups
+        row_pages = self.runner.max_blocks_per_seq
+        for share in plan.seqs:
+            seq, n = share.seq, share.num_tokens
+            if not 0 < n <= seq.num_pending or id(seq) in seen:
+                raise InvalidArgument(f"the plan gives sequence {seq.id} {n} tokens (it has {seq.num_pending} to run), "
+                                      f"or names it twice")
+            seen.add(id(seq))
+            first, last = seq.num_computed, seq.num_computed + n
+            pages = self.cache.blocks_for(last)
+            for g in groups:
+                held = len(seq.cache.tables[g])
+                if not pages <= held <= row_pages:
+                    raise InvalidArgument(f"sequence {seq.id} holds {held} pages of cache group {g}: {last} tokens "
+                                          f"take {pages}, a block-table row {row_pages}")
+            # One new token of a sequence that has sampled before is a decode; everything else (prompt portions,
+            # tokens computed again after an eviction) counts as prefill (engine.cpp:121-124).
+            if n == 1 and seq.state == SeqState.DECODING:
+                decoded_tokens += 1
+            else:
+                prompt_tokens += n
+            if last == len(seq.tokens):          # all it has is cached after this step: it samples
+                entries.append(StepEntry(seq.cache, first, seq.tokens[first:last], (n - 1,)))
+                sampling.append(seq)
+            else:
+                entries.append(StepEntry(seq.cache, first, seq.tokens[first:last], ()))
+        return entries, sampling, prompt_tokens, decoded_tokens
+
+    def _carry_out(self, plan: StepPlan) -> None:
+        try:
+            entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan)
+            began = time.perf_counter()
+            logits = self.runner.step(entries)        # queued on the GPU; the sampling kernels queue right behind
+        except BaseException:
+            # Nothing of the step counts: the pages reserved for it go back and the plan's sequences are free
+            # to be planned again.
+            for share in plan.seqs:
+                self.cache.truncate(share.seq.cache, share.seq.num_computed)
+            self.scheduler.abandon(plan)
+            raise
+        stats = self._stats
+        stats.steps += 1
+        stats.seqs_scheduled += len(plan.seqs)
+        stats.prefill_tokens += prompt_tokens
+        stats.decode_tokens += decoded_tokens
+        windows = self.cache.has_windows
+        for share in plan.seqs:
+            seq = share.seq
+            seq.num_computed += share.num_tokens
+            if windows:
+                self.cache.trim(seq.cache, seq.num_computed)     # pages a window has passed go back now
+        self.scheduler.complete(plan)
+        tokens: List[int] = []
+        if sampling:
+            try:
+                tokens = self.sampler.sample_rows(logits, [s.params for s in sampling], [s.rng for s in sampling])
+            except BaseException:
+                self._end_all(sampling, FinishReason.ERROR)
+                raise
+        stats.step_seconds += time.perf_counter() - began     # reading the tokens waited for the GPU
+        if sampling:
+            self._deliver(sampling, tokens)
+
+    def _end_all(self, seqs: Seq[Sequence], reason: FinishReason) -> None:
+        for seq in seqs:
+            if seq.state != SeqState.FINISHED:
+                self._end(seq, reason)
+
+    def _deliver(self, sampling: List[Sequence], tokens: List[int]) -> None:
+        callback, stop = self.on_token, self.stop_tokens
+        for i, seq in enumerate(sampling):
+            if seq.state == SeqState.FINISHED:       # cancelled by a callback earlier in this loop
+                continue
+            token = tokens[i]
+            seq.tokens.append(token)
+            seq.state = SeqState.DECODING
+            if callback is not None:
+                try:
+                    callback(seq.id, token)
+                except BaseException:
+                    # The sequences from here on have this step in their cache and will never see its token.
+                    self._end_all(sampling[i:], FinishReason.ERROR)
+                    raise
+                if seq.state == SeqState.FINISHED:   # its own callback cancelled it
+                    continue
+            if token in stop:
+                self._end(seq, FinishReason.STOP)
+            elif len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:
+                self._end(seq, FinishReason.LENGTH)
+
     # -------------------------------------------------------------- generate
     def generate(self, prompt: Seq[int], params: Optional[SamplingParams] = None) -> List[int]:
-        """Runs one request to completion; returns its generated tokens, a final stop token included."""
+        """One request from its prompt to its end; returns the generated tokens (a stop token included)."""
         seq_id = self.add_request(prompt, params)
+        seq = self.sequences[seq_id]
         try:
-            while self.sequence(seq_id).state != SeqState.FINISHED:
+            while seq.state != SeqState.FINISHED:
                 self.step()
         except BaseException:
-            seq = self.sequences.get(seq_id)
-            if seq is not None:
-                if seq.state != SeqState.FINISHED:
-                    self._finish(seq, FinishReason.ERROR)
-                del self.sequences[seq_id]
+            if seq.state != SeqState.FINISHED:
+                self._end(seq, FinishReason.ERROR)
+            self.sequences.pop(seq_id, None)
             raise
-        out = self.sequence(seq_id).generated
         self.release(seq_id)
-        return out
+        return seq.generated

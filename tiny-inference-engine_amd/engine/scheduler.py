@@ -1,33 +1,45 @@
-"""Continuous batching with chunked prefill, admission by free pages, and preemption by recompute.
+"""Which request runs how many tokens in the next step.
 
-The policy is the reference's ``BatchScheduler`` (``src/engine/batch_scheduler.cpp:78-174``).
-Each step, under the token budget, the cap on sequences and the free pages:
+The policy is the one of the reference's scheduler (``src/engine/batch_scheduler.cpp:78-174``:
+continuous batching, prompts in portions, admission by free pages, preemption by recompute); the
+code is organised around three small things of its own:
 
-1. every decoding sequence (one pending token) advances, oldest first. One that needs a page
-   when none is free preempts the newest sequence admitted after it that is idle and holds
-   pages; if there is none but a newer one is in flight it sits this step out; it preempts
-   itself only when no newer sequence holds pages or is in flight;
-2. partially prefilled sequences continue in admission order with as much as budget, chunk cap
-   and free pages allow;
-3. waiting sequences are admitted in policy order (first come first served, or least remaining
-   work first with aging). A watermark of pages stays free for running sequences to grow into,
-   and admission stops at the first sequence that does not fit, so a large request is not
-   overtaken forever. A sequence preempted in this step waits at least one step;
-4. if nothing could run, the oldest running sequence preempts newer ones until it can.
+* a ``StepPlan``: the shares (sequence, number of tokens) of one step;
+* a ``_Budget``: what a step may still take, in tokens and in sequences;
+* ``_make_room``: the one place that decides what happens when pages run out.
 
-When pages run out the answer is therefore preemption by recompute: the victim's pages and state
-slot go back, its tokens (prompt and generated) stay, and on re-admission all of them are
-prefilled again before it samples its next token. The oldest running sequence is never
-preempted, so it always finishes.
+A step is planned in rounds, each a method, each spending the same budget:
 
-Deciding a step (``schedule``) is separate from finishing it (``complete`` / ``abandon``); a
-sequence in a batch that is neither completed nor abandoned is not scheduled again.
+``_advance_decoders``  every sequence with exactly one token to run (a decode) goes first, oldest
+                       first, so that a running request never waits behind new prompts;
+``_continue_prompts``  sequences in the middle of their prompt take the next portion, as large as the
+                       budget, the portion cap (``prefill_chunk``) and the free pages allow;
+``_admit``             waiting sequences enter in policy order (first come first served, or least
+                       remaining work first where a waiting step counts ``aging`` tokens). Admission
+                       keeps ``watermark`` pages free for the running ones to grow into and stops at the
+                       first sequence that does not fit: a large request is not overtaken for ever;
+``_unblock_oldest``    only if all of that produced nothing: the oldest idle running sequence takes
+                       pages from newer ones until it can move, so the engine never stalls.
+
+When pages run out (``_make_room``), the sequence that needs one evicts the NEWEST sequence admitted
+after it that is idle and holds pages: the victim's pages and state slot go back, its tokens
+(prompt and generated) stay, and it waits to be admitted and computed again from its first token.
+With nobody to evict but a newer sequence still in an unfinished step, the sequence sits this step
+out (that step's end will free or advance something); otherwise it evicts itself. Sequences older
+than the one in need are never touched, so the oldest running sequence always finishes.
+
+When the engine is in its steady state - nobody waiting, every running sequence decoding, pages
+for all of them - the rounds would hand every sequence one token; ``_steady_decode`` sees that
+without walking through them.
+
+Deciding a step (``schedule``) is separate from ending it (``complete`` after it ran, ``abandon`` if
+it never did): a sequence of a planned step that has not ended is "in flight" and is left alone.
 """
 
 from __future__ import annotations
 
 import dataclasses
-from typing import List, Optional
+from typing import Dict, List, Optional
 
 from ..cache.manager import CacheManager
 from ..errors import InvalidArgument
@@ -36,11 +48,12 @@ from .serving import ServingConfig
 
 FCFS = "fcfs"
 SRPT_AGING = "srpt-aging"
+POLICIES = (FCFS, SRPT_AGING)
 
 
 def parse_policy(name: str) -> str:
-    if name not in (FCFS, SRPT_AGING):
-        raise InvalidArgument(f"scheduling policy must be fcfs or srpt-aging, got '{name}'")
+    if name not in POLICIES:
+        raise InvalidArgument(f"unknown scheduling policy '{name}': choose one of {', '.join(POLICIES)}")
     return name
 
 
@@ -48,30 +61,59 @@ def parse_policy(name: str) -> str:
 class SchedulerConfig:
     serving: ServingConfig = dataclasses.field(default_factory=ServingConfig)
     policy: str = SRPT_AGING
-    aging: int = 16                # srpt-aging: priority (in tokens) gained per step waited
-    watermark_blocks: int = -1     # pages admission leaves free; -1 = max(1, 1% of the pool)
+    aging: int = 16                # srpt-aging: tokens of priority a sequence gains per step it waits
+    watermark_blocks: int = -1     # pages that admission leaves free; -1 picks max(1, 1 % of the pool)
 
 
-@dataclasses.dataclass
-class ScheduledSeq:
-    seq: Sequence
-    num_tokens: int
+class Share:
+    """One sequence's part of a step."""
+
+    __slots__ = ("seq", "num_tokens")
+
+    def __init__(self, seq: Sequence, num_tokens: int):
+        self.seq = seq
+        self.num_tokens = num_tokens
 
 
-@dataclasses.dataclass
-class ScheduledBatch:
-    id: int = 0
-    seqs: List[ScheduledSeq] = dataclasses.field(default_factory=list)
+class StepPlan:
+    """The shares of one step, in the order they were granted."""
+
+    def __init__(self, plan_id: int = 0):
+        self.id = plan_id
+        self.seqs: List[Share] = []
+        self._tokens: Dict[int, int] = {}      # id(sequence) -> tokens granted
+        self.total_tokens = 0
+
+    def grant(self, seq: Sequence, num_tokens: int) -> None:
+        self.seqs.append(Share(seq, num_tokens))
+        self._tokens[id(seq)] = num_tokens
+        self.total_tokens += num_tokens
+
+    def tokens_of(self, seq: Sequence) -> int:
+        return self._tokens.get(id(seq), 0)
 
     def __bool__(self) -> bool:
         return bool(self.seqs)
 
-    def tokens_of(self, seq: Sequence) -> int:
-        return next((s.num_tokens for s in self.seqs if s.seq is seq), 0)
+    def __len__(self) -> int:
+        return len(self.seqs)
 
-    @property
-    def total_tokens(self) -> int:
-        return sum(s.num_tokens for s in self.seqs)
+
+class _Budget:
+    """What the step being planned may still take."""
+
+    __slots__ = ("tokens", "seats")
+
+    def __init__(self, tokens: int, seats: int):
+        self.tokens = tokens
+        self.seats = seats
+
+    def spent(self) -> bool:
+        return self.tokens <= 0 or self.seats <= 0
+
+
+# outcomes of _make_room
+_ROOM, _SIT_OUT, _EVICTED_ITSELF, _NO_ROOM = range(4)
 
 
 class BatchScheduler:
@@ -81,169 +123,193 @@ class BatchScheduler:
         self.config.serving.validate()
         parse_policy(self.config.policy)
         if self.config.aging < 0:
-            raise InvalidArgument(f"aging must be non-negative, got {self.config.aging}")
-        wm = self.config.watermark_blocks
-        if wm < -1 or wm >= cache.num_blocks:
-            raise InvalidArgument(
-                f"watermark of {wm} blocks must be -1 (auto) or below the pool's {cache.num_blocks} blocks")
-        self.watermark = wm if wm >= 0 else max(1, cache.num_blocks // 100)
+            raise InvalidArgument(f"aging counts tokens per waited step and cannot be negative ({self.config.aging})")
+        asked = self.config.watermark_blocks
+        if asked < -1 or asked >= cache.num_blocks:
+            raise InvalidArgument(f"a watermark of {asked} pages is neither -1 (choose for me) nor smaller than "
+                                  f"the pool of {cache.num_blocks} pages")
+        self.watermark = asked if asked >= 0 else max(1, cache.num_blocks // 100)
         self.waiting: List[Sequence] = []
-        self.running: List[Sequence] = []      # admission order, oldest first
-        self._in_flight = set()
-        self._step = 0
-        self._next_batch_id = 1
+        self.running: List[Sequence] = []      # in order of admission: the oldest first
         self.num_preemptions = 0
+        self.steady_steps = 0                  # steps planned by _steady_decode
+        self._clock = 0                        # counts planned steps; waiting times are measured in it
+        self._next_plan_id = 1
 
     # ------------------------------------------------------------- interface
     def add(self, seq: Sequence) -> None:
         seq.state = SeqState.WAITING
-        seq.waiting_since_step = self._step
+        seq.waiting_since_step = self._clock
+        seq.in_flight = False
         self.waiting.append(seq)
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting) or bool(self.running)
 
-    def complete(self, batch: ScheduledBatch) -> None:
-        for s in batch.seqs:
-            self._in_flight.discard(id(s.seq))
+    def complete(self, plan: StepPlan) -> None:
+        """The step ran: its sequences may be planned again."""
+        for share in plan.seqs:
+            share.seq.in_flight = False
 
-    def abandon(self, batch: ScheduledBatch) -> None:
-        for s in batch.seqs:
-            self._in_flight.discard(id(s.seq))
+    def abandon(self, plan: StepPlan) -> None:
+        """The step never ran (the caller has given its pages back): its sequences may be planned again."""
+        for share in plan.seqs:
+            share.seq.in_flight = False
 
     def finish(self, seq: Sequence) -> None:
-        self.waiting = [s for s in self.waiting if s is not seq]
-        self.running = [s for s in self.running if s is not seq]
-        self._in_flight.discard(id(seq))
+        """Forgets a sequence wherever it is; the caller gives back what it holds."""
+        for queue in (self.waiting, self.running):
+            for i, other in enumerate(queue):
+                if other is seq:
+                    del queue[i]
+                    break
+        seq.in_flight = False
 
-    # --------------------------------------------------------------- helpers
-    def _busy(self, seq: Sequence) -> bool:
-        return id(seq) in self._in_flight
+    # -------------------------------------------------------------- planning
+    def schedule(self) -> StepPlan:
+        self._clock += 1
+        plan = StepPlan(self._next_plan_id)
+        self._next_plan_id += 1
+        serving = self.config.serving
+        budget = _Budget(serving.max_tokens_per_step, serving.max_seqs)
+        if not self._steady_decode(plan, budget):
+            self._advance_decoders(plan, budget)
+            self._continue_prompts(plan, budget)
+            self._admit(plan, budget)
+            if not plan:
+                self._unblock_oldest(plan, budget)
+        for share in plan.seqs:
+            share.seq.in_flight = True
+        return plan
 
-    def _order_key(self, seq: Sequence):
-        if self.config.policy == SRPT_AGING:
-            score = seq.num_pending - self.config.aging * (self._step - seq.waiting_since_step)
-            return (score, seq.waiting_since_step, seq.id)
-        return (0, seq.waiting_since_step, seq.id)
+    def _grant(self, plan: StepPlan, budget: _Budget, seq: Sequence, num_tokens: int) -> None:
+        if not self.cache.reserve(seq.cache, seq.num_computed + num_tokens):
+            raise InvalidArgument(f"internal error of the scheduler: it granted sequence {seq.id} {num_tokens} tokens "
+                                  f"after counting pages for them, and the cache has no room for them")
+        plan.grant(seq, num_tokens)
+        budget.tokens -= num_tokens
+        budget.seats -= 1
 
-    def _fit(self, seq: Sequence, want: int) -> int:
-        return self.cache.fit(seq.cache, seq.num_computed, want)
-
-    def _chunk(self, seq: Sequence, budget: int) -> int:
-        n = min(seq.num_pending, budget)
+    def _portion(self, seq: Sequence, budget: _Budget) -> int:
+        """How much of its pending input a sequence would take if pages were no concern."""
         cap = self.config.serving.prefill_chunk
+        n = min(seq.num_pending, budget.tokens)
         return min(n, cap) if cap > 0 else n
 
-    def _newest_after(self, index: int) -> Optional[Sequence]:
-        """The newest running sequence admitted after ``index`` that is idle and holds pages."""
-        for j in range(len(self.running) - 1, index, -1):
-            cand = self.running[j]
-            if not self._busy(cand) and cand.cache.num_held() > 0:
-                return cand
-        return None
+    def _steady_decode(self, plan: StepPlan, budget: _Budget) -> bool:
+        """Every running sequence decodes, nobody waits, and there is a page for each that needs one."""
+        running = self.running
+        if self.waiting or not running or len(running) > min(budget.seats, budget.tokens):
+            return False
+        block_size = self.cache.block_size
+        at_page_edge = 0
+        for seq in running:
+            if seq.in_flight or len(seq.tokens) - seq.num_computed != 1:
+                return False
+            if seq.num_computed % block_size == 0:
+                at_page_edge += 1
+        if at_page_edge and not self.cache.has_free_pages(at_page_edge):
+            return False
+        for seq in running:
+            if seq.num_computed % block_size == 0:     # the others' last page has room: nothing to reserve
+                self._grant(plan, budget, seq, 1)
+            else:
+                plan.grant(seq, 1)
+        self.steady_steps += 1
+        return True
 
-    def _newer_busy(self, index: int) -> bool:
-        return any(self._busy(s) for s in self.running[index + 1:])
-
-    def _preempt(self, seq: Sequence) -> None:
-        self.cache.release(seq.cache)
-        seq.num_computed = 0               # its tokens stay and are recomputed on re-admission
-        seq.state = SeqState.WAITING
-        seq.waiting_since_step = self._step
-        seq.num_preemptions += 1
-        self.num_preemptions += 1
-        self.running = [s for s in self.running if s is not seq]
-        self.waiting.append(seq)
-
-    # -------------------------------------------------------------- schedule
-    def schedule(self) -> ScheduledBatch:
-        self._step += 1
-        batch = ScheduledBatch(id=self._next_batch_id)
-        self._next_batch_id += 1
-        serving = self.config.serving
-        budget = serving.max_tokens_per_step
-
-        def full() -> bool:
-            return budget == 0 or len(batch.seqs) == serving.max_seqs
-
-        def take(seq: Sequence, n: int) -> None:
-            nonlocal budget
-            if not self.cache.reserve(seq.cache, seq.num_computed + n):
-                raise InvalidArgument(
-                    f"scheduler bug: {n} tokens of sequence {seq.id} do not fit the blocks it counted")
-            batch.seqs.append(ScheduledSeq(seq, n))
-            budget -= n
-
-        # 1. decodes, oldest first
-        i = 0
-        while i < len(self.running) and not full():
-            seq = self.running[i]
-            if self._busy(seq) or seq.num_pending != 1:
-                i += 1
-                continue
-            preempted_self = deferred = False
-            while self._fit(seq, 1) == 0:
-                victim = self._newest_after(i)
-                if victim is None and self._newer_busy(i):
-                    deferred = True
-                    break
-                self._preempt(victim if victim is not None else seq)
-                if victim is None:
-                    preempted_self = True
-                    break
-            if deferred:
-                i += 1
-                continue
-            if preempted_self:
-                continue                   # running[i] is now the next sequence
-            take(seq, 1)
-            i += 1
-
-        # 2. partial prefills continue in admission order
+    def _advance_decoders(self, plan: StepPlan, budget: _Budget) -> None:
         for seq in list(self.running):
-            if full():
-                break
-            if self._busy(seq) or seq.num_pending <= 1 or batch.tokens_of(seq):
+            if budget.spent():
+                return
+            if seq.in_flight or seq.num_pending != 1 or seq.state == SeqState.WAITING:   # WAITING: evicted just now
                 continue
-            n = self._fit(seq, self._chunk(seq, budget))
-            if n > 0:
-                take(seq, n)
+            if self._make_room(seq, 1, may_give_way=True) == _ROOM:
+                self._grant(plan, budget, seq, 1)
 
-        # 3. admission in policy order
-        self.waiting.sort(key=self._order_key)
-        admitted = []
+    def _continue_prompts(self, plan: StepPlan, budget: _Budget) -> None:
+        for seq in list(self.running):
+            if budget.spent():
+                return
+            if seq.in_flight or seq.num_pending <= 1 or plan.tokens_of(seq):
+                continue
+            n = self.cache.fit(seq.cache, seq.num_computed, self._portion(seq, budget))
+            if n > 0:
+                self._grant(plan, budget, seq, n)
+
+    def _priority(self, seq: Sequence):
+        waited = self._clock - seq.waiting_since_step
+        work = seq.num_pending - self.config.aging * waited if self.config.policy == SRPT_AGING else 0
+        return (work, seq.waiting_since_step, seq.id)
+
+    def _admit(self, plan: StepPlan, budget: _Budget) -> None:
+        if not self.waiting:
+            return
+        self.waiting.sort(key=self._priority)
+        entered = 0
         for seq in self.waiting:
-            if full() or len(self.running) >= serving.max_seqs:
+            if budget.spent() or len(self.running) >= self.config.serving.max_seqs:
                 break
-            if seq.num_preemptions > 0 and seq.waiting_since_step == self._step:
-                continue                   # preempted in this very step: waits one step
-            n = self._chunk(seq, budget)
-            keep_free = self.watermark if self.running else 0
-            if not self.cache.can_admit(n, keep_free):
+            if seq.num_preemptions and seq.waiting_since_step == self._clock:
+                continue                       # evicted while this very step was planned: it waits a step
+            n = self._portion(seq, budget)
+            if not self.cache.can_admit(n, self.watermark if self.running else 0):
                 break
             seq.state = SeqState.PREFILLING
             self.running.append(seq)
-            take(seq, n)
-            admitted.append(seq)
-        if admitted:
-            self.waiting = [s for s in self.waiting if not any(s is a for a in admitted)]
+            self._grant(plan, budget, seq, n)
+            entered += 1
+        if entered:
+            self.waiting = [s for s in self.waiting if s.state == SeqState.WAITING]
 
-        # 4. never stall
-        if not batch.seqs:
-            for i, seq in enumerate(self.running):
-                if self._busy(seq):
-                    continue
-                want = self._chunk(seq, budget)
-                while self._fit(seq, want) == 0:
-                    victim = self._newest_after(i)
-                    if victim is None:
-                        break
-                    self._preempt(victim)
-                n = self._fit(seq, want)
-                if n > 0:
-                    take(seq, n)
+    def _unblock_oldest(self, plan: StepPlan, budget: _Budget) -> None:
+        for seq in self.running:
+            if seq.in_flight:
+                continue
+            want = self._portion(seq, budget)
+            self._make_room(seq, want, may_give_way=False)
+            n = self.cache.fit(seq.cache, seq.num_computed, want)
+            if n > 0:
+                self._grant(plan, budget, seq, n)
+            return
+
+    # ------------------------------------------------------------- out of pages
+    def _make_room(self, seq: Sequence, want: int, may_give_way: bool) -> int:
+        """Evicts newer sequences until ``seq`` can run at least one of ``want`` tokens.
+
+        ``may_give_way``: with nobody left to evict, the sequence itself yields - it sits the step out if a
+        newer sequence is in flight, else it is evicted. Without it the answer is just _NO_ROOM.
+        """
+        while self.cache.fit(seq.cache, seq.num_computed, want) == 0:
+            victim, newer_in_flight = None, False
+            for other in reversed(self.running):
+                if other is seq:
+                    break
+                if other.in_flight:
+                    newer_in_flight = True
+                elif self.cache.holds_pages(other.cache):
+                    victim = other
+                    break
+            if victim is not None:
+                self._evict(victim)
+                continue
+            if not may_give_way:
+                return _NO_ROOM
+            if newer_in_flight:
+                return _SIT_OUT
+            self._evict(seq)
+            return _EVICTED_ITSELF
+        return _ROOM
+
+    def _evict(self, seq: Sequence) -> None:
+        self.cache.release(seq.cache)
+        seq.num_computed = 0                   # prompt and generated tokens stay: all are computed again
+        seq.state = SeqState.WAITING
+        seq.waiting_since_step = self._clock
+        seq.num_preemptions += 1
+        self.num_preemptions += 1
+        for i, other in enumerate(self.running):
+            if other is seq:
+                del self.running[i]
                 break
-
-        for s in batch.seqs:
-            self._in_flight.add(id(s.seq))
-        return batch
+        self.waiting.append(seq)

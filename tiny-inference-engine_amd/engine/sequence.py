@@ -40,6 +40,7 @@ class Sequence:
         self.finish_reason = FinishReason.NONE
         self.waiting_since_step = 0            # scheduler step at which it last entered the waiting queue
         self.num_preemptions = 0
+        self.in_flight = False                 # part of a planned step that has neither run nor been abandoned
 
     @property
     def num_generated(self) -> int:

@@ -73,10 +73,30 @@ def sample(logits: np.ndarray, params: SamplingParams, rng: RandomStream) -> int
 
 
 class DeviceSampler:
-    """Samples the rows of one step's logits, on the GPU where the parameters allow it."""
+    """Samples the rows of one step's logits, on the GPU where the parameters allow it.
+
+    The results come back through one pinned host buffer that lives as long as the sampler: a step of
+    greedy rows is one kernel, one copy of ``2 R`` words and one wait."""
+
+    GREEDY, PLAIN, HOST = 0, 1, 2      # argmax kernel / temperature kernel / top-k or top-p on the host
 
     def __init__(self, device):
-        self.device = device
+        self.device = torch.device(device)
+        self._rows = 0
+        self._dev = self._host = None
+
+    def _buffers(self, rows: int):
+        if rows > self._rows:
+            self._rows = max(64, 2 * rows)
+            self._dev = torch.empty(3 * self._rows, dtype=torch.int32, device=self.device)
+            self._host = torch.empty(3 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        return self._dev, self._host
+
+    def _fetch(self, dev: torch.Tensor, host: torch.Tensor, count: int) -> np.ndarray:
+        host[:count].copy_(dev[:count], non_blocking=True)
+        if self.device.type == "cuda":
+            torch.cuda.current_stream(self.device).synchronize()
+        return host.numpy()[:count]
 
     def sample_rows(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                     rngs: Sequence[RandomStream]) -> List[int]:
@@ -85,42 +105,33 @@ class DeviceSampler:
         R = logits.shape[0]
         if R != len(params) or R != len(rngs):
             raise InvalidArgument("one set of sampling parameters and one random stream per row")
-        out = [0] * R
-        greedy_rows = [i for i, p in enumerate(params) if p.greedy]
-        plain_rows = [i for i, p in enumerate(params) if not p.greedy and p.top_k == 0 and p.top_p >= 1.0]
-        host_rows = [i for i in range(R) if i not in set(greedy_rows) and i not in set(plain_rows)]
-        # Kernels work on all rows at once; each kind's result is read where it applies.
-        host_argmax = host_max = None
-        if greedy_rows or plain_rows:
-            # index and maximum side by side in one buffer: one copy to the host, one wait for the GPU
-            both = torch.empty(2 * R, dtype=torch.int32, device=logits.device)
-            kernels.argmax_rows(logits, both[:R], both[R:].view(torch.float32))
-            host = both.cpu().numpy()
-            host_argmax = host[:R]
-            host_max = host[R:].view(np.float32)
-            for i in greedy_rows + plain_rows:
-                if host_argmax[i] < 0:
-                    raise InvalidArgument(f"a logit of row {i} is NaN")
-                if host_max[i] == -np.inf:
-                    raise InvalidArgument(f"all logits of row {i} are -inf")
-            for i in greedy_rows:
-                out[i] = int(host_argmax[i])
-        # A +inf logit is certain and does not consume a random number; the other rows draw one each.
-        drawing = [i for i in plain_rows if host_max[i] != np.inf]
-        for i in plain_rows:
-            out[i] = int(host_argmax[i])
-        if drawing:
-            inv_t = np.ones(R, dtype=np.float32)
-            uniform = np.zeros(R, dtype=np.float64)
-            for i in drawing:
-                inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
-                uniform[i] = rngs[i].unit()
-            drawn = torch.empty(R, dtype=torch.int32, device=logits.device)
-            kernels.sample_rows(logits, torch.from_numpy(inv_t).to(logits.device),
-                                torch.from_numpy(uniform).to(logits.device), drawn)
-            host_drawn = drawn.cpu().numpy()
-            for i in drawing:
-                out[i] = int(host_drawn[i])
-        for i in host_rows:
+        kinds = np.fromiter((self.GREEDY if p.greedy else (self.PLAIN if p.top_k == 0 and p.top_p >= 1.0 else self.HOST)
+                             for p in params), dtype=np.int8, count=R)
+        out = np.zeros(R, dtype=np.int64)
+        on_device = kinds != self.HOST
+        if on_device.any():
+            # Both kernels work on all rows at once; each kind's result is read where it applies. Index and
+            # maximum lie side by side, so one copy brings both.
+            dev, host = self._buffers(R)
+            kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
+            fetched = self._fetch(dev, host, 2 * R)
+            best, top = fetched[:R], fetched[R:].view(np.float32)
+            if (best[on_device] < 0).any():
+                raise InvalidArgument(f"a logit of row {int(np.flatnonzero(on_device & (best < 0))[0])} is NaN")
+            if (top[on_device] == -np.inf).any():
+                raise InvalidArgument(f"all logits of row {int(np.flatnonzero(on_device & (top == -np.inf))[0])} are -inf")
+            out[on_device] = best[on_device]
+            # A +inf logit is certain and consumes no random number; every other temperature row draws one.
+            drawing = np.flatnonzero((kinds == self.PLAIN) & (top != np.inf))
+            if drawing.size:
+                inv_t = np.ones(R, dtype=np.float32)
+                uniform = np.zeros(R, dtype=np.float64)
+                for i in drawing:
+                    inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
+                    uniform[i] = rngs[i].unit()
+                kernels.sample_rows(logits, torch.from_numpy(inv_t).to(logits.device),
+                                    torch.from_numpy(uniform).to(logits.device), dev[2 * R:3 * R])
+                out[drawing] = self._fetch(dev[2 * R:], host[2 * R:], R)[drawing]
+        for i in np.flatnonzero(kinds == self.HOST):
             out[i] = sample(logits[i].cpu().numpy(), params[i], rngs[i])
-        return out
+        return out.tolist()
