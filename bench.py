@@ -1,6 +1,8 @@
 """Decode and prefill throughput of the engine on one MI355X, Qwen3-8B shape, random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --shape 32b                 the same measurements at the Qwen3-32B sizes
+    python bench.py --workload stress           64 requests through the scheduler at the Qwen3-1.7B sizes
 
 Prints ONE JSON line. A "step" is one decode step of the engine (schedule, build the batch, run
 the model, sample greedily) at the default batch of 8 with every sequence near the benchmark
@@ -14,6 +16,12 @@ context length; ``value`` is decoded tokens a second. The same line carries
 
 The sizes are those of a Qwen3-8B config.json; weights are random (N(0, 0.02), norm weights
 1 + U(-0.1, 0.1)) and token ids are uniform, since neither checkpoints nor datasets exist here.
+
+``--workload stress`` is another measurement with a JSON line of its own: 64 requests at once, prompts of
+128 to 2048 tokens, 256 generated tokens each, prompts in portions of 512, a cache of 2 GB - far less than
+the requests need together, so sequences are evicted and computed again. It reports what the reference's
+bench report holds (``src/bench/report.h:29-36``): tokens a second, steps, mean sequences a step,
+preemptions, and percentiles of the time to the first token, between tokens and of whole requests.
 """
 
 import argparse
@@ -27,6 +35,10 @@ QWEN3_8B = {
     "head_dim": 128, "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0,
     "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "max_position_embeddings": 40960,
 }
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+QWEN3_1_7B = dict(QWEN3_8B, num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, intermediate_size=6144,
+                  tie_word_embeddings=True)
+SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "32b": ("Qwen3-32B", QWEN3_32B), "1.7b": ("Qwen3-1.7B", QWEN3_1_7B)}
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0          # MI355X: 8 TB/s
@@ -73,6 +85,27 @@ def prefill_flops(cfg, T, R=1):
     gemm = 2 * T * L * per_layer + 2 * R * V * D
     attention = 2 * T * T * cfg["head_dim"] * cfg["num_attention_heads"] * L   # causal: QK^T and PV over T^2 / 2 pairs
     return gemm + attention
+
+
+def measure_stress(model, cfg, args):
+    """The scheduler under pressure: returns the report of the run as a dict (and checks every page came back)."""
+    from tie_amd.api import create_engine
+    from tie_amd.bench import assign_arrivals, report_json, run_workload, summarize, synthetic_requests
+
+    engine = create_engine(model, kv_mem=args.kv_mem, block_size=BLOCK_SIZE, max_seqs=args.requests,
+                           max_tokens_per_step=512, prefill_chunk=512)
+    requests = synthetic_requests(args.requests, (128, 2048), (256, 256), cfg["vocab_size"], seed=0)
+    assign_arrivals(requests, float("inf"), seed=0)
+    warm = synthetic_requests(4, (600, 700), (8, 8), cfg["vocab_size"], seed=1)       # compiles nothing, but warms up
+    run_workload(engine, warm)
+    log(f"stress: {args.requests} requests, {sum(len(r.prompt) for r in requests)} prompt tokens, "
+        f"a cache of {engine.cache.num_blocks} pages ({engine.cache.num_blocks * BLOCK_SIZE} tokens)")
+    run = run_workload(engine, requests, progress=log)
+    assert engine.cache.num_free() == engine.cache.num_blocks, "a page was not given back"
+    report = report_json(summarize(run))
+    report["kv_blocks"] = engine.cache.num_blocks
+    report["graph_replays"] = engine.runner.graph_replays
+    return report
 
 
 def make_engine(model, batch, context, max_tokens_per_step):
@@ -168,7 +201,13 @@ def main():
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
-    parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the 36 of the shape (0 = all)")
+    parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
+    parser.add_argument("--shape", choices=sorted(SHAPES), default=None,
+                        help="layer sizes: 8b (default), 32b, or 1.7b (the default of --workload stress)")
+    parser.add_argument("--workload", choices=["decode", "stress"], default="decode",
+                        help="decode: the headline measurement; stress: many requests through a small cache")
+    parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
+    parser.add_argument("--kv-mem", type=int, default=2 << 30, help="stress: bytes of cache")
     parser.add_argument("--skip-points", action="store_true", help="skip batch 1, batch 64 and the prefill")
     parser.add_argument("--prefill-only", action="store_true",
                         help="run only the 2048-token prefill (for profiling); prints its figures alone")
@@ -186,14 +225,28 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
-    cfg = dict(QWEN3_8B)
+    shape_name, shape = SHAPES[args.shape or ("1.7b" if args.workload == "stress" else "8b")]
+    cfg = dict(shape)
     layers_of_shape = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    log(f"building {cfg['num_hidden_layers']} layers of the Qwen3-8B shape with random bf16 weights")
+    log(f"building {cfg['num_hidden_layers']} layers of the {shape_name} shape with random bf16 weights")
     started = time.perf_counter()
     model = build_model(cfg)
     log(f"model ready in {time.perf_counter() - started:.1f} s")
+
+    if args.workload == "stress":
+        report = measure_stress(model, cfg, args)
+        print(json.dumps({
+            "metric": f"total tok/s, {args.requests} concurrent requests, {shape_name} bf16, {args.kv_mem >> 20} MB of cache",
+            "value": round(report["total_tok_per_s"], 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"model": f"{shape_name} shape, random weights", "layers": layers_of_shape,
+                       "layers_run": cfg["num_hidden_layers"], "requests": args.requests, "prompt_len": "128:2048",
+                       "output_len": 256, "prefill_chunk": 512, "max_tokens_per_step": 512, "kv_bytes": args.kv_mem,
+                       "kv_block": BLOCK_SIZE, "policy": "srpt-aging", "sampling": "greedy"},
+            "report": report}), flush=True)
+        return 0
 
     if args.prefill_only:
         t = measure_prefill(model, cfg, PREFILL_TOKENS)
@@ -212,12 +265,12 @@ def main():
     log(f"decode batch {args.batch}: {ms_per_step:.3f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s ({replays} replays)")
 
     result = {
-        "metric": "decode tok/s @ batch 8, Qwen3-8B bf16 (plus prefill tok/s @ 2048 and batch 1/64 points)",
+        "metric": f"decode tok/s @ batch {args.batch}, {shape_name} bf16 (plus prefill tok/s @ 2048 and batch 1/64 points)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
-            "model": "Qwen3-8B shape, random weights", "layers": layers_of_shape, "layers_run": cfg["num_hidden_layers"],
+            "model": f"{shape_name} shape, random weights", "layers": layers_of_shape, "layers_run": cfg["num_hidden_layers"],
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
             "global_batch": args.batch, "seq_len": args.context, "kv_block": BLOCK_SIZE, "kv_dtype": "bf16",

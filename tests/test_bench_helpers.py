@@ -1,0 +1,97 @@
+"""The serving benchmark's helpers (no GPU): the workload, the percentiles, the report.
+
+The percentile vectors are those the reference's own test holds (tests/bench/test_report.cpp, read, not run)."""
+
+import json
+import math
+
+import pytest
+
+from tie_amd.bench import (BenchRequest, BenchRun, RequestTiming, assign_arrivals, format_report, parse_range, percentile,
+                           read_requests_jsonl, report_json, summarize, synthetic_requests)
+from tie_amd.errors import InvalidArgument
+
+
+def test_synthetic_requests_are_seeded_and_inside_their_ranges():
+    a = synthetic_requests(50, (3, 9), (2, 5), 100, seed=7)
+    b = synthetic_requests(50, (3, 9), (2, 5), 100, seed=7)
+    c = synthetic_requests(50, (3, 9), (2, 5), 100, seed=8)
+    assert [r.prompt for r in a] == [r.prompt for r in b] and [r.prompt for r in a] != [r.prompt for r in c]
+    assert all(3 <= len(r.prompt) <= 9 and 2 <= r.max_tokens <= 5 and all(0 <= t < 100 for t in r.prompt) for r in a)
+    assert {len(r.prompt) for r in a} == set(range(3, 10))          # both ends of the range are reached
+    assert all(r.arrival == 0.0 for r in a)
+    for bad in ((0, (1, 2), (1, 2), 10), (3, (0, 2), (1, 2), 10), (3, (1, 2), (5, 2), 10), (3, (1, 2), (1, 2), 0)):
+        with pytest.raises(InvalidArgument):
+            synthetic_requests(*bad, seed=0)
+
+
+def test_arrivals_are_poisson_in_order_or_all_at_once():
+    requests = [BenchRequest([1], 1) for _ in range(4000)]
+    assign_arrivals(requests, 50.0, seed=3)
+    times = [r.arrival for r in requests]
+    assert times == sorted(times) and times[0] > 0
+    assert abs(times[-1] / len(times) - 1 / 50.0) < 0.1 / 50.0       # the mean gap is 1 / rate
+    assign_arrivals(requests, math.inf, seed=3)
+    assert all(r.arrival == 0.0 for r in requests)
+    with pytest.raises(InvalidArgument):
+        assign_arrivals(requests, 0.0, seed=3)
+
+
+def test_ranges_and_workload_files(tmp_path):
+    assert parse_range("--prompt-len", "3:9") == (3, 9) and parse_range("--output-len", "7") == (7, 7)
+    for bad in ("9:3", "0", "a:b", "3:", ":3", ""):
+        if bad == "3:":
+            assert parse_range("--x", bad) == (3, 3)
+            continue
+        with pytest.raises(InvalidArgument):
+            parse_range("--x", bad)
+    path = tmp_path / "w.jsonl"
+    path.write_text('{"prompt_ids": [1, 2, 3], "max_tokens": 4}\n\n{"prompt_ids": [5]}\n')
+    got = read_requests_jsonl(str(path), default_max_tokens=9, vocab_size=10)
+    assert [(r.prompt, r.max_tokens) for r in got] == [([1, 2, 3], 4), ([5], 9)]
+    for text, match in (('{"prompt": "hello"}', "tokenizer"), ('{"prompt_ids": []}', "non-empty"), ("[1]", "prompt_ids"),
+                        ('{"prompt_ids": [1], "max_tokens": 0}', "max_tokens"), ("{", "not JSON"), ("\n", "no requests"),
+                        ('{"prompt_ids": [11]}', "vocabulary")):
+        path.write_text(text + "\n")
+        with pytest.raises(InvalidArgument, match=match):
+            read_requests_jsonl(str(path), 9, 10)
+
+
+def test_percentiles_interpolate_between_the_closest_ranks():
+    values = [10.0, 20.0, 30.0, 40.0]
+    assert percentile(values, 0) == 10.0 and percentile(values, 100) == 40.0
+    assert percentile(values, 50) == 25.0                               # rank 1.5
+    assert percentile([3.0, 1.0, 2.0], 50) == 2.0                       # sorted first
+    assert math.isclose(percentile(values, 90), 37.0) and percentile([], 50) == 0.0 and percentile([7.0], 99) == 7.0
+    # the reference's own vectors (tests/bench/test_bench.cpp:67-73, 109-113)
+    assert percentile([], 50) == 0.0 and percentile([4.0], 99) == 4.0 and math.isclose(percentile([1, 2, 3, 4], 50), 2.5)
+    assert percentile([4, 3, 2, 1], 0) == 1.0 and percentile([1, 2, 3, 4], 100) == 4.0
+    assert math.isclose(percentile([1, 2, 3, 4, 5], 90), 4.6)
+    for bad in (100.5, -1, math.nan, 101):
+        with pytest.raises(InvalidArgument):
+            percentile([1, 2, 3] if bad != 101 else [], bad)
+
+
+def test_the_report_sums_up_a_run():
+    run = BenchRun([RequestTiming(0.0, 10, [1.0, 1.5, 2.5]), RequestTiming(0.5, 20, [2.0]), RequestTiming(1.0, 5, [])],
+                   wall_seconds=4.0, steps=8, seqs_scheduled=12, preemptions=2)
+    r = summarize(run)
+    assert (r.requests, r.prompt_tokens, r.output_tokens, r.steps, r.preemptions) == (3, 35, 4, 8, 2)
+    assert r.requests_per_s == 0.75 and r.output_tok_per_s == 1.0 and r.total_tok_per_s == 39 / 4.0
+    assert r.mean_seqs_per_step == 1.5
+    assert r.ttft_ms["p50"] == 1250.0                 # first tokens 1.0 and 1.5 s after arrival
+    assert r.itl_ms["p50"] == 750.0                   # gaps of 0.5 and 1.0 s
+    assert r.e2e_ms["p50"] == 2000.0                  # 2.5 and 1.5 s from arrival to the last token
+    # the reference's own vector (tests/bench/test_bench.cpp:76-94)
+    theirs = summarize(BenchRun([RequestTiming(0.0, 10, [0.1, 0.2, 0.3]), RequestTiming(0.5, 20, [1.0, 1.5])],
+                                wall_seconds=2.0, steps=4, seqs_scheduled=6, preemptions=1))
+    assert (theirs.requests, theirs.output_tokens, theirs.prompt_tokens, theirs.preemptions) == (2, 5, 30, 1)
+    assert math.isclose(theirs.output_tok_per_s, 2.5) and math.isclose(theirs.total_tok_per_s, 17.5)
+    assert math.isclose(theirs.requests_per_s, 1.0) and math.isclose(theirs.mean_seqs_per_step, 1.5)
+    assert math.isclose(theirs.ttft_ms["p50"], 300.0) and math.isclose(theirs.e2e_ms["p50"], 650.0)
+    assert math.isclose(theirs.itl_ms["p50"], 100.0)
+    text = format_report(r)
+    assert "requests 3" in text and "2 preemptions" in text and "1.50 sequences/step" in text and "ttft" in text
+    assert set(json.loads(json.dumps(report_json(r)))) == {
+        "requests", "prompt_tokens", "output_tokens", "wall_s", "requests_per_s", "output_tok_per_s", "total_tok_per_s",
+        "ttft_ms", "itl_ms", "e2e_ms", "mean_seqs_per_step", "steps", "preemptions"}      # report.cpp:73-86

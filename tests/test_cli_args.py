@@ -6,7 +6,7 @@ import sys
 import pytest
 
 from conftest import ROOT
-from tie_amd.cli.args import parse_generate_args, parse_size
+from tie_amd.cli.args import parse_bench_args, parse_generate_args, parse_size
 from tie_amd.errors import InvalidArgument
 
 
@@ -58,7 +58,40 @@ def test_exit_codes_of_the_program():
     assert r.returncode == 1 and "usage: tie generate" in r.stderr
     r = run("--help")
     assert r.returncode == 0 and "usage: tie generate" in r.stdout
-    r = run("bench")
-    assert r.returncode == 1 and "tie: error: unknown command 'bench'" in r.stderr
+    r = run("serve")
+    assert r.returncode == 1 and "tie: error: unknown command 'serve'" in r.stderr
+    r = run("bench", "-m", "x")
+    assert r.returncode == 1 and "tie: error: give exactly one of --prompts or --synthetic" in r.stderr
     r = run("generate", "-m", "/nonexistent", "-p", "1", "--temp", "x")
     assert r.returncode == 1 and "tie: error: --temp expects a finite number" in r.stderr
+
+
+def test_bench_defaults_and_options():
+    """The reference's bench options (src/cli/args.cpp:169-215; tests/cli/test_args.cpp for the scenarios)."""
+    import math
+
+    o = parse_bench_args(["-m", "dir", "--synthetic", "8"])
+    assert o.synthetic == 8 and o.prompt_len == (512, 1024) and o.output_len == (128, 128) and o.max_tokens == 128
+    assert math.isinf(o.rate) and o.sampling.temperature == 0.0 and not o.json
+    assert (o.max_seqs, o.max_tokens_per_step, o.policy, o.aging, o.kv_bytes) == (64, 512, "srpt-aging", 16, 4 << 30)
+    o = parse_bench_args(["-m", "d", "--prompts", "w.jsonl", "--prompt-len", "3:9", "--output-len", "7", "--rate", "2.5",
+                          "--max-tokens", "5", "--json", "--temp", "0.5", "--seed", "4", "--kv-mem", "2G",
+                          "--prefill-chunk", "512", "--max-seqs", "16", "--policy", "fcfs"])
+    assert o.prompts == "w.jsonl" and o.prompt_len == (3, 9) and o.output_len == (7, 7) and o.rate == 2.5
+    assert o.max_tokens == 5 and o.json and o.sampling.temperature == 0.5 and o.sampling.seed == 4
+    assert o.kv_bytes == 2 << 30 and o.prefill_chunk == 512 and o.max_seqs == 16 and o.policy == "fcfs"
+
+
+@pytest.mark.parametrize("argv,match", [
+    (["--synthetic", "4"], "--model is required"), (["-m", "x"], "exactly one of"),
+    (["-m", "x", "--synthetic", "4", "--prompts", "f"], "exactly one of"), (["-m", "x", "--synthetic", "0"], "at least 1"),
+    (["-m", "x", "--synthetic", "4", "--prompt-len", "9:3"], "1 <= A <= B"),
+    (["-m", "x", "--synthetic", "4", "--output-len", "0"], "1 <= A <= B"),
+    (["-m", "x", "--synthetic", "4", "--rate", "0"], "positive or inf"),
+    (["-m", "x", "--synthetic", "4", "--max-tokens", "0"], "positive"),
+    (["-m", "x", "--synthetic", "4", "--max-seqs", "1000"], "max_seqs"),
+    (["-m", "x", "--synthetic", "4", "-p", "1"], "unknown option"),
+])
+def test_bad_bench_arguments_are_refused(argv, match):
+    with pytest.raises(InvalidArgument, match=match):
+        parse_bench_args(argv)

@@ -197,6 +197,59 @@ def test_a_crowded_engine_finishes_everything_twice_the_same_way(model_folders, 
     assert stats.preemptions > 0 and stats.seqs_scheduled > 2 * stats.steps
     second, _ = run()
     assert first == second
+    # And against the plain implementation: every token a greedy request chose is, given the tokens before it,
+    # the plain logits' maximum or within the precision's tolerance of it (a near-tie may fall either way).
+    weights = load_plain_weights(folder)
+    tolerance = 3e-2 if dtype == "bfloat16" else 1e-4
+    checked = 0
+    for (prompt, params), tokens in zip(reqs, first):
+        if params.temperature != 0.0:
+            continue
+        logits = plain.forward(weights, cfg, list(prompt) + tokens)
+        for k, token in enumerate(tokens):
+            row = logits[len(prompt) + k - 1]
+            assert float(row.max() - row[token]) <= tolerance * float(row.abs().max()), \
+                f"token {k} of a greedy request is not what the plain logits favour"
+            checked += 1
+    assert checked > 50
+
+
+def test_a_workload_through_the_bench_runner(model_folders):
+    """``tie bench``'s loop over a pool too small for its requests: every request gets its tokens, evictions
+    happen, the report's counts are the engine's, and every page and sequence is given back."""
+    from tie_amd.bench import assign_arrivals, run_workload, summarize, synthetic_requests
+
+    folder, cfg = model_folders["A"]
+    requests = synthetic_requests(14, (3, 30), (2, 9), cfg["vocab_size"], seed=5)
+    assign_arrivals(requests, float("inf"), seed=5)
+    for late in requests[-3:]:
+        late.arrival = 0.01                                  # three arrive while the others run
+    engine = make_engine(folder, 4, kv_blocks=14, max_seqs=6, max_tokens_per_step=24, prefill_chunk=8)
+    run = run_workload(engine, requests)
+    report = summarize(run)
+    assert report.requests == 14 and report.prompt_tokens == sum(len(r.prompt) for r in requests)
+    assert report.output_tokens == sum(r.max_tokens for r in requests)
+    assert report.preemptions > 0 and report.steps == engine.stats().steps and report.mean_seqs_per_step > 1.5
+    assert engine.cache.num_free() == 14 and not engine.sequences and not engine.has_work()
+    for timing, request in zip(run.requests, requests):
+        times = timing.token_times
+        assert len(times) == request.max_tokens and times == sorted(times) and times[0] >= timing.arrival
+    assert 0 < report.ttft_ms["p50"] <= report.ttft_ms["p99"] <= report.e2e_ms["p99"]
+    # the tokens are those each request generates alone
+    seen = {}
+    engine.on_token = lambda seq_id, token: seen.setdefault(seq_id, []).append(token)
+    ids = [engine.add_request(r.prompt, tie_amd_params(r.max_tokens)) for r in requests]
+    while engine.has_work():
+        engine.step()
+    for sid, r in zip(ids, requests):
+        alone = make_engine(folder, 4, max_seqs=1, max_tokens_per_step=16)
+        assert alone.generate(r.prompt, tie_amd_params(r.max_tokens)) == seen[sid]
+
+
+def tie_amd_params(max_tokens):
+    import tie_amd
+
+    return tie_amd.SamplingParams(max_tokens=max_tokens, temperature=0.0)
 
 
 def test_a_failing_step_is_rolled_back_and_offered_again(model_folders):

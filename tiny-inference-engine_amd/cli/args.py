@@ -1,4 +1,4 @@
-"""Command-line options of ``tie generate`` in the reference's manner (``src/cli/args.cpp``).
+"""Command-line options of ``tie generate`` and ``tie bench`` in the reference's manner (``src/cli/args.cpp``).
 
 Flags are ``--flag value`` pairs with strict numbers; an unknown flag, a missing value or a
 malformed number is an InvalidArgument. Names, meanings and defaults are the reference's where
@@ -6,7 +6,12 @@ it has them: ``-m/--model``, ``-p/--prompt``, ``--temp`` (0.7), ``--top-k`` (20)
 (0.8), ``--seed`` (0), ``--kv-mem`` (4G), ``--max-tokens`` (256), ``--device``. This engine has no
 tokenizer, so the prompt is a list of token ids and stop tokens are given as ids; ``--chat`` and
 ``--no-think`` are refused. Options the reference's ``bench`` command names for the serving shape
-(``--max-seqs``, ``--max-tokens-per-step``, ``--policy``, ``--aging``) are accepted here as well.
+(``--max-seqs``, ``--max-tokens-per-step``, ``--policy``, ``--aging``) are accepted by ``generate`` as well.
+
+``tie bench`` takes the reference's bench options (``args.cpp:169-215``): ``--synthetic N``,
+``--prompt-len A:B`` (512:1024), ``--output-len C:D`` (128), ``--max-tokens`` (128, for workload lines
+without one), ``--rate`` (inf), ``--json``, greedy unless ``--temp`` is given; ``--prompts FILE`` reads
+token ids (``{"prompt_ids": [...]}`` a line), since prompt text would need a tokenizer.
 """
 
 from __future__ import annotations
@@ -14,12 +19,13 @@ from __future__ import annotations
 import dataclasses
 import math
 import re
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 from ..errors import InvalidArgument
 from ..sampling.params import SamplingParams
 
 USAGE = """usage: tie generate -m <model_dir> -p <token ids> [options]
+       tie bench -m <model_dir> (--prompts FILE.jsonl | --synthetic N) [options]
        tie random-weights --config <config.json> --out <model_dir> [--seed S] [--dtype bfloat16|float32]
 
 generate options:
@@ -42,6 +48,17 @@ generate options:
   --prefill-chunk C        most prompt tokens of one sequence per step, 0 = budget only (default 0)
   --policy fcfs|srpt-aging admission order (default srpt-aging)
   --aging N                srpt-aging priority gained per step waited, in tokens (default 16)
+
+bench options (and -m, --device, --dtype, --temp (default 0), --top-k, --top-p, --seed, --kv-mem, --kv-blocks,
+--block-size, --max-seqs, --max-tokens-per-step, --prefill-chunk, --policy, --aging as above; --seed also seeds
+the synthetic workload and the arrivals):
+  --prompts FILE           JSONL, one {"prompt_ids": [...], "max_tokens": N} per line
+  --synthetic N            N requests of random tokens
+  --prompt-len A:B         synthetic prompt lengths (default 512:1024)
+  --output-len C:D         synthetic output lengths (default 128)
+  --max-tokens N           output tokens for JSONL lines without max_tokens (default 128)
+  --rate R                 requests per second, Poisson arrivals; inf = all at once (default inf)
+  --json                   print the report as one JSON object
 """
 
 
@@ -103,82 +120,166 @@ def parse_ids(flag: str, text: str) -> List[int]:
     return [parse_int(flag, p) for p in parts]
 
 
+class _Flags:
+    """Walks ``--flag value`` pairs."""
+
+    def __init__(self, args: Sequence[str]):
+        self.args = list(args)
+        self.i = 0
+        self.flag = ""
+
+    def __iter__(self):
+        while self.i < len(self.args):
+            self.flag = self.args[self.i]
+            yield self.flag
+            self.i += 1
+
+    def value(self) -> str:
+        if self.i + 1 >= len(self.args):
+            raise InvalidArgument(f"{self.flag} needs a value")
+        self.i += 1
+        return self.args[self.i]
+
+
+def _engine_flag(flag: str, flags: _Flags, o) -> bool:
+    """Options both commands share: the model, the precision, sampling, the cache and the serving shape."""
+    if flag in ("-m", "--model"):
+        o.model = flags.value()
+    elif flag == "--device":
+        o.device = flags.value()
+        if o.device not in ("hip", "gpu", "cuda"):
+            raise InvalidArgument(f"--device must be hip, got '{o.device}' (this engine has no CPU path)")
+    elif flag == "--dtype":
+        o.dtype = flags.value()
+        if o.dtype not in ("bfloat16", "float32", "bf16", "fp32"):
+            raise InvalidArgument(f"--dtype must be bfloat16 or float32, got '{o.dtype}'")
+    elif flag == "--temp":
+        o.sampling.temperature = parse_float(flag, flags.value())
+    elif flag == "--top-k":
+        o.sampling.top_k = parse_int(flag, flags.value())
+    elif flag == "--top-p":
+        o.sampling.top_p = parse_float(flag, flags.value())
+    elif flag == "--seed":
+        o.sampling.seed = parse_int(flag, flags.value())
+    elif flag == "--kv-mem":
+        try:
+            o.kv_bytes = parse_size(flags.value())
+        except InvalidArgument as e:
+            raise InvalidArgument(f"{flag}: {e}") from None
+    elif flag == "--kv-blocks":
+        o.kv_blocks = parse_int(flag, flags.value())
+    elif flag == "--block-size":
+        o.block_size = parse_int(flag, flags.value())
+    elif flag == "--max-seqs":
+        o.max_seqs = parse_int(flag, flags.value())
+    elif flag == "--max-tokens-per-step":
+        o.max_tokens_per_step = parse_int(flag, flags.value())
+    elif flag == "--prefill-chunk":
+        o.prefill_chunk = parse_int(flag, flags.value())
+    elif flag == "--policy":
+        from ..engine.scheduler import parse_policy
+        o.policy = parse_policy(flags.value())
+    elif flag == "--aging":
+        o.aging = parse_int(flag, flags.value())
+        if o.aging < 0:
+            raise InvalidArgument(f"--aging must be non-negative, got {o.aging}")
+    elif flag == "--threads":
+        parse_int(flag, flags.value())         # CPU threads of the reference's CPU backend: nothing to set here
+    else:
+        return False
+    return True
+
+
 def parse_generate_args(args: Sequence[str]) -> GenerateOptions:
     o = GenerateOptions()
-    i = 0
-
-    def value() -> str:
-        nonlocal i
-        if i + 1 >= len(args):
-            raise InvalidArgument(f"{flag} needs a value")
-        i += 1
-        return args[i]
-
-    while i < len(args):
-        flag = args[i]
-        if flag in ("-m", "--model"):
-            o.model = value()
-        elif flag in ("-p", "--prompt"):
-            o.prompt = parse_ids(flag, value())
+    flags = _Flags(args)
+    for flag in flags:
+        if _engine_flag(flag, flags, o):
+            continue
+        if flag in ("-p", "--prompt"):
+            o.prompt = parse_ids(flag, flags.value())
         elif flag == "--prompt-file":
-            path = value()
+            path = flags.value()
             try:
                 with open(path) as f:
                     o.prompt = parse_ids(flag, f.read())
             except OSError as e:
                 raise InvalidArgument(f"cannot read {path}: {e.strerror or e}") from None
-        elif flag == "--device":
-            o.device = value()
-            if o.device not in ("hip", "gpu", "cuda"):
-                raise InvalidArgument(f"--device must be hip, got '{o.device}' (this engine has no CPU path)")
-        elif flag == "--dtype":
-            o.dtype = value()
-            if o.dtype not in ("bfloat16", "float32", "bf16", "fp32"):
-                raise InvalidArgument(f"--dtype must be bfloat16 or float32, got '{o.dtype}'")
-        elif flag == "--temp":
-            o.sampling.temperature = parse_float(flag, value())
-        elif flag == "--top-k":
-            o.sampling.top_k = parse_int(flag, value())
-        elif flag == "--top-p":
-            o.sampling.top_p = parse_float(flag, value())
-        elif flag == "--seed":
-            o.sampling.seed = parse_int(flag, value())
         elif flag == "--max-tokens":
-            o.sampling.max_tokens = parse_int(flag, value())
+            o.sampling.max_tokens = parse_int(flag, flags.value())
         elif flag == "--stop-ids":
-            o.stop_ids = parse_ids(flag, value())
-        elif flag == "--kv-mem":
-            try:
-                o.kv_bytes = parse_size(value())
-            except InvalidArgument as e:
-                raise InvalidArgument(f"{flag}: {e}") from None
-        elif flag == "--kv-blocks":
-            o.kv_blocks = parse_int(flag, value())
-        elif flag == "--block-size":
-            o.block_size = parse_int(flag, value())
-        elif flag == "--max-seqs":
-            o.max_seqs = parse_int(flag, value())
-        elif flag == "--max-tokens-per-step":
-            o.max_tokens_per_step = parse_int(flag, value())
-        elif flag == "--prefill-chunk":
-            o.prefill_chunk = parse_int(flag, value())
-        elif flag == "--policy":
-            from ..engine.scheduler import parse_policy
-            o.policy = parse_policy(value())
-        elif flag == "--aging":
-            o.aging = parse_int(flag, value())
-            if o.aging < 0:
-                raise InvalidArgument(f"--aging must be non-negative, got {o.aging}")
-        elif flag == "--threads":
-            parse_int(flag, value())           # CPU threads of the reference's CPU backend: nothing to set here
+            o.stop_ids = parse_ids(flag, flags.value())
         elif flag in ("--chat", "--no-think"):
             raise InvalidArgument(f"{flag} needs a tokenizer, which this engine does not have: give token ids")
         else:
             raise InvalidArgument(f"unknown option '{flag}'")
-        i += 1
     if not o.model:
         raise InvalidArgument("--model is required")
     if not o.prompt:
         raise InvalidArgument("--prompt is required")
+    o.sampling.validate()
+    return o
+
+
+@dataclasses.dataclass
+class BenchOptions:
+    model: str = ""
+    prompts: str = ""                      # JSONL workload of token ids; empty with --synthetic
+    synthetic: int = 0                     # number of synthetic requests; 0 with --prompts
+    prompt_len: Tuple[int, int] = (512, 1024)
+    output_len: Tuple[int, int] = (128, 128)
+    max_tokens: int = 128                  # for workload lines without max_tokens
+    rate: float = math.inf
+    device: str = "hip"
+    dtype: str = "bfloat16"
+    sampling: SamplingParams = dataclasses.field(default_factory=lambda: SamplingParams(temperature=0.0))
+    kv_bytes: int = 4 << 30
+    kv_blocks: Optional[int] = None
+    block_size: int = 16
+    max_seqs: int = 64
+    max_tokens_per_step: int = 512
+    prefill_chunk: int = 0
+    policy: str = "srpt-aging"
+    aging: int = 16
+    json: bool = False
+
+
+def parse_bench_args(args: Sequence[str]) -> BenchOptions:
+    from ..bench.workload import parse_range
+    from ..engine.serving import ServingConfig
+
+    o = BenchOptions()
+    flags = _Flags(args)
+    for flag in flags:
+        if _engine_flag(flag, flags, o):
+            continue
+        if flag == "--prompts":
+            o.prompts = flags.value()
+        elif flag == "--synthetic":
+            o.synthetic = parse_int(flag, flags.value())
+            if o.synthetic < 1:
+                raise InvalidArgument(f"--synthetic needs at least 1 request, got {o.synthetic}")
+        elif flag == "--prompt-len":
+            o.prompt_len = parse_range(flag, flags.value())
+        elif flag == "--output-len":
+            o.output_len = parse_range(flag, flags.value())
+        elif flag == "--max-tokens":
+            o.max_tokens = parse_int(flag, flags.value())
+            if o.max_tokens < 1:
+                raise InvalidArgument(f"--max-tokens must be positive, got {o.max_tokens}")
+        elif flag == "--rate":
+            text = flags.value()
+            o.rate = math.inf if text == "inf" else parse_float(flag, text)
+            if not o.rate > 0:
+                raise InvalidArgument(f"--rate must be positive or inf, got '{text}'")
+        elif flag == "--json":
+            o.json = True
+        else:
+            raise InvalidArgument(f"unknown option '{flag}'")
+    if not o.model:
+        raise InvalidArgument("--model is required")
+    if bool(o.prompts) == bool(o.synthetic):
+        raise InvalidArgument("give exactly one of --prompts or --synthetic")
+    ServingConfig(o.max_tokens_per_step, o.max_seqs, o.prefill_chunk).validate()
     o.sampling.validate()
     return o

@@ -1,6 +1,7 @@
 """``tie``: the command line. ``tie generate`` prints the generated token ids, one line, and a
 summary on standard error with the reference's fields (``src/cli/main.cpp:100-109``): load time,
-prompt tokens, time to first token, prefill and decode rates, pages used.
+prompt tokens, time to first token, prefill and decode rates, pages used. ``tie bench`` runs a
+workload of many requests through the engine and prints the report of ``src/bench/report.cpp:61-88``.
 Exit codes as in the reference: 1 for an error of the engine's own kinds, 2 for anything else."""
 
 from __future__ import annotations
@@ -11,7 +12,7 @@ import time
 from typing import Sequence
 
 from ..errors import InvalidArgument, TieError
-from .args import USAGE, parse_generate_args, parse_int
+from .args import USAGE, parse_bench_args, parse_generate_args, parse_int
 
 
 def run_generate(argv: Sequence[str]) -> int:
@@ -65,6 +66,37 @@ def run_generate(argv: Sequence[str]) -> int:
     return 0
 
 
+def run_bench(argv: Sequence[str]) -> int:
+    opt = parse_bench_args(argv)
+    import torch
+
+    from ..api import create_engine
+    from ..bench import (assign_arrivals, format_report, read_requests_jsonl, report_json, run_workload, summarize,
+                         synthetic_requests)
+    from ..errors import KernelUnavailable
+
+    if not torch.cuda.is_available():
+        raise KernelUnavailable("no GPU is visible: this engine runs on HIP only")
+    engine = create_engine(opt.model, dtype=opt.dtype, kv_mem=opt.kv_bytes, kv_blocks=opt.kv_blocks,
+                           block_size=opt.block_size, max_seqs=opt.max_seqs,
+                           max_tokens_per_step=opt.max_tokens_per_step, prefill_chunk=opt.prefill_chunk,
+                           policy=opt.policy, aging=opt.aging)
+    vocab = engine.model.spec.vocab_size
+    if opt.synthetic:
+        requests = synthetic_requests(opt.synthetic, opt.prompt_len, opt.output_len, vocab, opt.sampling.seed)
+    else:
+        requests = read_requests_jsonl(opt.prompts, opt.max_tokens, vocab)
+    assign_arrivals(requests, opt.rate, opt.sampling.seed)
+    run = run_workload(engine, requests, opt.sampling,
+                       progress=lambda line: print(f"[tie] {line}", file=sys.stderr, flush=True))
+    report = summarize(run)
+    if opt.json:
+        print(json.dumps(report_json(report)))
+    else:
+        sys.stdout.write(format_report(report))
+    return 0
+
+
 def run_random_weights(argv: Sequence[str]) -> int:
     from ..config.base import read_config_json
     from ..weights.random_init import write_random_model
@@ -103,6 +135,8 @@ def main(argv: Sequence[str] = None) -> int:
     try:
         if argv[0] == "generate":
             return run_generate(argv[1:])
+        if argv[0] == "bench":
+            return run_bench(argv[1:])
         if argv[0] == "random-weights":
             return run_random_weights(argv[1:])
         raise InvalidArgument(f"unknown command '{argv[0]}'")
