@@ -327,6 +327,40 @@ def test_skinny_gemm_bf16(M, N, K):
         assert torch.equal(alone[:, 0], planes[:, M - 1])
 
 
+@pytest.mark.parametrize("M", [1, 8, 64])
+@pytest.mark.parametrize("N,K,gated", [(10240, 5120, False), (5120, 8192, False), (5120, 25600, False), (1600, 5120, True),
+                                       (2048, 6144, False), (4096, 2048, False)])
+def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
+    """The projections of the 32B shape (rows of 5120, K up to 25600) and of the 1.7B shape, packed, cut along K
+    as the plan says (2, 4 or 8 planes), with every pair of tile count and batch of loads the launcher may pick."""
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=41, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=42, scale=0.05, dtype=torch.bfloat16).cuda()
+    packed = kernels.pack_weight(w)
+    if gated:
+        g, u = w.cpu().view(N // 16, 2, 8, K)[:, 0].reshape(N // 2, K), w.cpu().view(N // 16, 2, 8, K)[:, 1].reshape(N // 2, K)
+        gate, up = plain.linear(x.cpu(), g), plain.linear(x.cpu(), u)
+        want = gate / (1 + torch.exp(-gate)) * up
+        out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device="cuda")
+        kernels.skinny_gemm_bf16(x, packed, out, gated=True)
+        close(out, want, 1e-2, f"gated skinny gemm {M}x{N}x{K}")
+        return
+    want = plain.linear(x.cpu(), w.cpu())
+    splits = kernels.skinny_splits(N, K)
+    assert splits in (2, 4, 8)
+    planes = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device="cuda")
+    kernels.skinny_gemm_bf16(x, packed, planes, splits=splits)
+    close(planes.cpu().to(F64).sum(0), want, 1e-5, f"skinny gemm {M}x{N}x{K} in {splits} planes")
+    lib = kernels._lib("skinny_gemm_bf16")
+    for rt, u in ((1, 8), (1, 2), (2, 4), (3, 2), (4, 2), (2, 8)):
+        again = torch.full_like(planes, float("nan"))
+        status = lib.tie_skinny_gemm_bf16_with(x.data_ptr(), packed.data_ptr(), again.data_ptr(), 0, 0, 0, M, N, K, splits, 1,
+                                               rt, u, kernels._stream())
+        assert status == 0
+        assert torch.equal(again, planes), f"tiles {rt}, batch {u}: the sums depend on the launch's shape"
+
+
 @pytest.mark.parametrize("R,n", [(1, 24), (5, 200), (8, 4096), (64, 1024), (3, 20000)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_add_partials_alone_and_with_rms_norm(R, n, out_dtype):
@@ -520,6 +554,15 @@ def test_attention_decode_bf16(H, KVH, Dh, bs, nsplit):
     case, S = attention_case(H, KVH, Dh, bs, lens_new=[1] * len(lens), lens_ctx=lens, seed=13, dtype=torch.bfloat16)
     out = run_decode(case, S, H, Dh, nsplit)
     close(out, case["want"], 1e-2, f"decode attention H={H} KVH={KVH} Dh={Dh} bs={bs} splits={nsplit}")
+
+
+@pytest.mark.parametrize("nsplit", [1, 16, 64])
+def test_attention_decode_bf16_groups_of_eight_query_heads(nsplit):
+    """64 query heads over 8 KV heads of 128 (the 32B shape's geometry), contexts around 4096."""
+    H, KVH, Dh = 64, 8, 128
+    case, S = long_decode_case(H, KVH, Dh, 16, [4096, 4001, 33], seed=35, spike_back=30)
+    out = run_decode(case, S, H, Dh, nsplit)
+    close(out, case["want"], 1e-2, f"decode attention, groups of 8, {nsplit} shares")
 
 
 @pytest.mark.parametrize("where", ["first", "page_edge", "tile_edge", "far", "last"])

@@ -283,8 +283,19 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
 
 template <typename TX>
 __device__ __forceinline__ float load_planes(const TX* p, size_t plane_stride, int planes) {
+  // The usual cuts (2, 4, 8) have all their loads in flight together; the sum is formed in plane order in every case.
+  if (planes == 2) return load_as_float(p) + load_as_float(p + plane_stride);
+  if (planes == 4 || planes == 8) {
+    float part[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) part[s] = s < planes ? load_as_float(p + static_cast<size_t>(s) * plane_stride) : 0.f;
+    float v = part[0];
+#pragma unroll
+    for (int s = 1; s < 8; ++s)
+      if (s < planes) v += part[s];
+    return v;
+  }
   float v = load_as_float(p);
-  if (planes == 2) return v + load_as_float(p + plane_stride);   // the usual cut: both loads in flight together
   for (int s = 1; s < planes; ++s) v += load_as_float(p + static_cast<size_t>(s) * plane_stride);
   return v;
 }
@@ -419,8 +430,19 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, qk_f4_t v) {
 
 template <typename TX>
 __device__ __forceinline__ qk_f4_t load4_planes(const TX* p, size_t plane_stride, int planes) {
+  if (planes == 2) return load4(p) + load4(p + plane_stride);
+  if (planes == 4 || planes == 8) {
+    qk_f4_t part[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+      part[s] = s < planes ? load4(p + static_cast<size_t>(s) * plane_stride) : qk_f4_t{0.f, 0.f, 0.f, 0.f};
+    qk_f4_t v = part[0];
+#pragma unroll
+    for (int s = 1; s < 8; ++s)
+      if (s < planes) v += part[s];
+    return v;
+  }
   qk_f4_t v = load4(p);
-  if (planes == 2) return v + load4(p + plane_stride);
   for (int s = 1; s < planes; ++s) v += load4(p + static_cast<size_t>(s) * plane_stride);
   return v;
 }

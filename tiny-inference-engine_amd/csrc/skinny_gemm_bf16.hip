@@ -51,18 +51,19 @@ __device__ __forceinline__ bf16x8_t zero_frag() {
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
-// MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 loaded ahead of the MFMAs.
+// MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 in one batch of loads.
 template <int MT, int RT, int U, typename TO, bool PACKED>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
                                                                          int accumulate, int gated, int per_wave) {
+  const int tile_group = blockIdx.x, split = blockIdx.y, num_splits = gridDim.y;
   __shared__ float red[SK_WAVES][MT][RT][256];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const int r = lane & 15;   // row of the 16-row tile (of w for B, of x for A)
   const int g = lane >> 4;   // which 8-element chunk of the 32-wide k block
-  const int n0 = blockIdx.x * 16 * RT;
+  const int n0 = tile_group * 16 * RT;
 
   // Rows beyond N are clamped for the loads; their columns are dropped at the store. wp[t] points at
   // this lane's 16 bytes of k-block 0; a k-block further on is KB_STRIDE elements further on.
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
 
   // This wave's k range, in blocks of 32: part (split, wave) of gridDim.y * SK_WAVES equal parts.
   const int kblocks = (K + 31) / 32;
-  const int kb_begin = min(kblocks, (static_cast<int>(blockIdx.y) * SK_WAVES + wave) * per_wave);
+  const int kb_begin = min(kblocks, (split * SK_WAVES + wave) * per_wave);
   const int kb_end = min(kblocks, kb_begin + per_wave);
 
   floatx4 acc[MT][RT];
@@ -94,25 +95,47 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     for (int t = 0; t < RT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   int kb = kb_begin;
-  // Main loop: U blocks at a time, all loads issued before the first MFMA.
-  for (; kb + U <= kb_end && (kb + U) * 32 <= K; kb += U) {
-    bf16x8_t b[RT][U];
-    bf16x8_t a[MT][U];
+  // Main loop: batches of U blocks. The loads of the next batch are issued before the matrix instructions
+  // of the current one, so 2 U blocks of every tile are in flight per wave: a workgroup's share of a narrow
+  // weight is a few dozen KB, and it is the bytes in flight, not the instruction rate, that its time hangs on.
+  const int batches = (min(kb_end, K / 32) - kb_begin) / U;
+  if (batches > 0) {
+    bf16x8_t b[RT][U], a[MT][U];
+    auto load_batch = [&](bf16x8_t (&bb)[RT][U], bf16x8_t (&aa)[MT][U], int at) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = (kb + u) * 32 + g * 8;
+      for (int u = 0; u < U; ++u) {
+        const int k = (at + u) * 32 + g * 8;
 #pragma unroll
-      for (int t = 0; t < RT; ++t) b[t][u] = load_weight_frag<PACKED>(wp[t] + static_cast<size_t>(kb + u) * KB_STRIDE);
+        for (int t = 0; t < RT; ++t) bb[t][u] = load_weight_frag<PACKED>(wp[t] + static_cast<size_t>(at + u) * KB_STRIDE);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) a[mt][u] = xvalid[mt] ? load_frag(xp[mt] + k) : zero_frag();
+        for (int mt = 0; mt < MT; ++mt) aa[mt][u] = xvalid[mt] ? load_frag(xp[mt] + k) : zero_frag();
+      }
+    };
+    auto multiply = [&](const bf16x8_t (&bb)[RT][U], const bf16x8_t (&aa)[MT][U]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int t = 0; t < RT; ++t)
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aa[mt][u], bb[t][u], acc[mt][t], 0, 0, 0);
+    };
+    load_batch(b, a, kb);
+    for (int i = 1; i < batches; ++i) {
+      bf16x8_t nb[RT][U], na[MT][U];
+      load_batch(nb, na, kb + U);
+      multiply(b, a);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) b[t][u] = nb[t][u];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) a[mt][u] = na[mt][u];
+      }
+      kb += U;
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < RT; ++t)
-          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt][u], b[t][u], acc[mt][t], 0, 0, 0);
+    multiply(b, a);
+    kb += U;
   }
   // Remainder, one block at a time; the last block may be partly beyond K.
   for (; kb < kb_end; ++kb) {
@@ -138,7 +161,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
       for (int v = 0; v < 4; ++v) red[wave][mt][t][(g * 4 + v) * 16 + r] = acc[mt][t][v];
   __syncthreads();
 
-  const bool partial = gridDim.y > 1;   // then TO is float and out holds one [M, N] plane per split
+  const bool partial = num_splits > 1;   // then TO is float and out holds one [M, N] plane per split
   for (int e = threadIdx.x; e < 256 * RT * MT; e += SK_WAVES * TIE_WAVE) {
     const int ee = e & 255;            // 16 x 16 outputs of a tile
     const int t = (e >> 8) % RT;
@@ -158,7 +181,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
       store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
       continue;
     }
-    TO* o = out + (static_cast<size_t>(partial ? blockIdx.y : 0) * M + m) * N + n;
+    TO* o = out + (static_cast<size_t>(partial ? split : 0) * M + m) * N + n;
     if (accumulate) sum = load_as_float(o) + sum;
     store_from_float(o, sum);
   }
@@ -198,24 +221,35 @@ static int choose_rt(int M, int N, int splits) {
 }
 
 // Ranges of K that a product over w[N, K] is cut into when its caller takes partial sums: weights with
-// few rows would otherwise give too few workgroups. By the shape of w alone.
-extern "C" int tie_skinny_gemm_splits(int N, int K) { return (N < 8192 && K >= 512) ? 2 : 1; }
+// few rows would otherwise give too few workgroups to keep enough bytes in flight. The smallest power of
+// two that makes about four workgroups a compute unit (1024), as long as a wave keeps four k-blocks and
+// at most 8; measured on the projections of the 1.7B, 8B and 32B shapes. By the shape of w alone.
+extern "C" int tie_skinny_gemm_splits(int N, int K) {
+  const int tiles = (N + 15) / 16;
+  int splits = 1;
+  while (splits < 8 && tiles * splits < 1024 && K / (32 * SK_WAVES * splits * 2) >= 4) splits *= 2;
+  return splits;
+}
 
 // gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
 // and receives silu(gate) * up.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 // packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
-extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
-                                    int M, int N, int K, int splits, int packed, hipStream_t stream) {
+extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out, int out_dtype, int accumulate,
+                                         int gated, int M, int N, int K, int splits, int packed, int rt, int u,
+                                         hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1 || splits > 64) return TIE_BAD_ARGUMENT;
   if (packed && (N % 16 != 0 || K % 32 != 0)) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || N % 16 != 0 || splits != 1)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int rt = choose_rt(M, N, splits);
+  if (rt == 0) rt = choose_rt(M, N, splits);
+  if (rt < 1 || rt > 4) return TIE_BAD_ARGUMENT;
   const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
   const int kblocks = (K + 31) / 32;
   const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
+  if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
+  if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
 #define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
   skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                             \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
@@ -225,11 +259,15 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
     if (packed) LAUNCH_P(MT, RT, U, TO, true); \
     else LAUNCH_P(MT, RT, U, TO, false);       \
   }
+#define LAUNCH_U(MT, RT, TO)                               \
+  if (u == 2) LAUNCH(MT, RT, 2, TO)                        \
+  else if (u == 4) LAUNCH(MT, RT, 4, TO)                   \
+  else LAUNCH(MT, RT, 8, TO)
 #define LAUNCH_RT(MT, TO)                                  \
-  if (rt == 1) LAUNCH(MT, 1, 4, TO)                        \
-  else if (rt == 2) LAUNCH(MT, 2, 4, TO)                   \
-  else if (rt == 3) LAUNCH(MT, 3, 2, TO)                   \
-  else LAUNCH(MT, 4, 2, TO)
+  if (rt == 1) { LAUNCH_U(MT, 1, TO) }                     \
+  else if (rt == 2) { LAUNCH_U(MT, 2, TO) }                \
+  else if (rt == 3) { LAUNCH_U(MT, 3, TO) }                \
+  else { LAUNCH_U(MT, 4, TO) }
 #define LAUNCH_MT(TO)                                      \
   if (mt == 1) { LAUNCH_RT(1, TO); }                       \
   else if (mt == 2) { LAUNCH_RT(2, TO); }                  \
@@ -239,7 +277,13 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH_MT
 #undef LAUNCH_RT
+#undef LAUNCH_U
 #undef LAUNCH
 #undef LAUNCH_P
   return tie_launch_status();
+}
+
+extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
+                                    int M, int N, int K, int splits, int packed, hipStream_t stream) {
+  return tie_skinny_gemm_bf16_with(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, 0, stream);
 }

@@ -20,6 +20,7 @@ import dataclasses
 import time
 from typing import Callable, Dict, List, Optional, Sequence as Seq, Tuple
 
+from .. import kernels
 from ..cache.manager import CacheManager
 from ..errors import CapacityError, InvalidArgument
 from ..models.builder import Model
@@ -49,6 +50,9 @@ class Engine:
         self.cache = cache
         self.serving = serving or ServingConfig()
         self.serving.validate()
+        if self.serving.max_tokens_per_step > kernels.MAX_STEP_TOKENS:
+            raise InvalidArgument(f"max_tokens_per_step of {self.serving.max_tokens_per_step} exceeds the "
+                                  f"{kernels.MAX_STEP_TOKENS} rows the kernels take in one step")
         self.scheduler = scheduler or BatchScheduler(cache, SchedulerConfig(serving=self.serving))
         self.stop_tokens = frozenset(int(t) for t in stop_tokens)
         self.runner = ModelRunner(model, cache, max_seq_len, use_graphs=use_graphs)

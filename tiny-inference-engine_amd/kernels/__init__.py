@@ -68,6 +68,8 @@ _SIGNATURES = {
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
+        "tie_skinny_gemm_bf16_with": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                      _c_int, _c_int, _c_int, _c_void],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void],
     },
@@ -633,9 +635,10 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
 
     Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take.
     """
-    target_waves = 2048
-    by_occupancy = -(-target_waves // max(1, num_seqs * num_kv_heads))
-    by_length = max(1, max_context // 128)          # at least four 32-key tiles a split
+    by_occupancy = -(-2048 // max(1, num_seqs * num_kv_heads))     # about 2048 waves ...
+    if by_occupancy > 8:
+        by_occupancy = -(-by_occupancy // 2)        # ... but half as many where that still leaves many shares to merge
+    by_length = max(1, max_context // 64)           # at least two 32-key tiles a share
     return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
 
 
