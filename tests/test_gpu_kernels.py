@@ -327,7 +327,7 @@ def test_skinny_gemm_bf16(M, N, K):
         assert torch.equal(alone[:, 0], planes[:, M - 1])
 
 
-@pytest.mark.parametrize("M", [1, 8, 64])
+@pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
 @pytest.mark.parametrize("N,K,gated", [(10240, 5120, False), (5120, 8192, False), (5120, 25600, False), (1600, 5120, True),
                                        (2048, 6144, False), (4096, 2048, False)])
 def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
@@ -353,7 +353,12 @@ def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
     kernels.skinny_gemm_bf16(x, packed, planes, splits=splits)
     close(planes.cpu().to(F64).sum(0), want, 1e-5, f"skinny gemm {M}x{N}x{K} in {splits} planes")
     lib = kernels._lib("skinny_gemm_bf16")
-    for rt, u in ((1, 8), (1, 2), (2, 4), (3, 2), (4, 2), (2, 8)):
+    # a row alone (one tile of x, read from memory) and the same row among 64 (x through LDS): the same bits
+    alone = torch.empty(splits, 1, N, dtype=torch.float32, device="cuda")
+    kernels.skinny_gemm_bf16(x[M - 1:M].contiguous(), packed, alone, splits=splits)
+    assert torch.equal(alone[:, 0], planes[:, M - 1])
+    # u = -1: x read from memory whatever M and N; u = 1: x through LDS whatever N (for more than 16 rows)
+    for rt, u in ((1, 8), (1, 2), (2, 4), (3, 2), (4, 2), (2, 8), (0, -1), (0, 1), (1, 1), (2, 1)):
         again = torch.full_like(planes, float("nan"))
         status = lib.tie_skinny_gemm_bf16_with(x.data_ptr(), packed.data_ptr(), again.data_ptr(), 0, 0, 0, M, N, K, splits, 1,
                                                rt, u, kernels._stream())

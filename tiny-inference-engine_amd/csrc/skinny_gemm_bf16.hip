@@ -187,6 +187,156 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   }
 }
 
+// ------------------------------------------------------------------ 17 to 64 rows: x through LDS
+// With more than one 16-row tile of x the kernel above spends most of its load instructions on x: every
+// weight block of 1 KB needs MT blocks of x, read as 16 rows' 64-byte pieces. Here the four waves of a
+// workgroup walk the SAME range of K, each over its own RT weight tiles, and share x: a batch of U k-blocks
+// of all rows is brought in by the whole workgroup with full-line loads, laid into LDS in the order the
+// matrix core takes its A operand (block (u, mt): lane l's 16 bytes at byte 16 l), and read from there by
+// all four waves. Weights still go from memory straight into registers, non-temporally, one batch ahead.
+//
+// The sums are the very ones of the kernel above: a plane's range of K is walked in the same four parts
+// of per_wave k-blocks, each summed by the matrix core in k order, and the parts are added in their order
+// (there: by the reduction through LDS; here: by folding the accumulator into a running total at each
+// part's end). A row's result therefore does not depend on which of the two kernels its batch size picks.
+template <int MT, int RT, int U, typename TO>
+__global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16_t* __restrict__ x,
+                                                                         const bf16_t* __restrict__ w,
+                                                                         TO* __restrict__ out, int M, int N, int K,
+                                                                         int accumulate, int gated, int per_wave) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][U][MT][512];
+  const int lane = threadIdx.x & (TIE_WAVE - 1);
+  const int wave = threadIdx.x / TIE_WAVE;
+  const int tiles = N / 16;
+  const int tile0 = (static_cast<int>(blockIdx.x) * SK_WAVES + wave) * RT;
+  const int split = blockIdx.y;
+  const int kblocks = K / 32;
+  const int kb_lo = min(kblocks, split * SK_WAVES * per_wave);
+  const int kb_hi = min(kblocks, kb_lo + SK_WAVES * per_wave);
+
+  const bf16_t* wp[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) wp[t] = w + static_cast<size_t>(min(tile0 + t, tiles - 1)) * kblocks * 512 + lane * 8;
+
+  // Staging: a batch is MT * 16 rows of U * 32 elements = MT * 64 * U pieces of 16 bytes, CH of them a thread;
+  // consecutive threads take consecutive pieces of a row, so a row's U * 64 bytes are read as whole lines.
+  constexpr int CH = MT * U / 4;
+  static_assert(MT * U % 4 == 0, "a batch must give every thread whole pieces");
+  sk_u32x4_t stage[CH];
+  auto fetch_rows = [&](int kb0) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int piece = c * (SK_WAVES * TIE_WAVE) + threadIdx.x;
+      const int row = piece / (4 * U), col = piece % (4 * U);          // col: 8-element piece of the batch's k range
+      const int kb = kb0 + col / 4;
+      stage[c] = (row < M && kb < kb_hi)
+                     ? *reinterpret_cast<const sk_u32x4_t*>(x + static_cast<size_t>(row) * K + kb * 32 + (col % 4) * 8)
+                     : sk_u32x4_t{0, 0, 0, 0};
+    }
+  };
+  auto store_rows = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int piece = c * (SK_WAVES * TIE_WAVE) + threadIdx.x;
+      const int row = piece / (4 * U), col = piece % (4 * U);
+      // element (row, k): tile row / 16, lane (k % 32 / 8) * 16 + row % 16 of block (u = col / 4, mt)
+      *reinterpret_cast<sk_u32x4_t*>(&xs[buf][col / 4][row / 16][((col % 4) * 16 + (row % 16)) * 8]) = stage[c];
+    }
+  };
+  bf16x8_t b[RT][U], nb[RT][U];
+  auto fetch_weights = [&](bf16x8_t (&bb)[RT][U], int kb0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+        bb[t][u] = (kb0 + u < kb_hi) ? load_weight_frag<true>(wp[t] + static_cast<size_t>(kb0 + u) * 512) : zero_frag();
+  };
+
+  floatx4 acc[MT][RT], total[MT][RT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[mt][t] = total[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bool first_part = true;
+  auto fold = [&]() {          // a part of K has ended: total = total + part, the first part as it is
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        if (first_part) total[mt][t] = acc[mt][t];
+        else
+#pragma unroll
+          for (int v = 0; v < 4; ++v) total[mt][t][v] += acc[mt][t][v];
+        acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+    first_part = false;
+  };
+
+  if (kb_lo < kb_hi) {
+    fetch_rows(kb_lo);
+    fetch_weights(b, kb_lo);
+    store_rows(0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += U) {
+      const bool more = kb0 + U < kb_hi;
+      if (more) {
+        fetch_rows(kb0 + U);
+        fetch_weights(nb, kb0 + U);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kb = kb0 + u;
+        if (kb < kb_hi) {
+          if (kb > kb_lo && (kb - kb_lo) % per_wave == 0) fold();
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const sk_u32x4_t av = *reinterpret_cast<const sk_u32x4_t*>(&xs[buf][u][mt][lane * 8]);
+            const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&av);
+#pragma unroll
+            for (int t = 0; t < RT; ++t) acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t][u], acc[mt][t], 0, 0, 0);
+          }
+        }
+      }
+      if (more) {
+        store_rows(buf ^ 1);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int t = 0; t < RT; ++t) b[t][u] = nb[t][u];
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
+  }
+  fold();
+
+  // D layout: lane holds rows (lane / 16) * 4 + v of a 16-row tile of x, column lane % 16 of the weight tile.
+  const int c = lane & 15, q4 = (lane >> 4) * 4;
+  const bool partial = gridDim.y > 1;
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    if (tile0 + t >= tiles) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = mt * 16 + q4 + v;
+        float sum = total[mt][t][v];
+        if (gated) {       // columns 0..7 are gates, 8..15 the ups of the same outputs
+          const float up = __shfl(sum, (lane & 48) | ((c + 8) & 15), TIE_WAVE);
+          if (m < M && c < 8)
+            store_from_float(out + static_cast<size_t>(m) * (N / 2) + (tile0 + t) * 8 + c, sum / (1.0f + __expf(-sum)) * up);
+          continue;
+        }
+        if (m >= M) continue;
+        TO* o = out + (static_cast<size_t>(partial ? split : 0) * M + m) * N + (tile0 + t) * 16 + c;
+        if (accumulate) sum = load_as_float(o) + sum;
+        store_from_float(o, sum);
+      }
+  }
+}
+
 static int compute_units() {
   static int cached = 0;
   if (cached == 0) {
@@ -243,6 +393,11 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   if (gated && (accumulate || N % 16 != 0 || splits != 1)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int forced_rt = rt;
+  const bool rows_kernel = u >= 0;          // u < 0: the kernel that reads x from memory, whatever M (tests compare the two)
+  const int forced_u = u;
+  if (u < 0) u = u == -1 ? 0 : -u;
+  if (u == 1) u = 0;
   if (rt == 0) rt = choose_rt(M, N, splits);
   if (rt < 1 || rt > 4) return TIE_BAD_ARGUMENT;
   const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
@@ -250,6 +405,30 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
   if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
   if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
+  // x through LDS pays where the weight has very many rows (the feed-forward of the largest shapes, the
+  // head): measured 20 to 25 % faster from 51200 rows on, slower or equal up to 24576, where too few waves
+  // are left to keep enough bytes in flight. u = 1 asks for it whatever N (tests).
+  const int tiles = (N + 15) / 16;
+  if (packed && mt > 1 && rows_kernel && (tiles >= 2048 || forced_u == 1)) {
+    const int rrt = (forced_rt == 0) ? (M <= 32 ? 2 : 1) : (forced_rt > 2 ? 2 : forced_rt);
+    const dim3 rgrid((tiles + SK_WAVES * rrt - 1) / (SK_WAVES * rrt), splits);
+#define LAUNCH_ROWS(MT, RT, U, TO)                                                                              \
+  skinny_rows_kernel<MT, RT, U, TO><<<rgrid, SK_WAVES * TIE_WAVE, 0, stream>>>(                                   \
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
+      gated, per_wave)
+#define LAUNCH_ROWS_TO(MT, RT, U)                                 \
+  if (out_dtype == TIE_F32) LAUNCH_ROWS(MT, RT, U, float);       \
+  else if (out_dtype == TIE_BF16) LAUNCH_ROWS(MT, RT, U, bf16_t); \
+  else return TIE_BAD_ARGUMENT
+    if (mt == 2) {
+      if (rrt == 1) { LAUNCH_ROWS_TO(2, 1, 8); } else { LAUNCH_ROWS_TO(2, 2, 4); }
+    } else {
+      if (rrt == 1) { LAUNCH_ROWS_TO(4, 1, 8); } else { LAUNCH_ROWS_TO(4, 2, 4); }
+    }
+#undef LAUNCH_ROWS_TO
+#undef LAUNCH_ROWS
+    return tie_launch_status();
+  }
 #define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
   skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                             \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
