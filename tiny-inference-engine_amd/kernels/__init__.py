@@ -127,7 +127,16 @@ def _lib(key: str, head_dim: int = 0):
     return lib
 
 
+# The current stream's handle, asked for at every launch. torch's public way (a Stream object built anew each time)
+# costs several microseconds a call, which at a few hundred launches a step is milliseconds of a prefill step
+# that the GPU then waits for; the raw call behind it costs a fraction of one.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None and _current_device is not None:
+        return _raw_stream(_current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -636,7 +645,7 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
     Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take.
     """
     by_occupancy = -(-2048 // max(1, num_seqs * num_kv_heads))     # about 2048 waves ...
-    if by_occupancy > 8:
+    if by_occupancy > 16:
         by_occupancy = -(-by_occupancy // 2)        # ... but half as many where that still leaves many shares to merge
     by_length = max(1, max_context // 64)           # at least two 32-key tiles a share
     return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
