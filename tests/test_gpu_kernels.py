@@ -417,7 +417,7 @@ def test_gemm_bf16(M, N, K, tile):
 
 @pytest.mark.parametrize("M,N,K", [(65, 72, 96), (100, 384, 224), (300, 200, 4096), (2048, 256, 512), (257, 132, 1024),
                                    (513, 516, 352), (1, 64, 128)])
-@pytest.mark.parametrize("tile", [4, 5])
+@pytest.mark.parametrize("tile", [4, 5, 6, 7, 8, 9])
 def test_gemm_bf16_loaded_straight_into_lds(M, N, K, tile):
     """The tiles whose operand slices bypass registers: ragged M and N, short and long K, every epilogue."""
     from tie_amd import kernels
@@ -479,10 +479,10 @@ def test_packed_weight_feeds_both_products_the_same_numbers(N, K):
             kernels.skinny_gemm_bf16(x, w, a, gated=True)
             kernels.skinny_gemm_bf16(x, packed, b_, gated=True)
             assert torch.equal(a, b_)
-    for M in (65, 300, 513):
+    for M in (40, 64, 65, 128, 300, 513):
         x = rnd(M, K, seed=60 + M, dtype=torch.bfloat16).cuda()
         want = plain.linear(x.cpu(), w.cpu())
-        for tile in (4, 5):
+        for tile in (4, 5, 6, 7, 8, 9):
             a = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
             b_ = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
             kernels.gemm_bf16(x, w, a, tile=tile)
@@ -499,7 +499,7 @@ def test_packed_weight_feeds_both_products_the_same_numbers(N, K):
             close(planes.cpu().to(F64).sum(0), want, 1e-5, f"packed weight in {s} planes")
     with pytest.raises(kernels.InvalidArgument):
         kernels.gemm_bf16(rnd(65, K, seed=1, dtype=torch.bfloat16).cuda(), packed,
-                          torch.zeros(65, N, device="cuda"), tile=1)          # only tiles 4 and 5 read the layout
+                          torch.zeros(65, N, device="cuda"), tile=1)          # only the tiles loaded straight into LDS read the layout
     with pytest.raises(kernels.InvalidArgument):
         kernels.linear(torch.zeros(2, K, device="cuda"), packed, torch.zeros(2, N, device="cuda"))   # float32 input
     assert not kernels.packable(w[:, :64].contiguous()) and not kernels.packable(w.float())

@@ -315,22 +315,25 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
 typedef __attribute__((ext_vector_type(4))) float floatx4_t;
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-#define GD_BM 256
 #define GD_BK 32
 #define GD_STAGES 4
 // Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
 // selects x, y, z, w; no swizzle, no stride (the compiler's own default for raw buffers on this target).
 #define GD_RSRC_FLAGS 0x27000
 
-template <int BN, int EPI, bool PW>
+// BM: 256, 128 or 64 rows of x a workgroup; the waves are 2 x 2 in every case, a wave covering BM / 2 rows.
+template <int BM, int BN, int EPI, bool PW>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x_all,
                                                             const bf16_t* __restrict__ w_all,
                                                             void* __restrict__ out_all, int M, int N, int K,
                                                             int tiles_m, int tiles_n, int slices_per_split) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int BM = GD_BM, BK = GD_BK;
+  constexpr int BK = GD_BK;
   constexpr int TN = BN / 64;                   // 32-column MFMA tiles of a wave
-  constexpr int PB = BN / 64;                   // wave instructions that stage w's rows (16 rows each, 4 waves)
+  constexpr int TM = BM / 64;                   // 32-row MFMA tiles of a wave
+  constexpr int PA = BM / 64;                   // wave instructions that stage x's rows (16 rows each, 4 waves)
+  constexpr int PB = BN / 64;                   // wave instructions that stage w's rows likewise
+  static_assert(BM == 256 || BM == 128 || BM == 64, "rows of a tile");
   constexpr int BUF = (BM + BN) * BK;           // elements of one stage
   extern __shared__ bf16_t lds[];
 
@@ -365,9 +368,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<bf16_t*>(x_all + static_cast<size_t>(row0) * K + static_cast<size_t>(k_begin) * BK), 0,
       static_cast<int>(min(BM, M - row0) * row_bytes - k_begin * BK * 2), GD_RSRC_FLAGS);
-  unsigned a_off[4], b_off[PB];
+  unsigned a_off[PA], b_off[PB];
 #pragma unroll
-  for (int p = 0; p < 4; ++p) a_off[p] = min(lr + p * 64, M - 1 - row0) * row_bytes + lchunk * 16;
+  for (int p = 0; p < PA; ++p) a_off[p] = min(lr + p * 64, M - 1 - row0) * row_bytes + lchunk * 16;
   // w: rows like x's, or (PW) the packed layout, where the 16 rows x 32 k that one wave instruction
   // stages are one block of 1 KB: block (tile, k-block) at ((tile * kblocks) + k-block) * 1 KB.
   const int tile0 = col0 / 16, last_tile = (N - 1) / 16;
@@ -388,7 +391,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   auto issue_x = [&](int kt) {
     bf16_t* buf = stage(kt);
 #pragma unroll
-    for (int p = 0; p < 4; ++p)
+    for (int p = 0; p < PA; ++p)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_void_t*)(buf + (p * 64 + wave * 16) * BK), 16, a_off[p],
                                                kt * BK * 2, 0, 0);
   };
@@ -400,9 +403,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                b_off[p], PW ? b_tile_off[p] + kt * 1024 : kt * BK * 2, 0, 0);
   };
 
-  floatx16 acc[4][TN];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -413,22 +416,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   // that one LDS cycle serves read 256 consecutive bytes.
   const int sw = (fr >> 1) & 3;
   const int koff0 = ((0 + fk) ^ sw) * 8, koff1 = ((2 + fk) ^ sw) * 8;
-  const int a_row = (wm * 128 + fr) * BK;
+  const int a_row = (wm * (BM / 2) + fr) * BK;
   const int b_row = PW ? BM * BK + (wn * (BN / 32) + (fr >> 4)) * 512 + (fr & 15) * 8
                        : (BM + wn * (BN / 2) + fr) * BK;
 
-  bf16x8_t fa[2][4], fb[2][TN];
+  bf16x8_t fa[2][TM], fb[2][TN];
   auto load_frags = [&](const bf16_t* buf, int ks, int set) {
     const int koff = ks ? koff1 : koff0;
     const int koff_w = PW ? (ks * 2 + fk) * 128 : koff;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fa[set][i] = *reinterpret_cast<const bf16x8_t*>(buf + a_row + i * 32 * BK + koff);
+    for (int i = 0; i < TM; ++i) fa[set][i] = *reinterpret_cast<const bf16x8_t*>(buf + a_row + i * 32 * BK + koff);
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[set][j] = *reinterpret_cast<const bf16x8_t*>(buf + b_row + j * 32 * BK + koff_w);
   };
   auto mfma_step = [&](int set) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
@@ -441,8 +444,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   issue_x(1);
   issue_w(1);
   issue_x(2);
-  if (PB == 4) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(10)\n\ts_barrier" ::: "memory");
+  // Slice 0 has landed when at most slice 1's loads and slice 2's x rows (2 PA + PB) are still in flight;
+  // in the loop, at most one slice's (PA + PB).
+#define GD_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ")\n\ts_barrier" ::: "memory")
+#define GD_WAIT_ALL_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+  constexpr int FIRST_WAIT = 2 * PA + PB, STEADY_WAIT = PA + PB;
+  if constexpr (FIRST_WAIT == 12) GD_WAIT_BARRIER(12);
+  else if constexpr (FIRST_WAIT == 10) GD_WAIT_BARRIER(10);
+  else if constexpr (FIRST_WAIT == 8) GD_WAIT_BARRIER(8);
+  else if constexpr (FIRST_WAIT == 6) GD_WAIT_BARRIER(6);
+  else if constexpr (FIRST_WAIT == 4) GD_WAIT_BARRIER(4);
+  else static_assert(FIRST_WAIT == 12, "a tile shape without its wait count");
+  auto steady_wait = [&]() {
+    if constexpr (STEADY_WAIT == 8) GD_WAIT_ALL_BARRIER(8);
+    else if constexpr (STEADY_WAIT == 6) GD_WAIT_ALL_BARRIER(6);
+    else if constexpr (STEADY_WAIT == 5) GD_WAIT_ALL_BARRIER(5);
+    else if constexpr (STEADY_WAIT == 4) GD_WAIT_ALL_BARRIER(4);
+    else if constexpr (STEADY_WAIT == 3) GD_WAIT_ALL_BARRIER(3);
+    else GD_WAIT_ALL_BARRIER(0);
+  };
   load_frags(stage(0), 0, 0);
 
   // One slice; its first fragments are in set 0 already. STEADY: slices up to kt + 3 exist, so the loads
@@ -452,7 +472,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     load_frags(stage(kt), 1, 1);
     if (STEADY || kt + 2 < k_tiles) issue_w(kt + 2);
     mfma_step(0);
-    if (STEADY) {
+    if (STEADY && BM == 256) {
 #pragma unroll
       for (int q = 0; q < (4 + TN) / 2; ++q) {
         __builtin_amdgcn_sched_group_barrier(0x008, TN / 2, 0);
@@ -467,20 +487,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     __builtin_amdgcn_sched_barrier(0);
     // My share of slice kt + 1 has landed and my reads of this stage are in registers; after the
     // barrier that holds for every wave.
-    if (STEADY) {
-      if (PB == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    } else if (kt + 2 < k_tiles) {
-      if (PB == 4) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (STEADY || kt + 2 < k_tiles) {
+      steady_wait();
     } else {
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      GD_WAIT_ALL_BARRIER(0);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (STEADY || kt + 1 < k_tiles) load_frags(stage(kt + 1), 0, 0);
     if (STEADY || kt + 3 < k_tiles) issue_x(kt + 3);
     mfma_step(1);
-    if (STEADY) {
+    if (STEADY && BM == 256) {
 #pragma unroll
       for (int q = 0; q < (4 + TN) / 2; ++q) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -504,10 +520,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   }
   for (; kt < k_tiles; ++kt) slice(kt, std::false_type{});
 
+#undef GD_WAIT_BARRIER
+#undef GD_WAIT_ALL_BARRIER
   const bool gated_n = EPI == 3;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = row0 + wm * 128 + i * 32 + fr;
+  for (int i = 0; i < TM; ++i) {
+    const int m = row0 + wm * (BM / 2) + i * 32 + fr;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -549,25 +567,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #endif
 }
 
-template <int BN, bool PW>
+template <int BM, int BN, bool PW>
 static int launch_gemm_dma(const void* x, const void* w, void* out, int epi, int M, int N, int K, int splits,
                            hipStream_t stream) {
-  const int tiles_m = (M + GD_BM - 1) / GD_BM, tiles_n = (N + BN - 1) / BN;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int k_slices = K / GD_BK;
   const int per_split = (k_slices + splits - 1) / splits;
   if (k_slices - per_split * (splits - 1) < 3) return TIE_BAD_ARGUMENT;   // the last range would be too short
-  const size_t shared = sizeof(bf16_t) * GD_STAGES * (GD_BM + BN) * GD_BK;
+  const size_t shared = sizeof(bf16_t) * GD_STAGES * (BM + BN) * GD_BK;
   const dim3 grid(tiles_m * tiles_n, splits);
 #define LAUNCH(EPI)                                                                                          \
   {                                                                                                          \
     static bool raised = false;                                                                              \
     if (!raised) {                                                                                           \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_dma_kernel<BN, EPI, PW>),      \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16_dma_kernel<BM, BN, EPI, PW>),  \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared)); \
       if (e != hipSuccess) return static_cast<int>(e);                                                       \
       raised = true;                                                                                         \
     }                                                                                                        \
-    gemm_bf16_dma_kernel<BN, EPI, PW><<<grid, 256, shared, stream>>>(                                        \
+    gemm_bf16_dma_kernel<BM, BN, EPI, PW><<<grid, 256, shared, stream>>>(                                    \
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n, per_split); \
   }
   if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
@@ -616,6 +634,18 @@ static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_sp
       if (tiles * r >= want && K / r >= shortest) return r;
     return 0;
   };
+  if (straight_to_lds && packed && M <= 128) {
+    // Few rows over packed weights: tiles of 64 or 128 rows (measured on the projections of the 1.7B, 8B and
+    // 32B shapes at 48 to 128 rows). Wide weights take 256 columns a tile, narrow ones 128 and more ranges of K.
+    const bool wide = M <= 64 ? N >= 8192 : N >= 5120;
+    const int tile = M <= 64 ? (wide ? 8 : 9) : (wide ? 6 : 7);
+    if (!may_split) return {tile, 1};
+    const long tiles = (N + (wide ? 255 : 127)) / (wide ? 256 : 128);
+    int r = ranges(tiles, 192, 512);
+    if (r == 0)
+      for (r = 8; r > 1 && K / r < 512; r /= 2) {}
+    return {tile, r};
+  }
   if (straight_to_lds && M >= 256) {
     if (t256 >= 160) return {4, 1};
     if (!may_split) return {t128 >= 128 || packed ? 5 : 1, 1};
@@ -639,6 +669,13 @@ static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_sp
 
 static bool straight_to_lds_shape(int N, int K) { return K % GD_BK == 0 && N % 4 == 0 && K <= (1 << 22) && K >= 3 * GD_BK; }
 
+// Whether a product of 33 to 64 rows runs faster here than on the decode product: over packed weights whose
+// shape the tiles that load straight into LDS take, unless it is gated and not very wide (measured).
+extern "C" int tie_gemm_bf16_wins_few_rows(int M, int N, int K, int packed, int gated) {
+  if (M <= 32 || M > 64 || !packed || !straight_to_lds_shape(N, K) || N % 16 != 0 || K < 1024) return 0;
+  return gated ? N >= 32768 : 1;
+}
+
 // Ranges of K that a product of M rows over w[N, K] is best cut into when its caller adds planes of
 // partial sums: few rows over a narrow weight give too few workgroups otherwise.
 extern "C" int tie_gemm_bf16_splits(int M, int N, int K, int packed) {
@@ -652,7 +689,8 @@ extern "C" int tie_gemm_bf16_splits(int M, int N, int K, int packed) {
 // (128x128 tiles; neither accumulate nor gated).
 // tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
 //       3 = 256x128 (eight waves of 64x64), 4 = 256x256 and 5 = 256x128 loaded straight into LDS (four
-//       waves of 128x128 or 128x64; K % 32 == 0, N % 4 == 0, 16-byte aligned operands, else refused).
+//       waves of 128x128 or 128x64; K % 32 == 0, N % 4 == 0, 16-byte aligned operands, else refused),
+//       6 = 128x256, 7 = 128x128, 8 = 64x256, 9 = 64x128 likewise, for fewer rows.
 // packed: w is stored in blocks of 16 rows x 32 k, 1 KB each, in the matrix cores' operand order (as the
 //       decode product reads it); N % 16 == 0, and only tiles 4 and 5 read it.
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
@@ -664,7 +702,7 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
   const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
-  if (packed && (N % 16 != 0 || !straight || (tile != 0 && tile != 4 && tile != 5))) return TIE_BAD_ARGUMENT;
+  if (packed && (N % 16 != 0 || !straight || (tile != 0 && (tile < 4 || tile > 9)))) return TIE_BAD_ARGUMENT;
   if (tile == 0) {
     if (splits > 1) {
       const GemmPlan plan = gemm_plan(M, N, K, straight, true, packed != 0);
@@ -675,13 +713,20 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   } else if (tile < 4 && splits > 1) {
     tile = 1;
   }
-  if (tile == 4 || tile == 5) {
+  if (tile >= 4 && tile <= 9) {
     if (!straight) return TIE_BAD_ARGUMENT;
-    if (tile == 4)
-      return packed ? launch_gemm_dma<256, true>(x, w, out, epi, M, N, K, splits, stream)
-                    : launch_gemm_dma<256, false>(x, w, out, epi, M, N, K, splits, stream);
-    return packed ? launch_gemm_dma<128, true>(x, w, out, epi, M, N, K, splits, stream)
-                  : launch_gemm_dma<128, false>(x, w, out, epi, M, N, K, splits, stream);
+#define DMA(BM, BN)                                                                            \
+  return packed ? launch_gemm_dma<BM, BN, true>(x, w, out, epi, M, N, K, splits, stream)       \
+                : launch_gemm_dma<BM, BN, false>(x, w, out, epi, M, N, K, splits, stream)
+    switch (tile) {
+      case 4: DMA(256, 256);
+      case 5: DMA(256, 128);
+      case 6: DMA(128, 256);
+      case 7: DMA(128, 128);
+      case 8: DMA(64, 256);
+      default: DMA(64, 128);
+    }
+#undef DMA
   }
   if (tile == 2) return launch_gemm<256, 256, 64, 2, 4>(x, w, out, epi, M, N, K, splits, stream);
   if (tile == 3) return launch_gemm<256, 128, 64, 4, 2>(x, w, out, epi, M, N, K, splits, stream);

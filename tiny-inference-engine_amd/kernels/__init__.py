@@ -10,7 +10,7 @@ InvalidArgument before anything is launched.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -75,6 +75,7 @@ _SIGNATURES = {
     },
     "gemm_bf16": {
         "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
+        "tie_gemm_bf16_wins_few_rows": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void],
     },
@@ -434,9 +435,29 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack([gate.reshape(I // 8, 8, K), up.reshape(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
 
 
+_few_rows_memo: Dict[tuple, bool] = {}
+
+
+def decode_product_rows(M: int, w, gated: bool = False) -> bool:
+    """Whether ``M`` rows against ``w`` go to the decode product (``skinny_gemm_bf16``) rather than the tiled one.
+
+    Up to 32 rows always, above 64 never; between, by the weight's shape and layout (the tiled product with
+    64-row tiles is the faster one over packed weights, except for gated products that are not very wide).
+    """
+    if M <= 32 or M > 64:
+        return M <= 32
+    N, K = w.shape
+    key = (M > 32, N, K, isinstance(w, PackedWeight), bool(gated))
+    tiled = _few_rows_memo.get(key)
+    if tiled is None:
+        tiled = _few_rows_memo[key] = bool(_lib("gemm_bf16").tie_gemm_bf16_wins_few_rows(
+            M, N, K, int(isinstance(w, PackedWeight)), int(gated)))
+    return not tiled
+
+
 def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tensor) -> None:
     """out = silu(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only."""
-    if x.shape[0] <= 64:
+    if decode_product_rows(x.shape[0], w_interleaved, gated=True):
         skinny_gemm_bf16(x, w_interleaved, out, gated=True)
     else:
         gemm_bf16(x, w_interleaved, out, gated=True)
@@ -446,7 +467,7 @@ def linear(x: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> N
     """out (+)= x @ w.T, on the fastest kernel that takes these operands (w a matrix or a ``PackedWeight``)."""
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and \
             not (accumulate and out.dtype != torch.float32):
-        if x.shape[0] <= 64:
+        if decode_product_rows(x.shape[0], w):
             skinny_gemm_bf16(x, w, out, accumulate)
         else:
             gemm_bf16(x, w, out, accumulate)

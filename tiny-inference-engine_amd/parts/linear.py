@@ -73,14 +73,15 @@ class Linear:
     def partial_planes(self, ctx, x: torch.Tensor, name: str):
         """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None.
 
-        Up to 64 rows the decode product decides by the weight's shape alone; above, the tiled
-        product is cut along K when its tiles alone would leave most of the GPU idle.
+        The decode product (up to 32 rows, or 64 where the tiled one is not the faster) decides by the weight's
+        shape alone; the tiled product is cut along K when its tiles alone would leave most of the GPU idle.
         """
         M, K = x.shape
         w = self.weight
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8:
             return None
-        if M <= 64:
+        decode_product = kernels.decode_product_rows(M, w)
+        if decode_product:
             if self._splits is None:
                 self._splits = kernels.skinny_splits(w.shape[0], K)
             splits = self._splits
@@ -91,7 +92,7 @@ class Linear:
         if splits <= 1:
             return None
         planes = ctx.scratch(name, (splits, M, w.shape[0]), torch.float32)
-        if M <= 64:
+        if decode_product:
             kernels.skinny_gemm_bf16(x, w, planes, splits=splits)
         else:
             kernels.gemm_bf16(x, w, planes, splits=splits)
