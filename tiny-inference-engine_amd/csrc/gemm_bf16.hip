@@ -646,6 +646,18 @@ static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_sp
       for (r = 8; r > 1 && K / r < 512; r /= 2) {}
     return {tile, r};
   }
+  if (straight_to_lds && packed && M <= 256) {
+    // Up to 256 rows over a weight so narrow, or a K so short, that even 256 x 128 tiles over every allowed range
+    // of K leave most compute units idle (the 1.7B shape's projections): 128 x 128.
+    int most = 8;
+    while (most > 1 && K / most < 512) most /= 2;
+    if (t128 * (may_split ? most : 1) < 192) {
+      const long t7 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+      if (!may_split) return {7, 1};
+      const int r7 = ranges(t7, 192, 512);
+      return {7, r7 ? r7 : most};
+    }
+  }
   if (straight_to_lds && M >= 256) {
     if (t256 >= 160) return {4, 1};
     if (!may_split) return {t128 >= 128 || packed ? 5 : 1, 1};
