@@ -660,7 +660,7 @@ static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_sp
   }
   if (straight_to_lds && M >= 256) {
     if (t256 >= 160) return {4, 1};
-    if (!may_split) return {t128 >= 128 || packed ? 5 : 1, 1};
+    if (!may_split) return {packed ? 6 : (t128 >= 128 ? 5 : 1), 1};   // 128 x 256: twice the workgroups of 256 x 256
     const int r256 = ranges(t256, 160, 1024), r128 = ranges(t128, 192, 1024);
     if (K >= 8192 && r256) return {4, r256};
     if (r128) return {5, r128};
