@@ -108,13 +108,13 @@ def measure_stress(model, cfg, args):
     return report
 
 
-def make_engine(model, batch, context, max_tokens_per_step):
+def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True):
     from tie_amd.api import create_engine
 
     blocks = batch * (-(-context // BLOCK_SIZE) + 1) + 8
     return create_engine(model, kv_blocks=blocks, block_size=BLOCK_SIZE, max_seqs=max(batch, 1),
                          max_tokens_per_step=max(max_tokens_per_step, batch), policy="fcfs", watermark_blocks=0,
-                         max_seq_len=context)
+                         max_seq_len=context, launch_ahead=launch_ahead)
 
 
 def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
@@ -174,7 +174,7 @@ def measure_prefill(model, cfg, tokens, repeats=3):
     import torch
     from tie_amd.sampling.params import SamplingParams
 
-    engine = make_engine(model, 1, tokens + 16, tokens)
+    engine = make_engine(model, 1, tokens + 16, tokens, launch_ahead=False)   # the step's token is read inside the step
     rng = random.Random(7)
     best = None
     for i in range(repeats + 1):               # the first run warms up

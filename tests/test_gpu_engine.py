@@ -337,3 +337,52 @@ def test_device_sampling_matches_the_host_sampler():
     from tie_amd.errors import InvalidArgument
     with pytest.raises(InvalidArgument, match="NaN"):
         sampler.sample_rows(bad, params, dev_rngs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kv_blocks", [256, 14])
+def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_folders_bf16, dtype, kv_blocks):
+    """Greedy requests with the next step queued before the last one's tokens are read, against the same engine
+    reading every step at once: equal tokens, through stop tokens (a sequence then ran one token too many,
+    which must leave no trace), ends by length, a cancellation and, with 14 pages, evictions."""
+    import tie_amd
+
+    folder, cfg = (model_folders_bf16 if dtype == "bfloat16" else model_folders)["A"]
+    vocab = cfg["vocab_size"]
+    reqs = [([(t * 7 + i * 13 + 1) % vocab for t in range(n)], m)
+            for i, (n, m) in enumerate(zip([3, 17, 9, 21, 1, 12], [30, 14, 40, 8, 26, 33]))]
+
+    def run(ahead, stop_tokens=()):
+        engine = make_engine(folder, 4, dtype=dtype, kv_blocks=kv_blocks, max_seqs=8, max_tokens_per_step=32,
+                             launch_ahead=ahead, stop_tokens=stop_tokens)
+        seen = []
+        engine.on_token = lambda seq_id, token: seen.append((seq_id, token))
+        ids = [engine.add_request(p, tie_amd.SamplingParams(max_tokens=m)) for p, m in reqs]
+        steps = 0
+        while engine.has_work():
+            engine.step()
+            steps += 1
+            if steps == 12:
+                engine.cancel(ids[2])
+            assert steps < 2000
+        assert engine.cache.num_free() == kv_blocks and engine._unread is None
+        out = [engine.sequence(i).generated for i in ids]
+        reasons = [engine.sequence(i).finish_reason.value for i in ids]
+        for i, tokens in zip(ids, out):
+            assert [t for s, t in seen if s == i] == tokens and -1 not in tokens
+        return out, reasons, engine
+
+    plain_out, plain_reasons, _ = run(False)
+    ahead_out, ahead_reasons, engine = run(True)
+    assert engine.steps_launched_ahead > 10
+    for i in (0, 1, 3, 4, 5):                                  # (the cancelled one stops wherever it was)
+        assert ahead_out[i] == plain_out[i] and ahead_reasons[i] == plain_reasons[i] == "length"
+    # a stop token in the middle of some outputs
+    stop = plain_out[0][7]
+    s_plain, r_plain, _ = run(False, stop_tokens=(stop,))
+    s_ahead, r_ahead, engine = run(True, stop_tokens=(stop,))
+    assert "stop" in r_plain and engine.steps_launched_ahead > 0
+    for i in (0, 1, 3, 4, 5):
+        assert s_ahead[i] == s_plain[i] and r_ahead[i] == r_plain[i]
+        if r_plain[i] == "stop":
+            assert s_plain[i][-1] == stop and stop not in s_plain[i][:-1]

@@ -26,11 +26,13 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
                   block_size: int = 16, max_seqs: int = 64, max_tokens_per_step: int = 512, prefill_chunk: int = 0,
                   policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1,
                   stop_tokens: Sequence[int] = (), max_seq_len: Optional[int] = None,
-                  device: str = "cuda:0", use_graphs: Optional[bool] = None) -> Engine:
+                  device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead: bool = True) -> Engine:
     """``model`` is a folder (config.json + safetensors) or a Model that is already loaded.
 
     ``use_graphs`` False runs every step eagerly; None (the default) records decode-only steps into HIP
-    graphs in bfloat16 mode when every part of the model allows it."""
+    graphs in bfloat16 mode when every part of the model allows it. ``launch_ahead``: in the steady state of
+    decoding the next step is queued before the last one's tokens are read (``Engine``'s module text says how);
+    tokens then appear one ``step()`` later."""
     if not isinstance(model, Model):
         model = load_model(model, normalize_mode(dtype), device)
     cache_dtype = "float32" if model.mode == FLOAT32 else "bfloat16"
@@ -43,7 +45,7 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
     scheduler = BatchScheduler(cache, SchedulerConfig(serving=serving, policy=policy, aging=aging,
                                                       watermark_blocks=watermark_blocks))
     return Engine(model, cache, scheduler, serving, stop_tokens=stop_tokens, max_seq_len=max_seq_len,
-                  use_graphs=use_graphs)
+                  use_graphs=use_graphs, launch_ahead=launch_ahead)
 
 
 def generate(model, prompt: Sequence[int], params: Optional[SamplingParams] = None, **engine_options) -> List[int]:

@@ -12,6 +12,17 @@ reference engine's (``src/engine/engine.cpp:26-235``):
   again; a failure after that (sampling, a token callback) ends the affected sequences with
   ``FinishReason.ERROR`` and frees what they hold, since their cache already counts the step;
 * a sequence ends on a stop token (which stays in its output) or after ``max_tokens`` tokens.
+
+Reading ahead (``launch_ahead``, not in the reference). A decode step's host work - planning, the batch
+arrays, the launch - lies between two steps while the GPU idles, because the next step's tokens are the
+ones just sampled. With ``launch_ahead`` a step of greedy rows only queues its argmax and leaves the
+tokens unread; if the next call to ``step()`` finds the steady state (nobody waiting, the very same
+sequences decoding, none at its last token), it queues the next step first - whose tokens the GPU
+takes from the argmax's own output - and reads the earlier step's tokens while that one runs. A
+sequence that turns out to have met a stop token has then run one token too many, which is dropped.
+In every other situation the unread tokens are read before anything is planned, and the engine behaves
+as without the option. Tokens (and callbacks) appear one ``step()`` later; ``has_work()`` stays true
+until they have.
 """
 
 from __future__ import annotations
@@ -29,7 +40,7 @@ from ..sampling.sampler import DeviceSampler
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import BatchScheduler, SchedulerConfig, StepPlan
-from .sequence import FinishReason, SeqState, Sequence
+from .sequence import UNREAD, FinishReason, SeqState, Sequence
 from .serving import ServingConfig
 
 
@@ -43,9 +54,21 @@ class EngineStats:
     preemptions: int = 0
 
 
+class _Unread:
+    """A launched step whose sampled tokens the host has not read: who sampled, where each token goes."""
+
+    __slots__ = ("sampling", "places", "ticket")
+
+    def __init__(self, sampling, places, ticket):
+        self.sampling = sampling      # the sequences that sampled, in the order of the step's rows
+        self.places = places          # per sequence, the index in its tokens that holds UNREAD
+        self.ticket = ticket
+
+
 class Engine:
     def __init__(self, model: Model, cache: CacheManager, scheduler=None, serving: Optional[ServingConfig] = None,
-                 stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None, use_graphs: Optional[bool] = None):
+                 stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None, use_graphs: Optional[bool] = None,
+                 launch_ahead: bool = False):
         self.model = model
         self.cache = cache
         self.serving = serving or ServingConfig()
@@ -62,6 +85,9 @@ class Engine:
         self._stats = EngineStats()
         self._ids = 0
         self._inside_step = False
+        self.launch_ahead = bool(launch_ahead)
+        self._unread: Optional[_Unread] = None
+        self.steps_launched_ahead = 0
 
     # -------------------------------------------------------------- requests
     def _token_limits(self) -> List[Tuple[int, str]]:
@@ -100,7 +126,7 @@ class Engine:
         return seq
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._unread is not None
 
     def cancel(self, seq_id: int) -> None:
         seq = self.sequence(seq_id)
@@ -119,6 +145,8 @@ class Engine:
         return dataclasses.replace(self._stats, preemptions=self.scheduler.num_preemptions)
 
     def _end(self, seq: Sequence, reason: FinishReason) -> None:
+        while seq.tokens and seq.tokens[-1] == UNREAD:      # tokens of steps that ran past its end
+            seq.tokens.pop()
         seq.state = SeqState.FINISHED
         seq.finish_reason = reason
         self.cache.release(seq.cache)
@@ -128,14 +156,31 @@ class Engine:
     def step(self) -> None:
         if self._inside_step:
             raise InvalidArgument("step() was called from inside a step (a token callback?)")
-        plan = self.scheduler.schedule()
-        if not plan:
-            return
         self._inside_step = True
         try:
-            self._carry_out(plan)
+            unread = self._unread
+            if unread is not None and not self._steady(unread):
+                self._read(unread)                 # anything but the steady state: know the tokens before planning
+                unread = None
+            plan = self.scheduler.schedule()
+            if plan:
+                self._carry_out(plan, unread)
+            elif unread is not None:
+                self._read(unread)
         finally:
             self._inside_step = False
+
+    def _steady(self, unread: _Unread) -> bool:
+        """Whether the next step can be planned without the unread tokens: the same sequences decode again."""
+        running = self.scheduler.running
+        if self.scheduler.waiting or len(running) != len(unread.sampling):
+            return False
+        for seq, sampled in zip(running, unread.sampling):
+            if seq is not sampled or len(seq.tokens) - seq.num_computed != 1:
+                return False
+            if len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:    # the unread token is its last
+                return False
+        return True
 
     def _entries_of(self, plan: StepPlan):
         """The plan as batch entries, checked on the way: a planner's mistake stops here, before any compute.
@@ -169,24 +214,45 @@ class Engine:
                 decoded_tokens += 1
             else:
                 prompt_tokens += n
+            tokens = seq.tokens[first:last]
+            if tokens[-1] == UNREAD:             # the GPU knows it, the host does not: the step takes it from there
+                if n != 1:
+                    raise InvalidArgument(f"sequence {seq.id} would run {n} tokens, one of them not read yet")
+                tokens = (0,)
             if last == len(seq.tokens):          # all it has is cached after this step: it samples
-                entries.append(StepEntry(seq.cache, first, seq.tokens[first:last], (n - 1,)))
+                entries.append(StepEntry(seq.cache, first, tokens, (n - 1,)))
                 sampling.append(seq)
             else:
-                entries.append(StepEntry(seq.cache, first, seq.tokens[first:last], ()))
+                entries.append(StepEntry(seq.cache, first, tokens, ()))
         return entries, sampling, prompt_tokens, decoded_tokens
 
-    def _carry_out(self, plan: StepPlan) -> None:
+    def _carry_out(self, plan: StepPlan, unread: Optional[_Unread] = None) -> None:
+        """Runs a plan. ``unread``: the step before it, whose tokens are still on the GPU (the steady state)."""
+        self._unread = None                # held in ``unread`` from here on; put back if this step never runs
         try:
+            if unread is not None and not (len(plan.seqs) == len(unread.sampling) and all(
+                    share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, unread.sampling))):
+                # Planning changed the picture (a sequence was evicted to make room): read first after all.
+                self._read(unread)
+                unread = None
+                for share in [s for s in plan.seqs if s.seq.state == SeqState.FINISHED]:
+                    plan.seqs.remove(share)          # it met a stop token; what was reserved for it went back with it
+                    plan.total_tokens -= share.num_tokens
+                if not plan.seqs:
+                    self.scheduler.complete(plan)
+                    return
             entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan)
             began = time.perf_counter()
-            logits = self.runner.step(entries)        # queued on the GPU; the sampling kernels queue right behind
+            # Queued on the GPU; the sampling kernels queue right behind.
+            logits = self.runner.step(entries, None if unread is None else unread.ticket.device_tokens)
         except BaseException:
             # Nothing of the step counts: the pages reserved for it go back and the plan's sequences are free
             # to be planned again.
             for share in plan.seqs:
-                self.cache.truncate(share.seq.cache, share.seq.num_computed)
+                if share.seq.state != SeqState.FINISHED:
+                    self.cache.truncate(share.seq.cache, share.seq.num_computed)
             self.scheduler.abandon(plan)
+            self._unread = unread
             raise
         stats = self._stats
         stats.steps += 1
@@ -200,29 +266,62 @@ class Engine:
             if windows:
                 self.cache.trim(seq.cache, seq.num_computed)     # pages a window has passed go back now
         self.scheduler.complete(plan)
+        if unread is not None:
+            self.steps_launched_ahead += 1
         tokens: List[int] = []
-        if sampling:
+        if sampling and self.launch_ahead and all(s.params.greedy for s in sampling):
+            try:
+                ticket = self.sampler.launch_greedy(logits)
+            except BaseException:
+                self._end_all(sampling, FinishReason.ERROR)
+                raise
+            for seq in sampling:
+                seq.tokens.append(UNREAD)
+                seq.state = SeqState.DECODING
+            self._unread = _Unread(sampling, [len(seq.tokens) - 1 for seq in sampling], ticket)
+            sampling = []
+        elif sampling:
             try:
                 tokens = self.sampler.sample_rows(logits, [s.params for s in sampling], [s.rng for s in sampling])
             except BaseException:
                 self._end_all(sampling, FinishReason.ERROR)
                 raise
         stats.step_seconds += time.perf_counter() - began     # reading the tokens waited for the GPU
+        if unread is not None:
+            self._read(unread, keep=self._unread)                 # the step before, while this one runs (keep: this one's)
         if sampling:
             self._deliver(sampling, tokens)
+
+    def _read(self, unread: _Unread, keep: Optional[_Unread] = None) -> None:
+        """Waits for a launched step's tokens, puts them where UNREAD stands, and delivers them."""
+        self._unread = keep
+        began = time.perf_counter()
+        try:
+            tokens = self.sampler.collect(unread.ticket)
+        except BaseException:
+            self._end_all(unread.sampling, FinishReason.ERROR)
+            raise
+        self._stats.step_seconds += time.perf_counter() - began
+        self._deliver(unread.sampling, tokens, unread.places)
 
     def _end_all(self, seqs: Seq[Sequence], reason: FinishReason) -> None:
         for seq in seqs:
             if seq.state != SeqState.FINISHED:
                 self._end(seq, reason)
 
-    def _deliver(self, sampling: List[Sequence], tokens: List[int]) -> None:
+    def _deliver(self, sampling: List[Sequence], tokens: List[int], places: Optional[List[int]] = None) -> None:
+        """Hands each sequence its token: appended, or (``places``) written where UNREAD stood for it."""
         callback, stop = self.on_token, self.stop_tokens
         for i, seq in enumerate(sampling):
-            if seq.state == SeqState.FINISHED:       # cancelled by a callback earlier in this loop
+            if seq.state == SeqState.FINISHED:       # cancelled meanwhile, or by a callback earlier in this loop
                 continue
             token = tokens[i]
-            seq.tokens.append(token)
+            if places is None:
+                seq.tokens.append(token)
+                count = len(seq.tokens) - seq.prompt_len
+            else:
+                seq.tokens[places[i]] = token
+                count = places[i] + 1 - seq.prompt_len       # a later token may stand behind it, still unread
             seq.state = SeqState.DECODING
             if callback is not None:
                 try:
@@ -235,7 +334,7 @@ class Engine:
                     continue
             if token in stop:
                 self._end(seq, FinishReason.STOP)
-            elif len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:
+            elif count >= seq.params.max_tokens:
                 self._end(seq, FinishReason.LENGTH)
 
     # -------------------------------------------------------------- generate

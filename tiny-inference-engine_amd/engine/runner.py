@@ -65,10 +65,14 @@ class ModelRunner:
         ctx = StepContext(batch, self.model.mode, self.device, self.workspace, self.cache, self.model.cache_plan)
         return self.model.forward(ctx)
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs one batch; returns float32 logits ``[wanted rows, vocab]`` on the device, or None.
 
         The returned tensor is scratch memory of the runner: it is valid until the next step.
+
+        ``device_tokens`` (int32 on the device, one per entry, in the entries' order; only for steps in which
+        every entry brings one token): the tokens to run, which the host does not know yet - an earlier step's
+        sampling kernel left them there. The entries' own token values are then ignored.
         """
         total = 0
         for e in entries:
@@ -80,6 +84,10 @@ class ModelRunner:
             raise CapacityError(f"a step of {total} tokens exceeds the {kernels.MAX_STEP_TOKENS} the kernels take; "
                                 f"cut the prompt into portions")
         batch = self.builder.build(entries)
+        if device_tokens is not None:
+            if not batch.all_decode or device_tokens.numel() != batch.num_tokens or device_tokens.dtype != torch.int32:
+                raise InvalidArgument("tokens on the device need a step of single tokens and one int32 per entry")
+            batch.tokens.copy_(device_tokens)      # queued behind the copy of the step's arrays, before any kernel
         if not (self.use_graphs and batch.all_decode and self.model.layer_hook is None):
             return self._forward(batch)
 

@@ -25,6 +25,9 @@ class FinishReason(enum.Enum):
     CANCELLED = "cancelled"
 
 
+UNREAD = -1      # stands in ``Sequence.tokens`` for a token the GPU has chosen and the host has not read yet
+
+
 class Sequence:
     """One request: its tokens (prompt, then generated), how many are cached, and what it holds."""
 
@@ -52,4 +55,8 @@ class Sequence:
 
     @property
     def generated(self) -> List[int]:
-        return self.tokens[self.prompt_len:]
+        """The generated tokens the host knows (a last one still on its way from the GPU is left out)."""
+        out = self.tokens[self.prompt_len:]
+        if out and out[-1] == UNREAD:
+            out.pop()
+        return out

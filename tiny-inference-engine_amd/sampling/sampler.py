@@ -72,25 +72,42 @@ def sample(logits: np.ndarray, params: SamplingParams, rng: RandomStream) -> int
     return int(pick if ids is None else ids[pick])
 
 
+class GreedyTicket:
+    """Rows whose argmax has been asked of the GPU and not yet read: see ``DeviceSampler.launch_greedy``."""
+
+    __slots__ = ("rows", "device_tokens", "host", "event")
+
+    def __init__(self, rows, device_tokens, host, event):
+        self.rows = rows
+        self.device_tokens = device_tokens     # int32 [rows] on the device: the chosen tokens, in row order
+        self.host = host                       # pinned int32 [2 * rows]: tokens, then the maxima's bits
+        self.event = event
+
+
 class DeviceSampler:
     """Samples the rows of one step's logits, on the GPU where the parameters allow it.
 
-    The results come back through one pinned host buffer that lives as long as the sampler: a step of
-    greedy rows is one kernel, one copy of ``2 R`` words and one wait."""
+    The results come back through pinned host buffers that live as long as the sampler: a step of greedy
+    rows is one kernel, one copy of ``2 R`` words and one wait. ``launch_greedy`` / ``collect`` split that
+    into asking and reading, so that a caller may queue the next step (whose tokens it takes from
+    ``ticket.device_tokens``) before it reads this one's; two sets of buffers alternate for that."""
 
     GREEDY, PLAIN, HOST = 0, 1, 2      # argmax kernel / temperature kernel / top-k or top-p on the host
 
     def __init__(self, device):
         self.device = torch.device(device)
         self._rows = 0
-        self._dev = self._host = None
+        self._sets = []
+        self._turn = 0
 
     def _buffers(self, rows: int):
         if rows > self._rows:
             self._rows = max(64, 2 * rows)
-            self._dev = torch.empty(3 * self._rows, dtype=torch.int32, device=self.device)
-            self._host = torch.empty(3 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda")
-        return self._dev, self._host
+            self._sets = [(torch.empty(3 * self._rows, dtype=torch.int32, device=self.device),
+                           torch.empty(3 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
+                          for _ in range(2)]
+        self._turn ^= 1
+        return self._sets[self._turn]
 
     def _fetch(self, dev: torch.Tensor, host: torch.Tensor, count: int) -> np.ndarray:
         host[:count].copy_(dev[:count], non_blocking=True)
@@ -98,6 +115,35 @@ class DeviceSampler:
             torch.cuda.current_stream(self.device).synchronize()
         return host.numpy()[:count]
 
+    # ------------------------------------------------------------- greedy rows, asked for and read apart
+    def launch_greedy(self, logits: torch.Tensor) -> GreedyTicket:
+        """Queues the argmax of every row and the copy of the results to the host; returns at once."""
+        from .. import kernels
+
+        R = logits.shape[0]
+        dev, host = self._buffers(R)
+        kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
+        host[:2 * R].copy_(dev[:2 * R], non_blocking=True)
+        event = None
+        if self.device.type == "cuda":
+            event = torch.cuda.Event()
+            event.record()
+        return GreedyTicket(R, dev[:R], host, event)
+
+    def collect(self, ticket: GreedyTicket) -> List[int]:
+        """Waits for a ticket's results; the tokens of its rows (ties went to the lowest id)."""
+        if ticket.event is not None:
+            ticket.event.synchronize()
+        R = ticket.rows
+        fetched = ticket.host.numpy()[:2 * R]
+        best, top = fetched[:R], fetched[R:].view(np.float32)
+        if (best < 0).any():
+            raise InvalidArgument(f"a logit of row {int(np.flatnonzero(best < 0)[0])} is NaN")
+        if (top == -np.inf).any():
+            raise InvalidArgument(f"all logits of row {int(np.flatnonzero(top == -np.inf)[0])} are -inf")
+        return best.tolist()
+
+    # ------------------------------------------------------------------------------------ any rows, at once
     def sample_rows(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                     rngs: Sequence[RandomStream]) -> List[int]:
         from .. import kernels
@@ -107,6 +153,8 @@ class DeviceSampler:
             raise InvalidArgument("one set of sampling parameters and one random stream per row")
         kinds = np.fromiter((self.GREEDY if p.greedy else (self.PLAIN if p.top_k == 0 and p.top_p >= 1.0 else self.HOST)
                              for p in params), dtype=np.int8, count=R)
+        if not kinds.any():
+            return self.collect(self.launch_greedy(logits))
         out = np.zeros(R, dtype=np.int64)
         on_device = kinds != self.HOST
         if on_device.any():
