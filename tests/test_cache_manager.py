@@ -50,6 +50,41 @@ def test_pool_sizing_from_a_byte_budget():
         CacheManager(plan, block_size=16, num_blocks=4, dtype="int8")
 
 
+def test_a_budget_pays_for_state_slots_first_and_gives_a_windowed_group_its_share_of_pages():
+    """A model of three kinds of layers: 4 that keep every key, 6 with a window of 256 keys, 2 with a state of
+    1024 floats a request. The budget covers all three; with a context hint the windowed group gets only the
+    pages its requests can hold at a time and the others get what that frees."""
+    needs = [PagedKV(2, 64)] * 4 + [PagedKV(2, 64, window=256)] * 6 + [FixedState((1024,))] * 2
+    plan = plan_cache(needs, [None] * len(needs))
+    full_page, window_page = 2 * 4 * 2 * 16 * 64 * 2, 2 * 6 * 2 * 16 * 64 * 2
+    state = 2 * 8 * 1024 * 4
+    budget = 64 << 20
+    even = CacheManager(plan, block_size=16, budget_bytes=budget, dtype="bfloat16", max_state_slots=8)
+    assert even.state_bytes == state and even.page_bytes == {0: full_page, 1: window_page}
+    assert even.pool_blocks == {0: even.num_blocks, 1: even.num_blocks}
+    assert even.num_blocks == (budget - state) // (full_page + window_page) and even.total_bytes() <= budget
+    hinted = CacheManager(plan, block_size=16, budget_bytes=budget, dtype="bfloat16", max_state_slots=8,
+                          context_hint=8192, step_tokens=512)
+    share = (256 + 512 + 32) / 8192
+    assert hinted.num_blocks == int((budget - state) // (full_page + share * window_page))
+    assert hinted.num_blocks > 2 * even.num_blocks                       # what the windows do not need goes to the rest
+    assert hinted.pool_blocks[1] == -(-int(share * hinted.num_blocks * 1e6) // int(1e6)) or \
+        abs(hinted.pool_blocks[1] - share * hinted.num_blocks) < 1
+    assert hinted.total_bytes() <= budget + window_page                   # (the share is rounded up to a page)
+    assert hinted.capacity_tokens == hinted.num_blocks * 16               # a request's length: the full groups' pages
+    # a long request runs through the small windowed pool, giving pages back as it goes
+    req = hinted.new_request()
+    length, chunk = 0, 512
+    while length < 8192 and hinted.reserve(req, length + chunk):
+        length += chunk
+        hinted.trim(req, length)
+    assert length == 8192 and hinted.pools[1].num_free > 0
+    hinted.release(req)
+    assert hinted.all_free()
+    with pytest.raises(CapacityError, match="state slots"):
+        CacheManager(plan, block_size=16, budget_bytes=state + 1000, dtype="bfloat16", max_state_slots=8)
+
+
 def test_reserve_is_all_or_nothing_and_slots_follow_the_table():
     cache = CacheManager(full_plan(), block_size=4, num_blocks=4)
     a, b = cache.new_request(), cache.new_request()

@@ -68,6 +68,28 @@ def test_the_command_line_generates_the_same_tokens(model_folders):
     assert proc.returncode == 1 and "tie: error:" in proc.stderr
 
 
+def test_the_command_line_runs_a_workload_and_prints_its_report(model_folders, tmp_path):
+    import json
+
+    folder, cfg = model_folders["A"]
+    run = lambda *a: subprocess.run([sys.executable, str(ROOT / "bin" / "tie"), "bench", "-m", folder, "--dtype", "float32",
+                                     "--block-size", "4", "--kv-blocks", "20", "--max-seqs", "4",
+                                     "--max-tokens-per-step", "16", *a], capture_output=True, text=True, timeout=600)
+    proc = run("--synthetic", "9", "--prompt-len", "3:20", "--output-len", "2:6", "--seed", "3", "--json")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    report = json.loads(proc.stdout)
+    assert report["requests"] == 9 and 18 <= report["output_tokens"] <= 54 and report["steps"] > 0
+    assert report["total_tok_per_s"] > 0 and set(report["ttft_ms"]) == {"p50", "p90", "p99"}
+    workload = tmp_path / "w.jsonl"
+    workload.write_text('{"prompt_ids": [1, 2, 3], "max_tokens": 4}\n{"prompt_ids": [9, 8]}\n')
+    proc = run("--prompts", str(workload), "--max-tokens", "3", "--rate", "50")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "requests 2" in proc.stdout and "5 prompt + 7 output" in proc.stdout and "ttft" in proc.stdout
+    workload.write_text('{"prompt": "text"}\n')
+    proc = run("--prompts", str(workload))
+    assert proc.returncode == 1 and "tokenizer" in proc.stderr
+
+
 def test_stop_token_max_tokens_and_pages_returned(model_folders):
     import tie_amd
 

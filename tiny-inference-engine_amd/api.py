@@ -38,9 +38,11 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
     cache_dtype = "float32" if model.mode == FLOAT32 else "bfloat16"
     if kv_blocks is None and kv_mem is None:
         kv_mem = DEFAULT_KV_BYTES
+    context = min(model.spec.max_positions, max_seq_len) if max_seq_len else model.spec.max_positions
     cache = CacheManager(model.cache_plan, block_size=block_size, num_blocks=kv_blocks,
                          budget_bytes=None if kv_blocks is not None else kv_mem, dtype=cache_dtype,
-                         device=model.device, max_state_slots=max_seqs)
+                         device=model.device, max_state_slots=max_seqs, context_hint=context,
+                         step_tokens=prefill_chunk or max_tokens_per_step)
     serving = ServingConfig(max_tokens_per_step=max_tokens_per_step, max_seqs=max_seqs, prefill_chunk=prefill_chunk)
     scheduler = BatchScheduler(cache, SchedulerConfig(serving=serving, policy=policy, aging=aging,
                                                       watermark_blocks=watermark_blocks))

@@ -28,6 +28,7 @@ slots exists and hands out indices, but no memory stands behind them.
 
 from __future__ import annotations
 
+import math
 from typing import Dict, Iterable, List, Optional
 
 import torch
@@ -64,7 +65,15 @@ class RequestCache:
 class CacheManager:
     def __init__(self, plan: CachePlan, block_size: int = 16, num_blocks: Optional[int] = None,
                  budget_bytes: Optional[int] = None, dtype: str = "bfloat16", device=None,
-                 max_state_slots: int = 64):
+                 max_state_slots: int = 64, context_hint: Optional[int] = None, step_tokens: int = 0):
+        """``num_blocks`` pages in every paged group, or as many as ``budget_bytes`` pay for.
+
+        A budget covers everything the cache holds: the state slots of fixed-size groups first, then pages.
+        With ``context_hint`` (the context length requests are expected to reach) a group with a window gets
+        only the share of pages its requests can hold at a time - the window, one step's new tokens
+        (``step_tokens``) and two pages of slack, out of ``context_hint`` - and the groups that keep every key
+        get the rest; without it every paged group gets the same number of pages.
+        """
         if block_size <= 0:
             raise InvalidArgument(f"block_size must be positive, got {block_size}")
         if dtype not in _DTYPES:
@@ -79,23 +88,45 @@ class CacheManager:
         self.device = device
         self.max_state_slots = max_state_slots
         elem = torch.empty((), dtype=_DTYPES[dtype]).element_size()
-        self.bytes_per_block = sum(
-            2 * g.num_planes * g.need.num_kv_heads * block_size * g.need.head_dim * elem
-            for g in plan.groups if isinstance(g.need, PagedKV))
+        self.page_bytes: Dict[int, int] = {
+            g: 2 * plan.groups[g].num_planes * plan.groups[g].need.num_kv_heads * block_size *
+            plan.groups[g].need.head_dim * elem for g in plan.paged_groups}
+        self.bytes_per_block = sum(self.page_bytes.values())      # one page of every paged group
+        self.state_bytes = 0
+        for g in plan.state_groups:
+            need = plan.groups[g].need
+            if need.dtype not in _STATE_DTYPES:
+                raise InvalidArgument(f"state dtype must be one of {', '.join(_STATE_DTYPES)}, got '{need.dtype}'")
+            count = 1
+            for d in need.shape:
+                count *= d
+            self.state_bytes += (plan.groups[g].num_planes * max_state_slots * count *
+                                 torch.empty((), dtype=_STATE_DTYPES[need.dtype]).element_size())
+        cap = _INT32_MAX // block_size                            # slots (page * block_size + offset) must fit in int32
+        share = {g: 1.0 for g in plan.paged_groups}
         if num_blocks is None:
+            if context_hint is not None and context_hint > 0:
+                for g in plan.paged_groups:
+                    window = plan.groups[g].need.window
+                    if window is not None:
+                        share[g] = min(1.0, (window + step_tokens + 2 * block_size) / context_hint)
+            left = budget_bytes - self.state_bytes
             if not plan.paged_groups:
                 num_blocks = 1
             else:
-                num_blocks = budget_bytes // self.bytes_per_block
+                per_full_page = sum(share[g] * self.page_bytes[g] for g in plan.paged_groups)
+                num_blocks = int(left // per_full_page) if left > 0 else 0
                 if num_blocks == 0:
                     raise CapacityError(
-                        f"KV budget of {budget_bytes} bytes is smaller than one {self.bytes_per_block}-byte block")
+                        f"a cache budget of {budget_bytes} bytes does not pay for the {self.state_bytes} bytes of "
+                        f"state slots and one {self.bytes_per_block}-byte page of every group")
         if num_blocks <= 0:
             raise InvalidArgument(f"the cache needs at least one block, got {num_blocks}")
-        # Slots (block * block_size + offset) must fit in int32.
-        self.num_blocks = min(num_blocks, _INT32_MAX // block_size)
+        self.num_blocks = min(num_blocks, cap)                    # pages of the groups that keep every key
+        self.pool_blocks: Dict[int, int] = {
+            g: max(1, min(self.num_blocks, math.ceil(share[g] * self.num_blocks - 1e-9))) for g in plan.paged_groups}
 
-        self.pools: Dict[int, BlockPool] = {g: BlockPool(self.num_blocks) for g in plan.paged_groups}
+        self.pools: Dict[int, BlockPool] = {g: BlockPool(self.pool_blocks[g]) for g in plan.paged_groups}
         self.has_windows = any(plan.groups[g].need.window is not None for g in plan.paged_groups)
         self._free_state_slots: List[int] = list(range(max_state_slots - 1, -1, -1))
         self._state_slot_used = [False] * max_state_slots
@@ -106,14 +137,20 @@ class CacheManager:
                 need = group.need
                 if isinstance(need, PagedKV):
                     self.kv[g] = torch.zeros(
-                        (group.num_planes, 2, self.num_blocks, need.num_kv_heads, block_size, need.head_dim),
+                        (group.num_planes, 2, self.pool_blocks[g], need.num_kv_heads, block_size, need.head_dim),
                         dtype=_DTYPES[dtype], device=device)
                 else:
-                    if need.dtype not in _STATE_DTYPES:
-                        raise InvalidArgument(
-                            f"state dtype must be one of {', '.join(_STATE_DTYPES)}, got '{need.dtype}'")
                     self.state[g] = torch.zeros((group.num_planes, max_state_slots) + tuple(need.shape),
                                                 dtype=_STATE_DTYPES[need.dtype], device=device)
+
+    def total_bytes(self) -> int:
+        """What the cache holds in all: every group's pages and the state slots."""
+        return sum(self.pool_blocks[g] * self.page_bytes[g] for g in self.pool_blocks) + self.state_bytes
+
+    def all_free(self) -> bool:
+        """Whether every page of every group and every state slot is back."""
+        return all(pool.num_free == pool.num_blocks for pool in self.pools.values()) and \
+            len(self._free_state_slots) == self.max_state_slots
 
     # ----------------------------------------------------------------- sizes
     def blocks_for(self, tokens: int) -> int:
@@ -141,7 +178,10 @@ class CacheManager:
 
     @property
     def capacity_tokens(self) -> int:
-        return self.num_blocks * self.block_size
+        """The most tokens one request can hold: the pages of the smallest group that keeps every key (a
+        group with a window gives pages back as a request grows and sets no such limit)."""
+        full = [self.pool_blocks[g] for g in self.pools if self.plan.groups[g].need.window is None]
+        return (min(full) if full else self.num_blocks) * self.block_size if self.pools else _INT32_MAX
 
     # -------------------------------------------------------------- requests
     def new_request(self) -> RequestCache:

@@ -60,7 +60,7 @@ def run_generate(argv: Sequence[str]) -> int:
     print(f"\n[tie] hip | load {load_seconds:.2f} s | prompt {len(opt.prompt)} tok | ttft {ttft * 1e3:.0f} ms | "
           f"prefill {prefill_rate:.1f} tok/s | decode {decode_rate:.1f} tok/s | {generated} tok generated | "
           f"kv {cache.blocks_for(total)} blocks for {total} tok, pool {cache.num_blocks} blocks "
-          f"({cache.bytes_per_block * cache.num_blocks / 2 ** 30:.2f} GiB)", file=sys.stderr)
+          f"({cache.total_bytes() / 2 ** 30:.2f} GiB)", file=sys.stderr)
     if effective < opt.sampling.max_tokens:
         print(f"[tie] note: max_tokens clamped to {effective} by the KV cache / context", file=sys.stderr)
     return 0

@@ -94,7 +94,7 @@ class Engine:
         """The three ceilings on a sequence's length (prompt and generated together), each with its name."""
         page = self.cache.block_size
         return [(self.model.spec.max_positions, "the model's context"),
-                (self.cache.num_blocks * page, f"the cache of {self.cache.num_blocks} pages (see --kv-mem)"),
+                (self.cache.capacity_tokens, f"the cache of {self.cache.num_blocks} pages (see --kv-mem)"),
                 (self.runner.max_blocks_per_seq * page, f"a block-table row of {self.runner.max_blocks_per_seq} pages")]
 
     def add_request(self, prompt: Seq[int], params: Optional[SamplingParams] = None) -> int:
