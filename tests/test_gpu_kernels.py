@@ -533,10 +533,6 @@ def test_gemm_bf16_in_planes(M, N, K, splits):
     planes = torch.full((splits, M, N), float("nan"), dtype=torch.float32, device="cuda")
     kernels.gemm_bf16(x, w, planes, splits=splits)
     close(planes.cpu().to(F64).sum(0), plain.linear(x.cpu(), w.cpu()), 1e-5, f"gemm {M}x{N}x{K} in {splits} planes")
-    assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(512, 4096, 4096) == 4
-    assert kernels.gemm_splits(2048, 4096, 4096) == 1 and kernels.gemm_splits(128, 4096, 256) == 1
-    assert kernels.gemm_splits(2048, 4096, 12288) == 2 and kernels.gemm_splits(1024, 4096, 12288) == 4
-    assert kernels.gemm_splits(2048, 24576, 4096) == 1 and kernels.gemm_splits(300, 200, 1000) == 2
 
 
 def run_decode(case, S, H, Dh, nsplit, window=None):

@@ -54,3 +54,33 @@ def test_a_float16_cache_is_refused_when_it_is_made():
     model = Model(build_qwen3_spec(Qwen3Config.from_json(TINY_A)))
     with pytest.raises(InvalidArgument, match="float16"):
         CacheManager(model.cache_plan, block_size=4, num_blocks=8, dtype="float16")
+
+
+TILE_ROWS_COLS = {4: (256, 256), 5: (256, 128), 6: (128, 256), 7: (128, 128)}
+
+
+def test_the_tiled_product_plans_by_rounds_of_workgroups():
+    """Above 128 rows the tile and the ranges of K come from an estimate of the time; these are the measured choices."""
+    from tie_amd import kernels
+
+    qkv, o, gate_up, down = (6144, 4096), (4096, 4096), (24576, 4096), (4096, 12288)    # [N, K] of an 8B layer
+    # 2048 rows, the prefill step that is measured: 256 x 256 tiles; O alone is too narrow for them and stays whole
+    assert (kernels.gemm_tile(2048, *qkv, True), kernels.gemm_splits(2048, *qkv, True)) == (4, 1)
+    assert (kernels.gemm_tile(2048, *o, True), kernels.gemm_splits(2048, *o, True)) == (6, 1)
+    assert kernels.gemm_tile(2048, *gate_up, True, 1) == 4
+    assert (kernels.gemm_tile(2048, *down, True), kernels.gemm_splits(2048, *down, True)) == (4, 2)
+    assert kernels.gemm_splits(1024, *down, True) == 4
+    # 768 rows: two ranges of 256 x 128 tiles would be 288 workgroups, a second round for 32 of them
+    tile, ranges = kernels.gemm_tile(768, *qkv, True), kernels.gemm_splits(768, *qkv, True)
+    rows, cols = TILE_ROWS_COLS[tile]
+    assert -(-768 // rows) * -(-6144 // cols) * ranges <= 256
+    # every plan: a tile that loads straight into LDS, 1 to 8 ranges, none shorter than 512 of K
+    for N, K in (qkv, o, down, (2048, 2048), (10240, 5120), (5120, 25600)):
+        for M in range(129, 2300, 61):
+            ranges = kernels.gemm_splits(M, N, K, True)
+            assert ranges in (1, 2, 4, 8) and (ranges == 1 or K // ranges >= 512), (M, N, K, ranges)
+            assert kernels.gemm_tile(M, N, K, True) in TILE_ROWS_COLS
+            assert kernels.gemm_tile(M, N, K, True, 1) in TILE_ROWS_COLS
+    # shapes the straight-to-LDS tiles do not take keep the older tiles and their rule
+    assert kernels.gemm_splits(300, 200, 1000) == 2 and kernels.gemm_tile(300, 200, 1000) == 1
+    assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(128, 4096, 256) == 1

@@ -606,10 +606,17 @@ static bool gemm_dma_takes(const void* x, const void* w, const void* out, int N,
 }
 
 // Which tile, and how many ranges of K (planes of partial sums that the caller adds), a product takes when
-// left to choose. Measured on the four weight shapes of an 8B model for 128 to 2048 rows: the 256 x 256
-// tile wherever it gives most CUs a workgroup by itself; else enough ranges of K to get there - with
-// the 256 x 256 tile over a long K, with 256 x 128 over a short one, each range at least 1024 long;
-// few rows (one row tile, half empty) stay on the 128 x 128 tile with up to 8 ranges.
+// left to choose.
+//
+// Up to 128 rows over packed weights: rules measured on the projections of the 1.7B, 8B and 32B shapes.
+// Above that, for shapes the straight-to-LDS tiles take: the cheapest of (tile, ranges) by an estimate of
+// the time, whose terms were fitted to sweeps over the same shapes at 256 to 2048 rows:
+//   * a compute unit holds one workgroup (two of the 128 x 128 tile), so the workgroups run in rounds of
+//     256; a round that is nearly empty lasts as long as a full one, which is what a rule by thresholds
+//     gets wrong (768 rows of 256 x 128 tiles over 6144 columns and two ranges: 288 workgroups, two rounds);
+//   * a round is a few microseconds of start and end plus its slices of 32 along K at the tile's own pace;
+//   * every plane is written once here and read once by its consumer.
+// Without the straight-to-LDS tiles (odd K or N) the older tiles and their rule stand.
 struct GemmPlan { int tile, splits; };
 
 static int legacy_splits(int M, int N, int K) {
@@ -626,56 +633,66 @@ static int legacy_splits(int M, int N, int K) {
   return 1;
 }
 
-static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, bool may_split, bool packed) {
-  const long rows256 = (M + 255) / 256;
-  const long t256 = rows256 * ((N + 255) / 256), t128 = rows256 * ((N + 127) / 128);
-  auto ranges = [&](long tiles, long want, int shortest) {
-    for (int r = 1; r <= 8; r *= 2)
-      if (tiles * r >= want && K / r >= shortest) return r;
-    return 0;
+struct DmaTile { int id, bm, bn; float start_us, full_us, slice_us; int per_cu; };
+// start_us: a round's start and end; full_us: what a round costs more when it fills every compute unit (measured
+// for the 256 x 256 tile only, whatever the length of K: 256 workgroups of it start about 11 us later than 192);
+// slice_us: one slice of 32 along K with the compute unit to itself.
+static const DmaTile kDmaTiles[] = {{4, 256, 256, 8.f, 11.f, 0.67f, 1}, {5, 256, 128, 5.f, 0.f, 0.53f, 1},
+                                    {6, 128, 256, 5.f, 0.f, 0.50f, 1}, {7, 128, 128, 4.f, 0.f, 0.36f, 2}};
+
+static float estimated_us(const DmaTile& t, int M, int N, int K, int ranges) {
+  const long wgs = static_cast<long>((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * ranges;
+  const int k_slices = K / GD_BK;
+  const int slices = (k_slices + ranges - 1) / ranges;
+  const long slots = 256L * t.per_cu;
+  const float pace = t.slice_us * (t.per_cu > 1 && wgs > 256 ? 1.6f : 1.0f);   // two workgroups share the matrix cores
+  auto round_us = [&](float fill) {
+    const float crowded = fminf(fmaxf((fill - 0.75f) * 4.0f, 0.f), 1.f);
+    return t.start_us + t.full_us * crowded + slices * pace;
   };
+  float us = static_cast<float>(wgs / slots) * round_us(1.0f);
+  if (wgs % slots) us += round_us(static_cast<float>(wgs % slots) / slots);
+  const float plane_mb = static_cast<float>(M) * N * 4e-6f;
+  return us + ranges * plane_mb * (1.0f / 6.0f + 1.0f / 5.0f);   // written here, read by the consumer: MB / (TB/s) = us
+}
+
+// splits: 0 = free to choose (the caller adds planes), else the number of ranges the caller has fixed (1: none).
+static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, int splits, bool packed) {
+  const bool may_split = splits == 0;
   if (straight_to_lds && packed && M <= 128) {
     // Few rows over packed weights: tiles of 64 or 128 rows (measured on the projections of the 1.7B, 8B and
     // 32B shapes at 48 to 128 rows). Wide weights take 256 columns a tile, narrow ones 128 and more ranges of K.
     const bool wide = M <= 64 ? N >= 8192 : N >= 5120;
     const int tile = M <= 64 ? (wide ? 8 : 9) : (wide ? 6 : 7);
-    if (!may_split) return {tile, 1};
+    if (!may_split) return {tile, splits};
     const long tiles = (N + (wide ? 255 : 127)) / (wide ? 256 : 128);
-    int r = ranges(tiles, 192, 512);
-    if (r == 0)
-      for (r = 8; r > 1 && K / r < 512; r /= 2) {}
+    for (int r = 1; r <= 8; r *= 2)
+      if (tiles * r >= 192 && K / r >= 512) return {tile, r};
+    int r = 8;
+    while (r > 1 && K / r < 512) r /= 2;
     return {tile, r};
   }
-  if (straight_to_lds && packed && M <= 256) {
-    // Up to 256 rows over a weight so narrow, or a K so short, that even 256 x 128 tiles over every allowed range
-    // of K leave most compute units idle (the 1.7B shape's projections): 128 x 128.
-    int most = 8;
-    while (most > 1 && K / most < 512) most /= 2;
-    if (t128 * (may_split ? most : 1) < 192) {
-      const long t7 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-      if (!may_split) return {7, 1};
-      const int r7 = ranges(t7, 192, 512);
-      return {7, r7 ? r7 : most};
+  if (straight_to_lds && M > 128) {
+    GemmPlan best = {4, may_split ? 1 : splits};
+    float best_us = 0.f;
+    const int k_slices = K / GD_BK;
+    for (int r = may_split ? 1 : splits; r <= (may_split ? 8 : splits); r *= 2) {
+      const int per = (k_slices + r - 1) / r;
+      if (may_split && r > 1 && (K / r < 512 || k_slices - per * (r - 1) < 3)) break;
+      for (const DmaTile& t : kDmaTiles) {
+        const float us = estimated_us(t, M, N, K, r);
+        if (best_us == 0.f || us < best_us * 0.98f) {       // ties go to fewer planes, then to the larger tile
+          best = {t.id, r};
+          best_us = us;
+        }
+      }
     }
-  }
-  if (straight_to_lds && M >= 256) {
-    if (t256 >= 160) return {4, 1};
-    if (!may_split) return {packed ? 6 : (t128 >= 128 ? 5 : 1), 1};   // 128 x 256: twice the workgroups of 256 x 256
-    const int r256 = ranges(t256, 160, 1024), r128 = ranges(t128, 192, 1024);
-    if (K >= 8192 && r256) return {4, r256};
-    if (r128) return {5, r128};
-    if (r256) return {4, r256};
-  }
-  if (packed) {
-    // Only the tiles that load straight into LDS read the packed layout: 256 x 128, with as many
-    // ranges of K (512 or longer) as it takes to give most CUs a workgroup, at most 8.
-    if (!may_split) return {5, 1};
-    int r = ranges(t128, 192, 512);
-    if (r == 0)
-      for (r = 8; r > 1 && K / r < 512; r /= 2) {}
-    return {5, r};
+    return best;
   }
   if (may_split) return {1, legacy_splits(M, N, K)};
+  if (splits > 1) return {1, splits};
+  const long rows256 = (M + 255) / 256;
+  const long t256 = rows256 * ((N + 255) / 256), t128 = rows256 * ((N + 127) / 128);
   return {t256 >= 160 ? 2 : (t128 >= 192 ? 3 : 1), 1};
 }
 
@@ -692,7 +709,13 @@ extern "C" int tie_gemm_bf16_wins_few_rows(int M, int N, int K, int packed, int 
 // partial sums: few rows over a narrow weight give too few workgroups otherwise.
 extern "C" int tie_gemm_bf16_splits(int M, int N, int K, int packed) {
   if (packed && !straight_to_lds_shape(N, K)) return 1;
-  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), true, packed != 0).splits;
+  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), 0, packed != 0).splits;
+}
+
+// The tile a product left to choose runs on (the numbers of tie_gemm_bf16's `tile`), with `splits` ranges of K
+// fixed by the caller (1: none) or 0 for the plan's own number; for tests and sweeps.
+extern "C" int tie_gemm_bf16_tile(int M, int N, int K, int packed, int splits) {
+  return gemm_plan(M, N, K, straight_to_lds_shape(N, K), splits, packed != 0).tile;
 }
 
 // out_dtype: TIE_F32 or TIE_BF16; accumulate adds into a float32 output; gated (bfloat16 output of N / 2
@@ -716,12 +739,7 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
   if (packed && (N % 16 != 0 || !straight || (tile != 0 && (tile < 4 || tile > 9)))) return TIE_BAD_ARGUMENT;
   if (tile == 0) {
-    if (splits > 1) {
-      const GemmPlan plan = gemm_plan(M, N, K, straight, true, packed != 0);
-      tile = plan.splits == splits ? plan.tile : (packed ? 5 : 1);
-    } else {
-      tile = gemm_plan(M, N, K, straight, false, packed != 0).tile;
-    }
+    tile = gemm_plan(M, N, K, straight, splits, packed != 0).tile;
   } else if (tile < 4 && splits > 1) {
     tile = 1;
   }

@@ -75,6 +75,7 @@ _SIGNATURES = {
     },
     "gemm_bf16": {
         "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
+        "tie_gemm_bf16_tile": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "tie_gemm_bf16_wins_few_rows": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "tie_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void],
@@ -402,6 +403,11 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
 def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
     """Ranges of K a product of M > 64 rows over a ``[N, K]`` weight is best cut into when its caller adds partial sums."""
     return int(_lib("gemm_bf16").tie_gemm_bf16_splits(M, N, K, int(packed)))
+
+
+def gemm_tile(M: int, N: int, K: int, packed: bool = False, splits: int = 0) -> int:
+    """The tile (``gemm_bf16``'s numbering) a product left to choose runs on, with ``splits`` ranges of K fixed (0: the plan's own)."""
+    return int(_lib("gemm_bf16").tie_gemm_bf16_tile(M, N, K, int(packed), splits))
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, tile: int = 0,
