@@ -42,7 +42,7 @@ constexpr int KS = DH / 16;            // k-steps of the score product
 constexpr int DT = (DH + 31) / 32;     // 32-row tiles of O^T; rows beyond DH are zero
 constexpr int KT = 64;                 // keys per tile
 constexpr int KROW = DH + 8;           // LDS row of a key, padded: 16-byte reads of 16 lanes hit distinct banks
-constexpr int VROW = KT + 4;           // LDS row of one value dimension, padded likewise for 8-byte reads
+constexpr int VROW = KT + 8;           // LDS row of one value dimension, padded likewise; its keys are permuted (below)
 constexpr int THREADS = 256;
 constexpr int K_CHUNKS = KT * DH / 8;          // 16-byte pieces of a key tile
 constexpr int V_CHUNKS = DT * 32 * (KT / 8);   // 8-key pieces of a value tile (rows beyond DH are zeros)
@@ -133,10 +133,13 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
     }                                                                                                              \
     _Pragma("unroll") for (int i_ = 0; i_ < V_PER_THREAD; ++i_) {                                                  \
       const int c_ = threadIdx.x + i_ * THREADS;                                                                   \
-      if (V_CHUNKS % THREADS == 0 || c_ < V_CHUNKS) { /* rows are 8-byte aligned, not 16 */                        \
-        u32x2_t* dst_ = reinterpret_cast<u32x2_t*>((v_dst) + (c_ / (KT / 8)) * VROW + (c_ % (KT / 8)) * 8);        \
-        dst_[0] = u32x2_t{vreg[i_].x, vreg[i_].y};                                                                 \
-        dst_[1] = u32x2_t{vreg[i_].z, vreg[i_].w};                                                                 \
+      if (V_CHUNKS % THREADS == 0 || c_ < V_CHUNKS) {                                                              \
+        /* Within a block of 16 keys the order in LDS is 0-3, 8-11, 4-7, 12-15: the 8 keys a lane supplies to */   \
+        /* one matrix instruction (4 keys, skip 4, 4 keys) then lie together and are read as one 16-byte piece. */ \
+        const int kg_ = c_ % (KT / 8);                                                                             \
+        bf16_t* row_ = (v_dst) + (c_ / (KT / 8)) * VROW + (kg_ / 2) * 16 + (kg_ % 2) * 4;                          \
+        *reinterpret_cast<u32x2_t*>(row_) = u32x2_t{vreg[i_].x, vreg[i_].y};                                       \
+        *reinterpret_cast<u32x2_t*>(row_ + 8) = u32x2_t{vreg[i_].z, vreg[i_].w};                                   \
       }                                                                                                            \
     }                                                                                                              \
   }
@@ -290,15 +293,13 @@ __global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
           for (int v = 0; v < 16; ++v) acc[dt][v] *= corr;
       }
       m = m_new;
-      // B operand slot hi*8 + e of 16-key block j holds key j*16 + hi*4 + e%4 + 8*(e/4): read V^T likewise.
+      // B operand slot hi*8 + e of 16-key block j holds key j*16 + hi*4 + e%4 + 8*(e/4): V^T lies in that order.
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           Frag a;
-          const bf16_t* vr = v_lds + (dt * 32 + r32) * VROW + j * 16 + hi * 4;
-          a.u2[0] = *reinterpret_cast<const uint2*>(vr);
-          a.u2[1] = *reinterpret_cast<const uint2*>(vr + 8);
+          a.u4 = *reinterpret_cast<const uint4*>(v_lds + (dt * 32 + r32) * VROW + j * 16 + hi * 8);
           acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, acc[dt], 0, 0, 0);
         }
       // The output accumulators are rescaled by ordinary multiplications: keep them in vector
