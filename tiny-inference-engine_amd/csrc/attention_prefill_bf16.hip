@@ -147,7 +147,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 // items: [num_items][2] = (sequence, index of its first new row handled here); the last items run first.
 // WIDE: the block size is a multiple of 8, so 8 keys of one value dimension lie together in a page.
 template <int HC, int QC, bool WIDE>
-__global__ __launch_bounds__(THREADS) void attention_prefill_kernel(
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
