@@ -84,3 +84,18 @@ def test_the_tiled_product_plans_by_rounds_of_workgroups():
     # shapes the straight-to-LDS tiles do not take keep the older tiles and their rule
     assert kernels.gemm_splits(300, 200, 1000) == 2 and kernels.gemm_tile(300, 200, 1000) == 1
     assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(128, 4096, 256) == 1
+
+
+def test_the_prefill_attention_kernel_refuses_caches_it_cannot_address():
+    """Its addresses are 32-bit counts of 8 bytes, a page's number times the page's size by a 24-bit multiply."""
+    import torch
+    from tie_amd import kernels
+
+    def plane(pages, kv_heads, block, dim):
+        return torch.empty((pages, kv_heads, block, dim), dtype=torch.bfloat16, device="meta")
+
+    assert kernels.prefill_addressable(plane(300_000, 8, 16, 128))          # 9.8 GB: a long cache of an 8B model
+    assert kernels.prefill_addressable(plane((1 << 20) - 1, 8, 16, 128))    # just under 32 GB
+    assert not kernels.prefill_addressable(plane(1 << 20, 8, 16, 128))      # 32 GB
+    assert not kernels.prefill_addressable(plane(4, 64, 4096, 256))         # a page of 128 MB
+    assert not kernels.prefill_addressable(plane(1 << 24, 1, 4, 16))        # 2^24 pages

@@ -63,6 +63,11 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 // calling kernel. Key positions are clamped into [first, last]: pages before or after the range this
 // workgroup may touch are never addressed (their table entries need not be valid); clamped keys are
 // masked by position later. A macro, so that the register arrays are plain locals of the kernel.
+//
+// Addresses are formed in units of 8 bytes from 32-bit numbers (a page's number times the units of a page
+// with the 24-bit multiply, which runs at full rate): the address arithmetic of the eight pieces a thread
+// copies per tile weighs as much as the softmax when done in 64 bits. The host refuses caches of 32 GB or
+// more and pages of 2^24 units or more, which this cannot address.
 #define PAGE_OF(kp) ((kp) >> block_shift)
 #define OFFSET_OF(kp) ((kp) & (block_size - 1))
 // LOAD_PAGES looks up the pages of every piece of a tile this thread copies; LOAD_TILE then reads the
@@ -80,10 +85,10 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
       const int c_ = threadIdx.x + i_ * THREADS;                                                                   \
       const int kg_ = c_ % (KT / 8);                                                                               \
       const bool live_ = (V_CHUNKS % THREADS == 0 || c_ < V_CHUNKS) && (DH % 32 == 0 || c_ / (KT / 8) < DH);       \
-      const int kp0_ = min(max(base_ + kg_ * 8, wg_first / VG * VG), wg_last / VG * VG);                           \
+      const int kp0_ = min(max(base_ + kg_ * 8, first_v), last_v);                                                 \
       vpage[i_][0] = live_ ? table[PAGE_OF(kp0_)] : 0;                                                             \
       if (!WIDE) {                                                                                                 \
-        const int kp1_ = min(max(base_ + kg_ * 8 + 4, wg_first / VG * VG), wg_last / VG * VG);                     \
+        const int kp1_ = min(max(base_ + kg_ * 8 + 4, first_v), last_v);                                           \
         vpage[i_][1] = live_ ? table[PAGE_OF(kp1_)] : 0;                                                           \
       }                                                                                                            \
     }                                                                                                              \
@@ -96,26 +101,27 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
       const int c_ = threadIdx.x + i_ * THREADS;                                                                   \
       if (K_CHUNKS % THREADS == 0 || c_ < K_CHUNKS) {                                                              \
         const int kp_ = min(max(base_ + c_ / (DH / 8), wg_first), wg_last);                                        \
-        kreg[i_] = *reinterpret_cast<const u32x4_t*>(k_cache + static_cast<size_t>(kpage[i_]) * page_stride +      \
-                                                     head_off + static_cast<size_t>(OFFSET_OF(kp_)) * DH +         \
-                                                     (c_ % (DH / 8)) * 8);                                         \
+        const uint32_t unit_ = __umul24(static_cast<uint32_t>(kpage[i_]), page_units) + head_units +               \
+                               static_cast<uint32_t>(OFFSET_OF(kp_)) * (DH / 4) + (c_ % (DH / 8)) * 2;             \
+        kreg[i_] = *reinterpret_cast<const u32x4_t*>(k_units + unit_);                                             \
       }                                                                                                            \
     }                                                                                                              \
     _Pragma("unroll") for (int i_ = 0; i_ < V_PER_THREAD; ++i_) {                                                  \
       const int c_ = threadIdx.x + i_ * THREADS;                                                                   \
       const int d_ = c_ / (KT / 8), kg_ = c_ % (KT / 8);                                                           \
       if ((V_CHUNKS % THREADS == 0 || c_ < V_CHUNKS) && (DH % 32 == 0 || d_ < DH)) {                               \
-        const int kp0_ = min(max(base_ + kg_ * 8, wg_first / VG * VG), wg_last / VG * VG);                         \
-        const bf16_t* v0_ = v_cache + static_cast<size_t>(vpage[i_][0]) * page_stride + head_off +                 \
-                            static_cast<size_t>(d_) * block_size + OFFSET_OF(kp0_);                                \
+        const int kp0_ = min(max(base_ + kg_ * 8, first_v), last_v);                                               \
+        const uint32_t row_ = head_units + static_cast<uint32_t>(d_) * row_units;   /* the same for every tile */  \
+        const uint32_t unit0_ = __umul24(static_cast<uint32_t>(vpage[i_][0]), page_units) + row_ +                 \
+                                (static_cast<uint32_t>(OFFSET_OF(kp0_)) >> 2);                                     \
         if (WIDE) {                                                                                                \
-          vreg[i_] = *reinterpret_cast<const u32x4_t*>(v0_);                                                       \
+          vreg[i_] = *reinterpret_cast<const u32x4_t*>(v_units + unit0_);                                          \
         } else {                                                                                                   \
-          const int kp1_ = min(max(base_ + kg_ * 8 + 4, wg_first / VG * VG), wg_last / VG * VG);                   \
-          const u32x2_t h0_ = *reinterpret_cast<const u32x2_t*>(v0_);                                              \
-          const u32x2_t h1_ = *reinterpret_cast<const u32x2_t*>(                                                   \
-              v_cache + static_cast<size_t>(vpage[i_][1]) * page_stride + head_off +                               \
-              static_cast<size_t>(d_) * block_size + OFFSET_OF(kp1_));                                             \
+          const int kp1_ = min(max(base_ + kg_ * 8 + 4, first_v), last_v);                                         \
+          const uint32_t unit1_ = __umul24(static_cast<uint32_t>(vpage[i_][1]), page_units) + row_ +               \
+                                  (static_cast<uint32_t>(OFFSET_OF(kp1_)) >> 2);                                   \
+          const u32x2_t h0_ = v_units[unit0_];                                                                     \
+          const u32x2_t h1_ = v_units[unit1_];                                                                     \
           vreg[i_] = u32x4_t{h0_.x, h0_.y, h1_.x, h1_.y};                                                          \
         }                                                                                                          \
       } else {                                                                                                     \
@@ -216,9 +222,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     tile_end = min(tile_end, tile_begin + per - 1);
   }
   const bool empty = tile_begin > tile_end;                      // uniform: a short row range has fewer tiles than splits
-  const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
-  const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
+  // In units of 8 bytes (4 elements): a page, this KV head inside a page, one value dimension's keys of a page.
+  const uint32_t page_units = static_cast<uint32_t>(KVH) * block_size * (DH / 4);
+  const uint32_t head_units = static_cast<uint32_t>(kvh) * block_size * (DH / 4);
+  const uint32_t row_units = static_cast<uint32_t>(block_size) / 4;
+  const u32x2_t* k_units = reinterpret_cast<const u32x2_t*>(k_cache);
+  const u32x2_t* v_units = reinterpret_cast<const u32x2_t*>(v_cache);
   constexpr int VG = WIDE ? 8 : 4;   // keys of one value dimension read in one piece
+  const int first_v = wg_first / VG * VG, last_v = wg_last / VG * VG;
   u32x4_t kreg[K_PER_THREAD], vreg[V_PER_THREAD];
   int kpage[K_PER_THREAD], vpage[V_PER_THREAD][WIDE ? 1 : 2];
   if (!empty) {
@@ -239,15 +250,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const int base = tile * KT;
     if (wave_active && base <= wave_last) {
       floatx16 sc[2];
+      const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) sc[u][v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           Frag a;
           a.u4 = *reinterpret_cast<const uint4*>(k_lds + (u * 32 + r32) * KROW + ks * 16 + hi * 8);
-          sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, sc[u], 0, 0, 0);
+          sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
         }
       }
       // Element v of sc[u] is key base + u*32 + 8*(v/4) + hi*4 + v%4 against this lane's row.

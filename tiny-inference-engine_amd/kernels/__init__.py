@@ -661,6 +661,15 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
                                           out.data_ptr(), R, V, _stream()), "sample")
 
 
+PREFILL_MAX_CACHE_BYTES = 1 << 35      # the prefill attention kernel addresses a cache plane in 32-bit units of 8 bytes
+
+
+def prefill_addressable(k_cache: torch.Tensor) -> bool:
+    """Whether the prefill attention kernel can address this cache plane: under 32 GB, pages under 128 MB, under 2^24 pages."""
+    pages, page_bytes = k_cache.shape[0], k_cache[0].numel() * k_cache.element_size()
+    return pages * page_bytes < PREFILL_MAX_CACHE_BYTES and page_bytes < (1 << 27) and pages < (1 << 24)
+
+
 def mfma_block_size(block_size: int) -> bool:
     """Block sizes the matrix-core attention kernels take: powers of two from 4 (others go to the generic kernel)."""
     return block_size >= 4 and block_size & (block_size - 1) == 0
@@ -767,6 +776,9 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if Dh not in MFMA_HEAD_DIMS or H % KVH or not mfma_block_size(bs):
         raise InvalidArgument(f"attention_prefill_bf16 takes head sizes in steps of 16 up to 256 and block sizes 4, 8, "
                               f"16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+    if not prefill_addressable(k_cache):
+        raise InvalidArgument(f"attention_prefill_bf16 addresses cache planes under 32 GB (pages under 128 MB, under 2^24 "
+                              f"pages); got {NB} pages of {k_cache[0].numel() * k_cache.element_size()} bytes")
     _i32(query_start, "query_start")
     _i32(context_lens, "context_lens")
     _i32(block_tables, "block tables")
@@ -852,6 +864,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids)
+        if items is not None and not prefill_addressable(k_cache):
+            # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
+            # (which runs every row of the step; the single rows above are simply computed again).
+            paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
+                                    batch.seq_of_row, num_heads, scale, window)
+            return
         if items is not None:
             rows = q.shape[0]
             nsplit = prefill_splits(num_items, KVH, G, batch.plan_context, rows)
