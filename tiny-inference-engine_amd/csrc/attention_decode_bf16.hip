@@ -266,7 +266,7 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
 #undef LAUNCH
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
-  attention_merge_kernel<<<dim3(H, num_seqs), attention_merge_threads(nsplit), 0, stream>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), nullptr, query_start, seq_ids, H, nsplit);
+  launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), nullptr, query_start, seq_ids, H, nsplit, num_seqs,
+                         stream);
   return tie_launch_status();
 }

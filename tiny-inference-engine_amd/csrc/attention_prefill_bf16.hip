@@ -444,7 +444,7 @@ extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, co
   else LAUNCH(1, 4);
 #undef LAUNCH
   if (status != TIE_OK || nsplit == 1) return status;
-  attention_merge_kernel<<<dim3(H, num_merge_rows), attention_merge_threads(nsplit), 0, stream>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, nullptr, nullptr, H, nsplit);
+  launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, nullptr, nullptr, H, nsplit,
+                         num_merge_rows, stream);
   return tie_launch_status();
 }
