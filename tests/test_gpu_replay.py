@@ -85,6 +85,26 @@ def test_all_ways_of_cutting(folders, name, dtype):
                 assert float((a - b).abs().max() / a.abs().max()) < 1e-5, f"{name}: whole vs {label}, request {rid}"
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_single_rows_beside_portions_on_either_attention_kernel(folders, name, monkeypatch):
+    """In a mixed step a few single decoded rows run in the prefill attention kernel beside the portions, many in
+    the decode kernel: the mixed trace through both ways (the traces above only meet the first)."""
+    from tie_amd import kernels
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["bfloat16"][name]
+    requests = th.make_requests(cfg["vocab_size"], LENGTHS[name], seed=6)
+    want = reference_logits(folder, cfg, requests)
+    steps, peak = th.mixed(requests, max_live=4, seed=4)
+    assert any(sum(len(e["tokens"]) == 1 for e in s["entries"]) and any(len(e["tokens"]) > 1 for e in s["entries"])
+               for s in steps), "no step mixes single rows with a portion"
+    got = {}
+    for ride_along in (kernels.SINGLE_ROWS_RIDE_ALONG, 0):
+        monkeypatch.setattr(kernels, "SINGLE_ROWS_RIDE_ALONG", ride_along)
+        got[ride_along] = th.collect(TraceReplayer.from_folder(folder, "bfloat16", peak, block_size=BLOCK_SIZE[name]), steps)
+        check(got[ride_along], want, "bfloat16", f"{name}/bfloat16/mixed, single rows riding along up to {ride_along}")
+
+
 def test_pages_are_used_again(folders):
     """A pool of exactly one request's pages serves request after request."""
     from tie_amd.engine.replay import TraceReplayer

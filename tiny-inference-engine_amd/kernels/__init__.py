@@ -661,6 +661,10 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
                                           out.data_ptr(), R, V, _stream()), "sample")
 
 
+# Up to this many workgroups of single decoded rows run in the prefill attention kernel beside a step's prompt
+# portions rather than in a launch (and a merge) of the decode kernel of their own; a row costs a 32-row tile
+# there, so many of them are better off in the decode kernel, which takes a group's heads as its columns.
+SINGLE_ROWS_RIDE_ALONG = 128
 PREFILL_MAX_CACHE_BYTES = 1 << 35      # the prefill attention kernel addresses a cache plane in 32-bit units of 8 bytes
 
 
@@ -845,6 +849,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             single = [s for s, n in enumerate(new) if n == 1] if G <= 16 else []
             if len(single) == len(new):
                 single = []                                   # nothing but single rows and yet not a decode step
+            elif len(single) * KVH * -(-G // min(G, 4)) <= SINGLE_ROWS_RIDE_ALONG:
+                single = []         # a few single rows: items of the prefill kernel, one launch and one merge less
             taken = set(single)
             items = [it for it in prefill_items(new, G) if it[0] not in taken]
             starts = [0]
