@@ -124,22 +124,33 @@ class Workspace:
     the addresses stay put, which replaying a recorded step relies on.
     """
 
+    MAX_VIEWS = 4096      # views kept for reuse; steps of ever new sizes start the memo afresh
+
     def __init__(self, device):
         self.device = device
-        self._buffers: Dict[str, torch.Tensor] = {}
+        self._buffers: Dict[Any, torch.Tensor] = {}
+        self._views: Dict[Any, torch.Tensor] = {}     # (name, dtype, shape) -> view: a layer asks again every step
         self.generation = 0   # grows whenever a buffer is replaced: recorded steps are then stale
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         numel = 1
         for d in shape:
             numel *= int(d)
-        key = f"{name}:{dtype}"
+        key = (name, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < numel:
             buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self.generation += 1
-        return buf[:numel].view(*shape)
+            self._views = {k: v for k, v in self._views.items() if k[:2] != key}     # they showed the old buffer
+        if len(self._views) >= self.MAX_VIEWS:
+            self._views.clear()
+        view = self._views[(name, dtype, shape)] = buf[:numel].view(*shape)
+        return view
 
     def nbytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._buffers.values())
