@@ -105,6 +105,36 @@ def test_single_rows_beside_portions_on_either_attention_kernel(folders, name, m
         check(got[ride_along], want, "bfloat16", f"{name}/bfloat16/mixed, single rows riding along up to {ride_along}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_layers_of_one_shape_run_from_one_layers_launch_list(tmp_path, dtype, use_graphs):
+    """With four or more layers alike, only the first three run the parts' code in a step; the others run the
+    same launches with their own weights and cache planes. Every logit must be the very bits of a run in which
+    every layer runs its own code, through portions, mixed steps and decoding (recorded into graphs or not)."""
+    from conftest import TINY_B
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.weights.random_init import write_random_model
+
+    cfg = dict(TINY_B, num_hidden_layers=7)
+    folder = tmp_path / "seven_layers"
+    write_random_model(folder, cfg, seed=31, dtype=dtype)
+    requests = th.make_requests(cfg["vocab_size"], [150, 37, 90, 64, 121], seed=8)
+    want = reference_logits(folder, cfg, requests)
+    steps, peak = th.mixed(requests, max_live=4, seed=5)
+    got = {}
+    for replay in (True, False):
+        rep = TraceReplayer.from_folder(folder, dtype, peak, block_size=16, use_graphs=use_graphs)
+        rep.model.replay_layers = replay
+        assert rep.model._alike == {0: 7}
+        got[replay] = th.collect(rep, steps)
+        assert (rep.model.layers_replayed > 0) == replay
+        assert rep.cache.num_free() == rep.cache.num_blocks
+    check(got[True], want, dtype, f"seven layers alike/{dtype}")
+    for rid in requests:
+        for position, row in got[True][rid].items():
+            assert torch.equal(row, got[False][rid][position]), f"request {rid}, position {position}"
+
+
 def test_pages_are_used_again(folders):
     """A pool of exactly one request's pages serves request after request."""
     from tie_amd.engine.replay import TraceReplayer

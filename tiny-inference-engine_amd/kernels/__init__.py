@@ -142,6 +142,34 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+_recording: Optional[list] = None     # while a list: every launch is also noted in it, as (function, arguments, name)
+
+
+def start_recording() -> list:
+    """From now on every kernel launch is also noted, as ``(function, arguments, name)``; returns the list."""
+    global _recording
+    _recording = []
+    return _recording
+
+
+def stop_recording() -> None:
+    global _recording
+    _recording = None
+
+
+def _call(fn, what: str, *args) -> None:
+    """One kernel launch through the C interface: its status checked, the call noted if launches are being recorded."""
+    status = fn(*args)
+    if _recording is not None:
+        _recording.append((fn, args, what))
+    _check(status, what)
+
+
+def replay_call(fn, what: str, args) -> None:
+    """A noted launch again, with the arguments given (see ``models.builder``: layers of one shape)."""
+    _check(fn(*args), what)
+
+
 def _check(status: int, what: str) -> None:
     if status == 0:
         return
@@ -220,8 +248,8 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     V, D = table.shape
     _i32(ids, "token ids")
     _f32(out, "embedding output", (T, D))
-    _check(_lib("elementwise").tie_embed(table.data_ptr(), _code(table, "embedding table"), ids.data_ptr(),
-                                         out.data_ptr(), T, D, _stream()), "embed")
+    _call(_lib("elementwise").tie_embed, "embed", table.data_ptr(), _code(table, "embedding table"), ids.data_ptr(),
+                                         out.data_ptr(), T, D, _stream())
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
@@ -239,9 +267,9 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
             raise InvalidArgument(f"rms_norm output {list(out.shape)} does not match input {list(x.shape)}")
     else:
         _i32(rows, "rms_norm rows", R)
-    _check(_lib("elementwise").tie_rms_norm(x.data_ptr(), _code(x, "rms_norm input"), weight.data_ptr(), float(eps),
+    _call(_lib("elementwise").tie_rms_norm, "rms_norm", x.data_ptr(), _code(x, "rms_norm input"), weight.data_ptr(), float(eps),
                                             out.data_ptr(), _code(out, "rms_norm output"), _ptr(rows), R, n,
-                                            _stream()), "rms_norm")
+                                            _stream())
 
 
 def add_partials(x: torch.Tensor, partials: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 0.0,
@@ -264,9 +292,9 @@ def add_partials(x: torch.Tensor, partials: torch.Tensor, weight: Optional[torch
         if tuple(out.shape) != (R, n):
             raise InvalidArgument(f"rms_norm output {list(out.shape)} does not match input {[R, n]}")
         code = _code(out, "rms_norm output")
-    _check(_lib("elementwise").tie_add_partials_rms_norm(
+    _call(_lib("elementwise").tie_add_partials_rms_norm, "add_partials",
         x.data_ptr(), partials.data_ptr(), R * n, partials.shape[0], _ptr(weight), float(eps), _ptr(out), code, R, n,
-        _stream()), "add_partials")
+        _stream())
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
@@ -276,8 +304,8 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     T, two_i = gate_up.shape
     if two_i % 2 or tuple(out.shape) != (T, two_i // 2):
         raise InvalidArgument(f"swiglu: input {list(gate_up.shape)} and output {list(out.shape)} do not match")
-    _check(_lib("elementwise").tie_swiglu(gate_up.data_ptr(), _code(gate_up, "swiglu input"), out.data_ptr(),
-                                          _code(out, "swiglu output"), T, two_i // 2, _stream()), "swiglu")
+    _call(_lib("elementwise").tie_swiglu, "swiglu", gate_up.data_ptr(), _code(gate_up, "swiglu input"), out.data_ptr(),
+                                          _code(out, "swiglu output"), T, two_i // 2, _stream())
 
 
 def cast(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -285,8 +313,8 @@ def cast(x: torch.Tensor, out: torch.Tensor) -> None:
     _gpu(out, "cast output")
     if x.numel() != out.numel():
         raise InvalidArgument("cast: sizes differ")
-    _check(_lib("elementwise").tie_cast(x.data_ptr(), _code(x, "cast input"), out.data_ptr(),
-                                        _code(out, "cast output"), x.numel(), _stream()), "cast")
+    _call(_lib("elementwise").tie_cast, "cast", x.data_ptr(), _code(x, "cast input"), out.data_ptr(),
+                                        _code(out, "cast output"), x.numel(), _stream())
 
 
 def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -298,9 +326,9 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate
     N, K2 = w.shape
     if K != K2 or tuple(out.shape) != (T, N):
         raise InvalidArgument(f"matmul: input {list(x.shape)}, weight {list(w.shape)}, output {list(out.shape)}")
-    _check(_lib("gemm_generic").tie_gemm_generic(
+    _call(_lib("gemm_generic").tie_gemm_generic, "gemm_generic",
         x.data_ptr(), _code(x, "matmul input"), w.data_ptr(), _code(w, "matmul weight"), out.data_ptr(),
-        _code(out, "matmul output"), int(accumulate), T, N, K, _stream()), "gemm_generic")
+        _code(out, "matmul output"), int(accumulate), T, N, K, _stream())
 
 
 class PackedWeight:
@@ -395,9 +423,9 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
         raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows, got {M}")
     if gated and accumulate:
         raise InvalidArgument("a gated product does not accumulate")
-    _check(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16(
+    _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16, "skinny_gemm_bf16",
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
-        int(splits), int(isinstance(w, PackedWeight)), _stream()), "skinny_gemm_bf16")
+        int(splits), int(isinstance(w, PackedWeight)), _stream())
 
 
 def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
@@ -427,10 +455,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         M, N, K = _bf16_product_operands(x, w, out, gated, "gemm_bf16")
     if accumulate and (gated or out.dtype != torch.float32):
         raise InvalidArgument("gemm_bf16 accumulates into float32 outputs only, and not in a gated product")
-    _check(_lib("gemm_bf16").tie_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
+    _call(_lib("gemm_bf16").tie_gemm_bf16, "gemm_bf16", x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"),
                                            int(accumulate), int(gated), M, N, K, tile, int(splits),
-                                           int(isinstance(w, PackedWeight)), _stream()),
-           "gemm_bf16")
+                                           int(isinstance(w, PackedWeight)), _stream())
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -491,8 +518,8 @@ def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tens
     _i32(positions, "positions", T)
     _f32(inv_freq, "inv_freq", (half,))
     _f32(out, "rope angles", (T, 2 * half))
-    _check(_lib("elementwise").tie_rope_angles(positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), T, half,
-                                               _stream()), "rope_angles")
+    _call(_lib("elementwise").tie_rope_angles, "rope_angles", positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), T, half,
+                                               _stream())
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
@@ -561,13 +588,13 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _gpu(v_cache, "v cache")
         _check_cache(k_cache, v_cache, KVH, block_size, Dh)
         cache_code = _code(k_cache, "k cache")
-    _check(_lib("elementwise").tie_qk_norm_rope_kv_write(
+    _call(_lib("elementwise").tie_qk_norm_rope_kv_write, "qk_norm_rope_kv_write",
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
         _ptr(k_weight), float(eps), _ptr(inv_freq), _ptr(angles), positions.data_ptr(),
         _ptr(slots) if write_kv else None,
         _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None, cache_code, int(write_kv),
         _ptr(k_dense), T, H, KVH, Dh, block_size, in_row, q_out.stride(0), k_row, int(plane_stride), int(planes),
-        rotary_dim, int(pairing == "interleaved"), _stream()), "qk_norm_rope_kv_write")
+        rotary_dim, int(pairing == "interleaved"), _stream())
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -598,11 +625,11 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _i32(block_tables, "block tables")
     if block_tables.dim() != 2 or block_tables.shape[0] < S:
         raise InvalidArgument(f"block tables {list(block_tables.shape)} do not cover {S} sequences")
-    _check(_lib("attention_generic").tie_paged_attention_generic(
+    _call(_lib("attention_generic").tie_paged_attention_generic, "paged_attention_generic",
         q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache, "k cache"),
         out.data_ptr(), _code(out, "attention output"), query_start.data_ptr(), context_lens.data_ptr(),
         block_tables.data_ptr(), seq_of_row.data_ptr(), T, H, KVH, Dh, bs, block_tables.shape[1], float(scale),
-        int(window or 0), _stream()), "paged_attention_generic")
+        int(window or 0), _stream())
 
 
 _argmax_workspace = {}
@@ -621,8 +648,8 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor, max_out: Optional[torch
         rows = max(R, 64)
         ws = _argmax_workspace[key] = (torch.empty(rows * 64, dtype=torch.float32, device=logits.device),
                                        torch.empty(rows * 64, dtype=torch.int32, device=logits.device))
-    _check(_lib("elementwise").tie_argmax(logits.data_ptr(), out.data_ptr(), _ptr(max_out), ws[0].data_ptr(),
-                                          ws[1].data_ptr(), R, V, _stream()), "argmax")
+    _call(_lib("elementwise").tie_argmax, "argmax", logits.data_ptr(), out.data_ptr(), _ptr(max_out), ws[0].data_ptr(),
+                                          ws[1].data_ptr(), R, V, _stream())
 
 
 ARGMAX_STATIC_MAX_ROWS = 1024     # TIE_ARGMAX_STATIC_MAX_ROWS of csrc/argmax_static.h
@@ -643,8 +670,8 @@ def argmax_rows_static(logits: torch.Tensor, out: torch.Tensor, max_out: Optiona
         raise InvalidArgument(f"argmax_rows_static takes at most {ARGMAX_STATIC_MAX_ROWS} rows (the size of its static "
                               f"scratch array), got {R}")
     with torch.cuda.device(logits.device):
-        _check(_lib("elementwise").tie_argmax_static(logits.data_ptr(), out.data_ptr(), _ptr(max_out), R, V,
-                                                     _stream()), "argmax_static")
+        _call(_lib("elementwise").tie_argmax_static, "argmax_static", logits.data_ptr(), out.data_ptr(), _ptr(max_out), R, V,
+                                                     _stream())
 
 
 def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
@@ -657,8 +684,8 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
     if uniform.dtype != torch.float64 or uniform.numel() != R:
         raise InvalidArgument("uniform numbers must be float64, one per row")
     _i32(out, "sample output", R)
-    _check(_lib("elementwise").tie_sample(logits.data_ptr(), inv_temperature.data_ptr(), uniform.data_ptr(),
-                                          out.data_ptr(), R, V, _stream()), "sample")
+    _call(_lib("elementwise").tie_sample, "sample", logits.data_ptr(), inv_temperature.data_ptr(), uniform.data_ptr(),
+                                          out.data_ptr(), R, V, _stream())
 
 
 # Up to this many workgroups of single decoded rows run in the prefill attention kernel beside a step's prompt
@@ -733,10 +760,10 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         if part_o.numel() < num_seqs * H * nsplit * Dh or part_ml.numel() < num_seqs * H * nsplit * 2:
             raise InvalidArgument("the buffers for the splits are too small")
     lib = _lib("attention_decode_bf16", Dh)
-    _check(lib.tie_attention_decode_bf16(
+    _call(lib.tie_attention_decode_bf16, "attention_decode_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), nsplit, _stream()), "attention_decode_bf16")
+        block_tables.shape[1], float(scale), int(window or 0), nsplit, _stream())
 
 
 def prefill_items(new_tokens, group_size: int) -> "list":
@@ -799,11 +826,11 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         if part_o.numel() < rows * H * nsplit * Dh or part_ml.numel() < rows * H * nsplit * 2 or not 0 < num_merge <= 65535:
             raise InvalidArgument("the buffers for the splits are too small, or no (or too many) rows to merge")
     lib = _lib("attention_prefill_bf16", Dh)
-    _check(lib.tie_attention_prefill_bf16(
+    _call(lib.tie_attention_prefill_bf16, "attention_prefill_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
         block_tables.shape[1], float(scale), int(window or 0), int(nsplit), _ptr(part_o), _ptr(part_ml),
-        _ptr(merge_rows), num_merge, _stream()), "attention_prefill_bf16")
+        _ptr(merge_rows), num_merge, _stream())
 
 
 def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:

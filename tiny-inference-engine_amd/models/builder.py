@@ -16,12 +16,51 @@ import torch
 from ..cache.spec import CachePlan, plan_cache
 from ..config.registry import resolve_architecture
 from ..errors import InvalidArgument
+from .. import kernels
 from ..parts import base as parts_base
-from ..parts.base import StepContext, TensorSpec, build_part
+from ..parts.base import Part, StepContext, TensorSpec, build_part
 from ..weights.binder import BFLOAT16, check_tensors, normalize_mode, place_tensor
 from ..weights.loader import ModelFiles, load_model_folder
 from ..weights.safetensors_io import StoredTensor
 from .spec import ModelSpec
+
+
+def _walk_parts(obj, tensors, classes, seen) -> None:
+    """The device tensors ``(address, bytes, shape, dtype)`` and the part classes of an object tree, in a fixed order."""
+    if isinstance(obj, torch.Tensor):
+        if obj.is_cuda:
+            tensors.append((obj.data_ptr(), obj.numel() * obj.element_size(), tuple(obj.shape), obj.dtype))
+    elif isinstance(obj, kernels.PackedWeight):
+        blocks = obj.blocks
+        tensors.append((blocks.data_ptr(), blocks.numel() * blocks.element_size(), tuple(obj.shape), "packed"))
+    elif isinstance(obj, Part):
+        if id(obj) in seen:
+            return
+        seen.add(id(obj))
+        classes.append(type(obj))
+        for name in sorted(vars(obj)):
+            _walk_parts(getattr(obj, name), tensors, classes, seen)
+    elif isinstance(obj, (list, tuple)):
+        for value in obj:
+            _walk_parts(value, tensors, classes, seen)
+    elif isinstance(obj, dict):
+        for name in sorted(obj, key=str):
+            _walk_parts(obj[name], tensors, classes, seen)
+    elif type(obj).__module__.startswith(__name__.split(".")[0] + ".") and hasattr(obj, "__dict__"):
+        if id(obj) in seen:          # a helper object of this package that a part holds (a Linear with its weight)
+            return
+        seen.add(id(obj))
+        for name in sorted(vars(obj)):
+            _walk_parts(getattr(obj, name), tensors, classes, seen)
+
+
+class _Launch:
+    """One noted kernel launch of a layer and where another layer's pointers go into its arguments."""
+
+    __slots__ = ("fn", "what", "args", "patches")
+
+    def __init__(self, fn, what, args, patches):
+        self.fn, self.what, self.args, self.patches = fn, what, args, patches    # patches: (argument, tensor, offset)
 
 
 class LayerParts:
@@ -52,6 +91,12 @@ class Model:
         self.mode: Optional[str] = None
         self.device = None
         self.layer_hook: Optional[Callable[[int, torch.Tensor], None]] = None
+        # Entries of the run order whose layers have the same shape launch the same kernels with the same numbers
+        # and differ only in the addresses of their weights and caches: see _run_alike.
+        self.replay_layers = True
+        self.layers_replayed = 0                      # entries of the run order run from another's launch list
+        self._alike: Dict[int, int] = {}              # first entry of a run of layers alike -> one past its last
+        self._layer_tensors: Dict[int, list] = {}     # entry -> (address, bytes) of its layer's device tensors
 
     # --------------------------------------------------------------- tensors
     def _all_parts(self):
@@ -84,6 +129,7 @@ class Model:
             part.load_all(fetch, mode, device)
         self.mode = mode
         self.device = device
+        self._find_layers_alike()
         wide = sorted(name for (name, role), t in placed.items() if role == "matrix" and t.dtype == torch.float32)
         if mode == BFLOAT16 and wide:
             # Stored in 32 bits (or F16, widened): kept so, and every product over them runs on the float32
@@ -97,17 +143,142 @@ class Model:
         """Whether every part allows its launches to be recorded and replayed (see ``Part.capturable``)."""
         return all(part.all_capturable() for part in self._all_parts())
 
+    # ---------------------------------------------------------- layers alike
+    MIN_ALIKE = 4     # the first runs as it is, two are noted and compared, the rest replayed: fewer gain nothing
+
+    def _find_layers_alike(self) -> None:
+        """Finds runs of consecutive entries of the run order whose layers are of one shape.
+
+        Alike: the same part classes, every one of them ``replayable``, device tensors of the same shapes and
+        dtypes in the same places, the same kind of cache binding; each entry a layer of its own.
+        """
+        self._alike, self._layer_tensors = {}, {}
+        signatures = []
+        for index, call in enumerate(self.spec.order):
+            tensors, classes = [], []
+            _walk_parts(self.layers[call.layer].parts(), tensors, classes, set())
+            self._layer_tensors[index] = [(address, size) for address, size, _, _ in tensors]
+            entry = self.cache_plan.calls[index]
+            binding = None if entry is None else (entry.group, entry.writes)
+            ok = all(getattr(c, "replayable", False) for c in classes)
+            signatures.append((tuple(classes), tuple(t[2:] for t in tensors), binding) if ok else None)
+        start = 0
+        while start < len(signatures):
+            end = start + 1
+            if signatures[start] is not None:
+                layers = {self.spec.order[start].layer}
+                while (end < len(signatures) and signatures[end] == signatures[start]
+                       and self.spec.order[end].layer not in layers):
+                    layers.add(self.spec.order[end].layer)
+                    end += 1
+            # A tensor is every layer's own or shared by all of them (a table built once): two of the layers
+            # sharing one would pass for "the same argument" when their launches are compared.
+            for slot in range(len(self._layer_tensors[start])):
+                addresses = {self._layer_tensors[i][slot][0] for i in range(start, end)}
+                if len(addresses) not in (1, end - start):
+                    end = start + 1
+                    break
+            if end - start >= self.MIN_ALIKE:
+                self._alike[start] = end
+            start = end
+
+    def _entry_tensors(self, ctx: StepContext, index: int, cache) -> list:
+        """(address, bytes) of everything entry ``index`` owns on the device: its layer's tensors and its cache."""
+        tensors = list(self._layer_tensors[index])
+        for name in ("k_cache", "v_cache", "state"):
+            t = getattr(cache, name, None)
+            if isinstance(t, torch.Tensor):
+                tensors.append((t.data_ptr(), t.numel() * t.element_size()))
+        return tensors
+
+    @staticmethod
+    def _launch_list(noted_a, noted_b, tensors_a, tensors_b) -> Optional[List[_Launch]]:
+        """The launches of one layer as a list another layer of the same shape can run, or None.
+
+        Two layers' noted launches must be the same functions with the same arguments, except where an
+        argument is an address inside the same tensor of either layer (a weight, a cache plane) at the same
+        offset; anything else that differs means the layers are not alike after all.
+        """
+        if len(noted_a) != len(noted_b) or not noted_a:
+            return None
+        launches = []
+        for (fn_a, args_a, what), (fn_b, args_b, _) in zip(noted_a, noted_b):
+            if fn_a is not fn_b or len(args_a) != len(args_b):
+                return None
+            patches = []
+            for position, (a, b) in enumerate(zip(args_a, args_b)):
+                if a == b and type(a) is type(b):
+                    continue
+                if type(a) is not int or type(b) is not int:
+                    return None
+                for slot, ((base_a, size_a), (base_b, size_b)) in enumerate(zip(tensors_a, tensors_b)):
+                    if 0 <= a - base_a < size_a and a - base_a == b - base_b and size_a == size_b:
+                        patches.append((position, slot, a - base_a))
+                        break
+                else:
+                    return None
+            launches.append(_Launch(fn_a, what, args_a, tuple(patches)))
+        return launches
+
+    def _run_alike(self, ctx: StepContext, x: torch.Tensor, start: int, end: int) -> None:
+        """Runs entries ``start`` to ``end`` of the run order, layers of one shape.
+
+        What a layer launches depends on the step (rows, splits, work lists) but not on which of these layers it
+        is: only the addresses of its weights and cache differ. So the parts' own code runs for the first three
+        (the first may differ: it settles what the entry before it left), the launches of the second and third
+        are noted and compared, and the others run from that list with their own addresses, which takes a
+        fraction of the host time; small models' steps of many short kernels wait for the host otherwise.
+        """
+        def run(index):
+            cache = ctx.cache_of(index)
+            layer = self.layers[self.spec.order[index].layer]
+            layer.block.forward(ctx, x, layer, cache)
+            return cache
+
+        run(start)
+        noted, tensors = [], []
+        for index in (start + 1, start + 2):
+            record = kernels.start_recording()
+            try:
+                cache = run(index)
+            finally:
+                kernels.stop_recording()
+            noted.append(record)
+            tensors.append(self._entry_tensors(ctx, index, cache))
+        launches = self._launch_list(noted[0], noted[1], tensors[0], tensors[1])
+        for index in range(start + 3, end):
+            if launches is None:
+                run(index)
+                continue
+            own = self._entry_tensors(ctx, index, ctx.cache_of(index))
+            for launch in launches:
+                if launch.patches:
+                    args = list(launch.args)
+                    for position, slot, offset in launch.patches:
+                        args[position] = own[slot][0] + offset
+                    kernels.replay_call(launch.fn, launch.what, args)
+                else:
+                    kernels.replay_call(launch.fn, launch.what, launch.args)
+            self.layers_replayed += 1
+
     # ------------------------------------------------------------------ step
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """Runs the tokens of ``ctx.batch``; returns float32 logits ``[R, vocab]`` or None if none are wanted."""
         batch = ctx.batch
         x = self.embedding.forward(ctx, batch.tokens)
-        for index, call in enumerate(self.spec.order):
-            layer = self.layers[call.layer]
+        index, entries = 0, len(self.spec.order)
+        while index < entries:
+            alike_to = self._alike.get(index) if self.replay_layers and self.layer_hook is None else None
+            if alike_to is not None:
+                self._run_alike(ctx, x, index, alike_to)
+                index = alike_to
+                continue
+            layer = self.layers[self.spec.order[index].layer]
             layer.block.forward(ctx, x, layer, ctx.cache_of(index))
             if self.layer_hook is not None:
                 ctx.settle()
                 self.layer_hook(index, x)
+            index += 1
         ctx.settle()     # the last layer's product may still be owed to the stream
         if batch.num_logit_rows == 0:
             return None

@@ -28,6 +28,8 @@ from .linear import Linear
 
 @register_part("mixer", "paged_attention")
 class PagedAttention(Mixer):
+    replayable = True
+
     def __init__(self, params):
         super().__init__(params)
         self.hidden = int(params["hidden"])

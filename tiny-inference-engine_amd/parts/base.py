@@ -88,6 +88,11 @@ class Part:
     """
 
     capturable = True
+    # True: in a step, what the part launches is the same for every layer of the same shape except for the
+    # addresses of the layer's own tensors and cache (no host-side work per layer beyond kernel launches, no
+    # torch operations, nothing that depends on which layer it is). The model then runs such layers from the
+    # launch list of one of them (``Model._run_alike``). Parts defined elsewhere keep the default.
+    replayable = False
 
     def __init__(self, params: Mapping[str, Any]):
         self.params = dict(params)

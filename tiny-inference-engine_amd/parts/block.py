@@ -16,6 +16,7 @@ from .base import Block, StepContext, register_part
 
 @register_part("block", "pre_norm")
 class PreNormBlock(Block):
+    replayable = True
     NORMS = ("pre_mixer", "pre_feed_forward")
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:

@@ -21,6 +21,8 @@ from .linear import Linear
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
+    replayable = True
+
     def __init__(self, params):
         super().__init__(params)
         self.hidden = int(params["hidden"])

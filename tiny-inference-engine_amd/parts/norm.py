@@ -18,6 +18,7 @@ from .base import Norm, StepContext, TensorSpec, register_part
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
+    replayable = True
     adds_owed = True
 
     def __init__(self, params):

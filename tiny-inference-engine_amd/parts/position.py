@@ -19,6 +19,8 @@ from .base import Position, register_part
 
 @register_part("position", "rope_neox")
 class RopeNeox(Position):
+    replayable = True
+
     def __init__(self, params):
         super().__init__(params)
         self.head_dim = int(params["head_dim"])
@@ -55,6 +57,8 @@ class RopeNeox(Position):
 @register_part("position", "none")
 class NoPosition(Position):
     """No position encoding: queries and keys are left as they are."""
+
+    replayable = True
 
     def rotary_table(self):
         return None, 0, "none"
