@@ -345,6 +345,12 @@ def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
         out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device="cuda")
         kernels.skinny_gemm_bf16(x, packed, out, gated=True)
         close(out, want, 1e-2, f"gated skinny gemm {M}x{N}x{K}")
+        lib = kernels._lib("skinny_gemm_bf16")
+        for rt, u in ((0, -1), (3, 1), (6, 1), (8, 1)):      # from memory; through LDS in the three workgroup shapes
+            again = torch.full_like(out, float("nan"))
+            assert lib.tie_skinny_gemm_bf16_with(x.data_ptr(), packed.data_ptr(), again.data_ptr(), 1, 0, 1, M, N, K, 1, 1,
+                                                 rt, u, kernels._stream()) == 0
+            assert torch.equal(again, out), f"gated, tiles {rt}, batch {u}: the sums depend on the launch's shape"
         return
     want = plain.linear(x.cpu(), w.cpu())
     splits = kernels.skinny_splits(N, K)
@@ -357,8 +363,9 @@ def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
     alone = torch.empty(splits, 1, N, dtype=torch.float32, device="cuda")
     kernels.skinny_gemm_bf16(x[M - 1:M].contiguous(), packed, alone, splits=splits)
     assert torch.equal(alone[:, 0], planes[:, M - 1])
-    # u = -1: x read from memory whatever M and N; u = 1: x through LDS whatever N (for more than 16 rows)
-    for rt, u in ((1, 8), (1, 2), (2, 4), (3, 2), (4, 2), (2, 8), (0, -1), (0, 1), (1, 1), (2, 1)):
+    # u = -1: x read from memory whatever M and N; u = 1: x through LDS whatever N (for more than 16 rows),
+    # in workgroups of rt tiles (3, 6 or 8)
+    for rt, u in ((1, 8), (1, 2), (2, 4), (3, 2), (4, 2), (2, 8), (0, -1), (0, 1), (3, 1), (6, 1), (8, 1)):
         again = torch.full_like(planes, float("nan"))
         status = lib.tie_skinny_gemm_bf16_with(x.data_ptr(), packed.data_ptr(), again.data_ptr(), 0, 0, 0, M, N, K, splits, 1,
                                                rt, u, kernels._stream())

@@ -189,26 +189,38 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
 
 // ------------------------------------------------------------------ 17 to 64 rows: x through LDS
 // With more than one 16-row tile of x the kernel above spends most of its load instructions on x: every
-// weight block of 1 KB needs MT blocks of x, read as 16 rows' 64-byte pieces. Here the four waves of a
-// workgroup walk the SAME range of K, each over its own RT weight tiles, and share x: a batch of U k-blocks
-// of all rows is brought in by the whole workgroup with full-line loads, laid into LDS in the order the
-// matrix core takes its A operand (block (u, mt): lane l's 16 bytes at byte 16 l), and read from there by
-// all four waves. Weights still go from memory straight into registers, non-temporally, one batch ahead.
+// weight block of 1 KB needs MT blocks of x, and a compute unit serves a load instruction of a wave in about 65
+// cycles whether it comes from HBM or from L2, so at 64 rows (7 loads for 3 KB of weights) the weights stream
+// at 3.6 TB/s. Here the WAVES waves of a workgroup walk the SAME range of K, each over its own RT weight
+// tiles, and share x: a chunk of XU k-blocks of all rows goes from global memory straight into LDS (buffer
+// loads with the lds flag; one instruction brings one 16-row block of 32 k, lane l's 16 bytes - row l % 16,
+// k-chunk l / 16 - to byte 16 l, which is the order the matrix core takes its A operand), one chunk ahead
+// of the arithmetic, and all waves read their fragments from there. Weights still go from memory straight
+// into registers, non-temporally, one chunk ahead. x then costs MT / (WAVES x RT) of the weights' load
+// instructions; the price is a barrier a chunk, so only long, wide products gain (rows_kernel_tiles below).
 //
 // The sums are the very ones of the kernel above: a plane's range of K is walked in the same four parts
 // of per_wave k-blocks, each summed by the matrix core in k order, and the parts are added in their order
 // (there: by the reduction through LDS; here: by folding the accumulator into a running total at each
 // part's end). A row's result therefore does not depend on which of the two kernels its batch size picks.
-template <int MT, int RT, int U, typename TO>
-__global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16_t* __restrict__ x,
-                                                                         const bf16_t* __restrict__ w,
-                                                                         TO* __restrict__ out, int M, int N, int K,
-                                                                         int accumulate, int gated, int per_wave) {
+typedef __attribute__((address_space(3))) void sk_lds_void_t;
+#define SK_XU 8
+// Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
+// selects x, y, z, w; no swizzle, no stride.
+#define SK_RSRC_FLAGS 0x27000
+
+template <int MT, int RT, int WAVES, typename TO>
+__global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16_t* __restrict__ x,
+                                                                      const bf16_t* __restrict__ w,
+                                                                      TO* __restrict__ out, int M, int N, int K,
+                                                                      int accumulate, int gated, int per_wave) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int U = SK_XU;
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][U][MT][512];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
-  const int wave = threadIdx.x / TIE_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TIE_WAVE);
   const int tiles = N / 16;
-  const int tile0 = (static_cast<int>(blockIdx.x) * SK_WAVES + wave) * RT;
+  const int tile0 = (static_cast<int>(blockIdx.x) * WAVES + wave) * RT;
   const int split = blockIdx.y;
   const int kblocks = K / 32;
   const int kb_lo = min(kblocks, split * SK_WAVES * per_wave);
@@ -218,29 +230,20 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const b
 #pragma unroll
   for (int t = 0; t < RT; ++t) wp[t] = w + static_cast<size_t>(min(tile0 + t, tiles - 1)) * kblocks * 512 + lane * 8;
 
-  // Staging: a batch is MT * 16 rows of U * 32 elements = MT * 64 * U pieces of 16 bytes, CH of them a thread;
-  // consecutive threads take consecutive pieces of a row, so a row's U * 64 bytes are read as whole lines.
-  constexpr int CH = MT * U / 4;
-  static_assert(MT * U % 4 == 0, "a batch must give every thread whole pieces");
-  sk_u32x4_t stage[CH];
-  auto fetch_rows = [&](int kb0) {
+  // x as a buffer: rows beyond M lie beyond its end and read as zeros.
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(x), 0, static_cast<int>(static_cast<size_t>(M) * K * 2), SK_RSRC_FLAGS);
+  const unsigned lane_off = (static_cast<unsigned>(lane & 15) * K + (lane >> 4) * 8) * 2;   // bytes, within a 16-row block
+  const unsigned tile_rows = 16u * K * 2;
+  // Blocks (u, mt) of a chunk are dealt to the waves in turn.
+  auto fetch_rows = [&](int kb0, int buf) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int piece = c * (SK_WAVES * TIE_WAVE) + threadIdx.x;
-      const int row = piece / (4 * U), col = piece % (4 * U);          // col: 8-element piece of the batch's k range
-      const int kb = kb0 + col / 4;
-      stage[c] = (row < M && kb < kb_hi)
-                     ? *reinterpret_cast<const sk_u32x4_t*>(x + static_cast<size_t>(row) * K + kb * 32 + (col % 4) * 8)
-                     : sk_u32x4_t{0, 0, 0, 0};
-    }
-  };
-  auto store_rows = [&](int buf) {
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int piece = c * (SK_WAVES * TIE_WAVE) + threadIdx.x;
-      const int row = piece / (4 * U), col = piece % (4 * U);
-      // element (row, k): tile row / 16, lane (k % 32 / 8) * 16 + row % 16 of block (u = col / 4, mt)
-      *reinterpret_cast<sk_u32x4_t*>(&xs[buf][col / 4][row / 16][((col % 4) * 16 + (row % 16)) * 8]) = stage[c];
+    for (int i = 0; i < (U * MT + WAVES - 1) / WAVES; ++i) {
+      const int b = i * WAVES + wave;
+      const int u = b / MT, mt = b % MT;
+      if (b < U * MT && kb0 + u < kb_hi)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (sk_lds_void_t*)(&xs[buf][u][mt][0]), 16,
+                                                 lane_off + mt * tile_rows, (kb0 + u) * 64, 0, 0);
     }
   };
   bf16x8_t b[RT][U], nb[RT][U];
@@ -273,15 +276,14 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const b
   };
 
   if (kb_lo < kb_hi) {
-    fetch_rows(kb_lo);
+    fetch_rows(kb_lo, 0);
     fetch_weights(b, kb_lo);
-    store_rows(0);
-    __syncthreads();
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     int buf = 0;
     for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += U) {
       const bool more = kb0 + U < kb_hi;
       if (more) {
-        fetch_rows(kb0 + U);
+        fetch_rows(kb0 + U, buf ^ 1);          // everyone's reads of that buffer ended before the last barrier
         fetch_weights(nb, kb0 + U);
       }
 #pragma unroll
@@ -299,13 +301,14 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const b
         }
       }
       if (more) {
-        store_rows(buf ^ 1);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
           for (int t = 0; t < RT; ++t) b[t][u] = nb[t][u];
       }
-      __syncthreads();
+      // The next chunk of x (and of the weights: they were asked for after it) has landed; after the barrier
+      // it may be read, and this chunk's buffer written again.
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       buf ^= 1;
     }
   }
@@ -335,6 +338,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_rows_kernel(const b
         store_from_float(o, sum);
       }
   }
+#endif
 }
 
 static int compute_units() {
@@ -370,6 +374,18 @@ static int choose_rt(int M, int N, int splits) {
   return best;
 }
 
+// Weight tiles a workgroup of the kernel that shares x through LDS takes (8: four waves x two tiles, 6: three
+// waves x two), or 0 where the kernel that reads x from memory is as fast or faster. Measured on the
+// projections of the 1.7B, 8B and 32B shapes: very wide weights (the lm_head, a gate/up of 51200 rows) gain 10
+// to 20 % from 17 rows on (5 % with K = 2048, in the smaller workgroups, and only up to 32 rows); a gate/up of 24576 x 4096 gains 11 % at 64 rows and nothing below 48; narrow
+// weights cut along K (O, down, QKV) and short K (2048) lose up to 40 %, their workgroups being too short
+// to pay for the extra barrier a chunk.
+static int rows_kernel_tiles(int M, int N, int K, int gated) {
+  if (N >= 32768) return K >= 4096 ? 8 : (M <= 32 ? 6 : 0);
+  if (gated && M > 48 && N >= 16384 && K >= 4096) return 6;
+  return 0;
+}
+
 // Ranges of K that a product over w[N, K] is cut into when its caller takes partial sums: weights with
 // few rows would otherwise give too few workgroups to keep enough bytes in flight. The smallest power of
 // two that makes about four workgroups a compute unit (1024), as long as a wave keeps four k-blocks and
@@ -395,40 +411,44 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int forced_rt = rt;
   const bool rows_kernel = u >= 0;          // u < 0: the kernel that reads x from memory, whatever M (tests compare the two)
-  const int forced_u = u;
+  const bool rows_forced = u == 1;          // u = 1: the kernel that shares x through LDS, whatever the shape
   if (u < 0) u = u == -1 ? 0 : -u;
   if (u == 1) u = 0;
-  if (rt == 0) rt = choose_rt(M, N, splits);
-  if (rt < 1 || rt > 4) return TIE_BAD_ARGUMENT;
-  const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
   const int kblocks = (K + 31) / 32;
   const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
-  if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
-  if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
-  // x through LDS pays where the weight has very many rows (the feed-forward of the largest shapes, the
-  // head): measured 20 to 25 % faster from 51200 rows on, slower or equal up to 24576, where too few waves
-  // are left to keep enough bytes in flight. u = 1 asks for it whatever N (tests).
+  // x through LDS (17 to 64 rows over packed weights, x within 32-bit byte offsets). With u = 1, rt is the
+  // number of tiles a workgroup takes: up to 3 three waves x one tile, up to 6 three waves x two, else four x two.
   const int tiles = (N + 15) / 16;
-  if (packed && mt > 1 && rows_kernel && (tiles >= 2048 || forced_u == 1)) {
-    const int rrt = (forced_rt == 0) ? (M <= 32 ? 2 : 1) : (forced_rt > 2 ? 2 : forced_rt);
-    const dim3 rgrid((tiles + SK_WAVES * rrt - 1) / (SK_WAVES * rrt), splits);
-#define LAUNCH_ROWS(MT, RT, U, TO)                                                                              \
-  skinny_rows_kernel<MT, RT, U, TO><<<rgrid, SK_WAVES * TIE_WAVE, 0, stream>>>(                                   \
+  const bool rows_fit = static_cast<size_t>(M) * K * 2 < (1ull << 31);
+  const int by_rule = rows_kernel_tiles(M, N, K, gated);
+  if (packed && mt > 1 && rows_kernel && rows_fit && (by_rule != 0 || rows_forced)) {
+    const int asked = rows_forced && forced_rt != 0 ? forced_rt : (by_rule != 0 ? by_rule : 6);
+    const int per_wg = asked <= 3 ? 3 : (asked <= 6 ? 6 : 8);
+    const dim3 rgrid((tiles + per_wg - 1) / per_wg, splits);
+#define LAUNCH_ROWS(MT, RT, WAVES, TO)                                                                          \
+  skinny_rows_kernel<MT, RT, WAVES, TO><<<rgrid, WAVES * TIE_WAVE, 0, stream>>>(                                  \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
       gated, per_wave)
-#define LAUNCH_ROWS_TO(MT, RT, U)                                 \
-  if (out_dtype == TIE_F32) LAUNCH_ROWS(MT, RT, U, float);       \
-  else if (out_dtype == TIE_BF16) LAUNCH_ROWS(MT, RT, U, bf16_t); \
+#define LAUNCH_ROWS_TO(MT, RT, WAVES)                                 \
+  if (out_dtype == TIE_F32) LAUNCH_ROWS(MT, RT, WAVES, float);       \
+  else if (out_dtype == TIE_BF16) LAUNCH_ROWS(MT, RT, WAVES, bf16_t); \
   else return TIE_BAD_ARGUMENT
-    if (mt == 2) {
-      if (rrt == 1) { LAUNCH_ROWS_TO(2, 1, 8); } else { LAUNCH_ROWS_TO(2, 2, 4); }
-    } else {
-      if (rrt == 1) { LAUNCH_ROWS_TO(4, 1, 8); } else { LAUNCH_ROWS_TO(4, 2, 4); }
-    }
+#define LAUNCH_ROWS_MT(MT)                                  \
+  if (per_wg == 8) { LAUNCH_ROWS_TO(MT, 2, 4); }            \
+  else if (per_wg == 6) { LAUNCH_ROWS_TO(MT, 2, 3); }       \
+  else { LAUNCH_ROWS_TO(MT, 1, 3); }
+    if (mt == 2) { LAUNCH_ROWS_MT(2) } else { LAUNCH_ROWS_MT(4) }
+#undef LAUNCH_ROWS_MT
 #undef LAUNCH_ROWS_TO
 #undef LAUNCH_ROWS
     return tie_launch_status();
   }
+  if (rows_forced) rt = 0;                  // asked for the other kernel, which does not take this shape: by the rule
+  if (rt == 0) rt = choose_rt(M, N, splits);
+  if (rt < 1 || rt > 4) return TIE_BAD_ARGUMENT;
+  const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
+  if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
+  if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
 #define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
   skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                             \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
