@@ -542,7 +542,7 @@ def test_gemm_bf16_in_planes(M, N, K, splits):
     close(planes.cpu().to(F64).sum(0), plain.linear(x.cpu(), w.cpu()), 1e-5, f"gemm {M}x{N}x{K} in {splits} planes")
 
 
-def run_decode(case, S, H, Dh, nsplit, window=None):
+def run_decode(case, S, H, Dh, nsplit, window=None, depth=0):
     from tie_amd import kernels
 
     q = case["q"]
@@ -550,8 +550,24 @@ def run_decode(case, S, H, Dh, nsplit, window=None):
     part_o = torch.empty(S * H * nsplit * Dh, dtype=torch.float32, device="cuda")
     part_ml = torch.empty(S * H * nsplit * 2, dtype=torch.float32, device="cuda")
     kernels.attention_decode_bf16(q, case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
-                                  case["tables"], S, H, Dh ** -0.5, window, nsplit, part_o, part_ml)
+                                  case["tables"], S, H, Dh ** -0.5, window, nsplit, part_o, part_ml, depth=depth)
     return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(6, 2, 32, 16), (5, 5, 80, 16), (8, 2, 128, 16), (2, 1, 256, 32), (4, 4, 112, 64)])
+@pytest.mark.parametrize("nsplit,window", [(1, None), (2, None), (5, None), (1, 100), (3, 77)])
+def test_attention_decode_bf16_with_tiles_in_flight(H, KVH, Dh, bs, nsplit, window):
+    """Pages of 16 positions or more: the kernels that keep two to four tiles of keys in registers against the
+    one that looks its pages up per lane and against the plain formula, at lengths around every count of tiles
+    that the ring's first, middle and last parts take (1 to 12 tiles a share), with and without a window."""
+    lens = [1, 31, 32, 33, 64, 65, 96, 127, 129, 160, 200, 257, 300, 321, 385, 700, 1000]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=[1] * len(lens), lens_ctx=lens, seed=17, dtype=torch.bfloat16,
+                             window=window)
+    first = run_decode(case, S, H, Dh, nsplit, window=window, depth=1)
+    close(first, case["want"], 1e-2, f"decode attention H={H} KVH={KVH} Dh={Dh} bs={bs} splits={nsplit} window={window}")
+    for depth in (2, 3, 4):
+        again = run_decode(case, S, H, Dh, nsplit, window=window, depth=depth)
+        assert torch.equal(again, first), f"{depth} tiles in flight: other bits than one"
 
 
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
@@ -648,7 +664,7 @@ def test_attention_decode_bf16_one_sequence_past_32k(H, KVH):
     from tie_amd import kernels
 
     Dh, ctx = 64, 40000
-    nsplit = kernels.decode_splits(1, KVH, 65536)
+    nsplit = kernels.decode_splits(1, KVH, 65536, 8)
     assert nsplit == kernels.MAX_KEY_SPLITS or KVH > 8
     case, S = long_decode_case(H, KVH, Dh, 16, [ctx], seed=33, spike_back=39000)
     out = run_decode(case, S, H, Dh, nsplit)

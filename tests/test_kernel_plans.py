@@ -17,11 +17,16 @@ def test_key_shares_never_exceed_what_the_merge_takes():
     for seqs in (1, 2, 3, 4, 7, 8, 64, 256):
         for kv_heads in (1, 2, 4, 8, 16):
             for context in contexts:
-                n = kernels.decode_splits(seqs, kv_heads, context)
-                assert 1 <= n <= kernels.MAX_KEY_SPLITS, (seqs, kv_heads, context, n)
+                for block_size in (4, 8, 16, 64):
+                    n = kernels.decode_splits(seqs, kv_heads, context, block_size)
+                    assert 1 <= n <= kernels.MAX_KEY_SPLITS, (seqs, kv_heads, context, block_size, n)
     # the cases that used to ask for more than the kernel takes
-    assert kernels.decode_splits(1, 4, 65536) == kernels.MAX_KEY_SPLITS
-    assert kernels.decode_splits(1, 2, 81920) == kernels.MAX_KEY_SPLITS
+    assert kernels.decode_splits(1, 4, 65536, 8) == kernels.MAX_KEY_SPLITS
+    assert kernels.decode_splits(1, 2, 81920, 8) == kernels.MAX_KEY_SPLITS
+    assert kernels.decode_splits(1, 1, 65536, 16) == kernels.MAX_KEY_SPLITS
+    # about 512 waves in shares of at least 128 keys where a wave keeps several tiles in flight
+    assert kernels.decode_splits(8, 8, 4096) == 8 and kernels.decode_splits(64, 8, 4096) == 1
+    assert kernels.decode_splits(1, 8, 4096) == 32 and kernels.decode_splits(1, 8, 200) == 1
     for items in (1, 2, 5, 40, 300):
         for kv_heads in (1, 2, 8):
             for group in (1, 3, 4, 8, 16):

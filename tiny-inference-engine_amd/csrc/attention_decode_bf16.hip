@@ -42,6 +42,85 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ bf16x8_t frag(u32x4_t v) { return *reinterpret_cast<const bf16x8_t*>(&v); }
 
+// One tile of 32 keys for the 16 columns of a wave: scores, online softmax in float32, values. kf: the keys'
+// fragments of the two 16-key sub-tiles, vf: the values' fragments, qf: the queries. Shared by the kernels
+// below, so that a position's result does not depend on which of them ran.
+__device__ __forceinline__ void attend_tile(const u32x4_t (&kf)[2][KSTEPS], const u32x4_t (&vf)[DTILES],
+                                            const u32x4_t (&qf)[KSTEPS], floatx4 (&acc)[DTILES], float& m, float& l,
+                                            int base, int start, int pos, int quad, float scale_log2e) {
+  // ---- first product: two 16-key sub-tiles
+  floatx4 sc[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    sc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st)
+      sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(kf[u][st]), frag(qf[st]), sc[u], 0, 0, 0);
+  }
+  // ---- softmax of this lane's column over its 8 keys (quad * 8 + u * 4 + v), then across the four quads.
+  // Scores stay unscaled; scale * log2(e) > 0 enters in the exponent: p = 2^(s c - m c).
+  float sv[8];
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int kp = base + quad * 8 + u * 4 + v;
+      const float x = (kp <= pos && kp >= start) ? sc[u][v] : -INFINITY;
+      sv[u * 4 + v] = x;
+      tile_max = fmaxf(tile_max, x);
+    }
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, TIE_WAVE));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, TIE_WAVE));
+  const float m_new = fmaxf(m, tile_max);
+  const float neg_mc = (m_new == -INFINITY) ? 0.f : -m_new * scale_log2e;
+  const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
+  u32x4_t pf;
+  float psum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const float p0 = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, neg_mc));       // masked: 0
+    const float p1 = __builtin_amdgcn_exp2f(fmaf(sv[i + 1], scale_log2e, neg_mc));
+    psum += p0;
+    psum += p1;
+    pf[i / 2] = pack_bf16x2(p0, p1);
+  }
+  l = l * corr + psum;
+  m = m_new;
+  // ---- second product
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[dt][v] *= corr;
+    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(vf[dt]), frag(pf), acc[dt], 0, 0, 0);
+  }
+}
+
+// What a wave leaves when its keys are done: the output row itself with one share, else its (maximum, sum,
+// accumulator) for the merge. h: the query head of this lane's column, z: the sequence's place in the launch.
+__device__ __forceinline__ void store_share(const floatx4 (&acc)[DTILES], float m, float l, bf16_t* __restrict__ out,
+                                            float* __restrict__ part_o, float* __restrict__ part_ml, int t, int z,
+                                            int h, int H, int quad, int nsplit, int split, float scale_log2e) {
+  if (nsplit == 1) {  // no merge needed: normalise and store
+    bf16_t* o = out + (static_cast<size_t>(t) * H + h) * DH;
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+      *reinterpret_cast<u32x2_t*>(o + dt * 16 + quad * 4) =
+          u32x2_t{pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv), pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv)};
+    return;
+  }
+  const size_t slot = (static_cast<size_t>(z) * H + h) * nsplit + split;
+  float* po = part_o + slot * DH;
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt)
+    *reinterpret_cast<float4*>(po + dt * 16 + quad * 4) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
+  if (quad == 0) {
+    part_ml[slot * 2] = m * scale_log2e;     // the merge works in the exponent's units (base 2)
+    part_ml[slot * 2 + 1] = l;
+  }
+}
+
 // Keys of a 32-key tile are taken in runs of 8: row r of 16-key sub-tile u is key (r / 4) * 8 + u * 4 + r % 4
 // of the tile. The scores a lane then holds (rows quad * 4 + v of both sub-tiles) are those of the 8
 // consecutive keys quad * 8 .. + 7, which is also how the values of one dimension lie in a page: with
@@ -164,78 +243,130 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
       load_values(base + 32, pages, vf_next);
       if (tile + 2 < tile_end) lookup(base + 64, pages);
     }
-    // ---- first product: two 16-key sub-tiles
-    floatx4 sc[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      sc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int st = 0; st < KSTEPS; ++st)
-        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(kf[u][st]), frag(qf[st]), sc[u], 0, 0, 0);
-    }
-    // ---- softmax of this lane's column over its 8 keys (quad * 8 + u * 4 + v), then across the four quads.
-    // Scores stay unscaled; scale * log2(e) > 0 enters in the exponent: p = 2^(s c - m c).
-    float sv[8];
-    float tile_max = -INFINITY;
-    const bool whole = base >= start && base + 31 <= pos;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int kp = base + quad * 8 + u * 4 + v;
-        const float x = (whole || (kp <= pos && kp >= start)) ? sc[u][v] : -INFINITY;
-        sv[u * 4 + v] = x;
-        tile_max = fmaxf(tile_max, x);
-      }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, TIE_WAVE));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, TIE_WAVE));
-    const float m_new = fmaxf(m, tile_max);
-    const float neg_mc = (m_new == -INFINITY) ? 0.f : -m_new * scale_log2e;
-    const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
-    u32x4_t pf;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; i += 2) {
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, neg_mc));       // masked: 0
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(sv[i + 1], scale_log2e, neg_mc));
-      psum += p0;
-      psum += p1;
-      pf[i / 2] = pack_bf16x2(p0, p1);
-    }
-    l = l * corr + psum;
-    m = m_new;
-    // ---- second product
-#pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt) {
-#pragma unroll
-      for (int v = 0; v < 4; ++v) acc[dt][v] *= corr;
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(vf[dt]), frag(pf), acc[dt], 0, 0, 0);
-    }
+    attend_tile(kf, vf, qf, acc, m, l, base, start, pos, quad, scale_log2e);
   }
 
   // The column's sum over all keys of this split.
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
-  const int h = kvh * G + col;
-  if (nsplit == 1) {  // no merge needed: normalise and store
-    bf16_t* o = out + (static_cast<size_t>(t) * H + h) * DH;
-    const float inv = 1.0f / l;
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e);
+}
+
+// The same for pages of 16 positions or more, with DEPTH - 1 tiles in flight behind the one that is computed.
+// The kernel above asks for a tile's data after it has waited for the lookup of its pages, and the counter of
+// outstanding vector loads runs in order: waiting for a lookup waits for every data load issued before it, so
+// a wave never has more than one tile (16 KB at head size 128) on its way and its time is one memory latency
+// a tile. Here a half tile of 16 positions lies in one page, so the two page numbers of a tile are the same
+// for all lanes and come by scalar loads, which have a counter of their own; the tiles live in a ring of
+// DEPTH register sets that is walked with constant indices, so no set is copied (a copy would wait for its
+// loads). The arithmetic of a tile and the order of the tiles are those of the kernel above: the same bits.
+template <int DEPTH>
+__global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ query_start, const int* __restrict__ context_lens,
+    const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
+    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit) {
+  const int lane = threadIdx.x;
+  const int col = lane & 15;
+  const int quad = lane >> 4;
+  const int split = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int s = seq_ids ? seq_ids[blockIdx.z] : blockIdx.z;
+  const int G = H / KVH;
+  const int t = query_start[s];
+  const int pos = context_lens[s] - 1;
+  const int start = window > 0 ? max(0, pos - window + 1) : 0;
+  const int* table = block_tables + static_cast<size_t>(s) * max_blocks;
+
+  const int first_tile = start / 32;
+  const int num_tiles = pos / 32 + 1;
+  const int per_split = (num_tiles - first_tile + nsplit - 1) / nsplit;
+  const int tile_begin = first_tile + split * per_split;
+  const int tile_end = min(num_tiles, tile_begin + per_split);
+
+  u32x4_t qf[KSTEPS];
+  {
+    const bool valid = col < G;
+    const bf16_t* qr = q + (static_cast<size_t>(t) * H + static_cast<size_t>(kvh) * G + (valid ? col : 0)) * DH;
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+      const int d = st * 32 + quad * 8;
+      qf[st] = (valid && d < DH) ? *reinterpret_cast<const u32x4_t*>(qr + d) : u32x4_t{0, 0, 0, 0};
+    }
+  }
+  floatx4 acc[DTILES];
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
+  const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
+  const int krow0 = (col >> 2) * 8 + (col & 3);
+  const bool keys_in_upper_half = krow0 >= 16;      // both sub-tiles' rows (krow0, krow0 + 4) lie in one half
+  const bool values_in_upper_half = quad >= 2;      // positions quad * 8 .. + 7
+  const int in_page = block_size - 1;
+  const size_t dim_off = static_cast<size_t>(col) * block_size;
+
+  struct Tile { u32x4_t k[2][KSTEPS]; u32x4_t v[DTILES]; };
+  // Positions are clamped into [start, pos] for addresses only; a clamped position stays in its half of 16.
+  auto issue = [&](int tile, Tile& tl) {
+    const int base = tile * 32;
+    const int page_lo = table[min(max(base, start), pos) >> block_shift];
+    const int page_hi = table[min(max(base + 16, start), pos) >> block_shift];
+    const bf16_t* kpage = k_cache + static_cast<size_t>(keys_in_upper_half ? page_hi : page_lo) * page_stride + head_off;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kp = min(max(base + krow0 + u * 4, start), pos);
+      const bf16_t* kr = kpage + static_cast<size_t>(kp & in_page) * DH;
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) {
+        // Every load is issued whatever the lane (a load under a lane's condition makes the count of loads
+        // in flight unknown to the compiler, which then waits for all of them): a head size that is no
+        // multiple of 32 reads its last step's upper pieces from the row's start and drops them.
+        const int d = st * 32 + quad * 8;
+        const bool inside = DH % 32 == 0 || d < DH;
+        const u32x4_t piece = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kr + (inside ? d : 0)));
+        tl.k[u][st] = inside ? piece : u32x4_t{0, 0, 0, 0};
+      }
+    }
+    const int vp = min(max(base + quad * 8, start / 8 * 8), pos / 8 * 8);
+    const bf16_t* vr = v_cache + static_cast<size_t>(values_in_upper_half ? page_hi : page_lo) * page_stride + head_off +
+                       (vp & in_page) + dim_off;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
-      *reinterpret_cast<u32x2_t*>(o + dt * 16 + quad * 4) =
-          u32x2_t{pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv), pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv)};
-    return;
-  }
-  const size_t slot = (static_cast<size_t>(blockIdx.z) * H + h) * nsplit + split;
-  float* po = part_o + slot * DH;
+      tl.v[dt] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vr + static_cast<size_t>(dt) * 16 * block_size));
+  };
+
+  // Tile i of the wave lives in set i % DEPTH. The groups of DEPTH tiles in the middle issue and compute
+  // without a condition, so the compiler knows how many loads are in flight and waits for the oldest tile
+  // only; the first DEPTH - 1 tiles before and the last 2 DEPTH - 2 at most after them are issued under
+  // conditions, where it waits for more than it must.
+  Tile ring[DEPTH];
 #pragma unroll
-  for (int dt = 0; dt < DTILES; ++dt)
-    *reinterpret_cast<float4*>(po + dt * 16 + quad * 4) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
-  if (quad == 0) {
-    part_ml[slot * 2] = m * scale_log2e;     // the merge works in the exponent's units (base 2)
-    part_ml[slot * 2 + 1] = l;
+  for (int j = 0; j < DEPTH - 1; ++j)
+    if (tile_begin + j < tile_end) issue(tile_begin + j, ring[j]);
+  int tile = tile_begin;
+  for (; tile + 2 * DEPTH - 2 < tile_end; tile += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+      issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
+      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, pos, quad, scale_log2e);
+    }
   }
+#pragma unroll
+  for (int j = 0; j < 2 * DEPTH - 2; ++j) {
+    if (tile + j < tile_end) {
+      if (j < DEPTH - 1 && tile + j + DEPTH - 1 < tile_end) issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
+      attend_tile(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, pos, quad, scale_log2e);
+    }
+  }
+
+  l += __shfl_xor(l, 16, TIE_WAVE);
+  l += __shfl_xor(l, 32, TIE_WAVE);
+  if (col >= G) return;
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e);
 }
 
 #include "attention_merge.h"
@@ -243,30 +374,49 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 extern "C" int tie_attention_decode_head_dim() { return DH; }
 extern "C" int tie_attention_max_splits() { return MERGE_MAX_SPLITS; }
 
-extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                         float* part_o, float* part_ml, const int* query_start,
-                                         const int* context_lens, const int* block_tables, const int* seq_ids,
-                                         int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
-                                         int window, int nsplit, hipStream_t stream) {
+// depth: 0 = by the rule, 1 = the kernel that looks its pages up per lane (any page size), 2 to 4 = the ring
+// kernel with that many register sets (pages of 16 positions or more); for tests and sweeps.
+extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              float* part_o, float* part_ml, const int* query_start,
+                                              const int* context_lens, const int* block_tables, const int* seq_ids,
+                                              int num_seqs, int H, int KVH, int block_size, int max_blocks,
+                                              float scale, int window, int nsplit, int depth, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
-      nsplit > MERGE_MAX_SPLITS ||
+      nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
       !(scale > 0.f))   // the running maximum is kept on unscaled scores
     return TIE_BAD_ARGUMENT;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr)) return TIE_BAD_ARGUMENT;
+  // Measured: the ring of three register sets where the keys are cut into shares, of four where a wave walks
+  // a whole sequence.
+  if (depth == 0) depth = block_size < 16 ? 1 : (nsplit == 1 ? 4 : 3);
   const dim3 grid(nsplit, KVH, num_seqs);
   const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
-#define LAUNCH(WIDE)                                                                                            \
-  attention_decode_kernel<WIDE><<<grid, TIE_WAVE, 0, stream>>>(                                                  \
+#define LAUNCH(KERNEL)                                                                                          \
+  KERNEL<<<grid, TIE_WAVE, 0, stream>>>(                                                                         \
       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),  \
       static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH,     \
       block_size, block_shift, max_blocks, scale_log2e, window, nsplit)
-  if (block_size % 8 == 0) LAUNCH(true); else LAUNCH(false);
+  if (depth == 4) LAUNCH(attention_decode_ring_kernel<4>);
+  else if (depth == 3) LAUNCH(attention_decode_ring_kernel<3>);
+  else if (depth == 2) LAUNCH(attention_decode_ring_kernel<2>);
+  else if (block_size % 8 == 0) LAUNCH(attention_decode_kernel<true>);
+  else LAUNCH(attention_decode_kernel<false>);
 #undef LAUNCH
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
   launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), nullptr, query_start, seq_ids, H, nsplit, num_seqs,
                          stream);
   return tie_launch_status();
+}
+
+extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                         float* part_o, float* part_ml, const int* query_start,
+                                         const int* context_lens, const int* block_tables, const int* seq_ids,
+                                         int num_seqs, int H, int KVH, int block_size, int max_blocks, float scale,
+                                         int window, int nsplit, hipStream_t stream) {
+  return tie_attention_decode_bf16_with(q, k_cache, v_cache, out, part_o, part_ml, query_start, context_lens,
+                                        block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale, window,
+                                        nsplit, 0, stream);
 }

@@ -92,6 +92,9 @@ _SIGNATURES = {
         "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                       _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                       _c_void],
+        "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                           _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                                           _c_int, _c_int, _c_void],
     },
 }
 
@@ -706,11 +709,18 @@ def mfma_block_size(block_size: int) -> bool:
     return block_size >= 4 and block_size & (block_size - 1) == 0
 
 
-def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> int:
+def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int, block_size: int = 16) -> int:
     """How many ways the keys of each sequence are split so that a decode step fills the GPU.
 
-    Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take.
+    Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take. With pages of 16
+    positions or more the kernel keeps several tiles of keys in flight a wave, and about 512 waves (half
+    the GPU's wave slots) with shares of at least 128 keys measured best from batch 1 to 128; with smaller
+    pages a wave has one tile in flight and the GPU wants four times the waves.
     """
+    if block_size >= 16:
+        by_occupancy = -(-512 // max(1, num_seqs * num_kv_heads))
+        by_length = max(1, max_context // 128)          # at least four 32-key tiles a share
+        return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
     by_occupancy = -(-2048 // max(1, num_seqs * num_kv_heads))     # about 2048 waves ...
     if by_occupancy > 16:
         by_occupancy = -(-by_occupancy // 2)        # ... but half as many where that still leaves many shares to merge
@@ -731,8 +741,12 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                           num_seqs: int, num_heads: int, scale: float, window: Optional[int], nsplit: int,
                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
-                          seq_ids: Optional[torch.Tensor] = None) -> None:
-    """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all)."""
+                          seq_ids: Optional[torch.Tensor] = None, depth: int = 0) -> None:
+    """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all).
+
+    ``depth`` picks the kernel (0: by the library's rule; 1: page lookups per lane, any page size; 2 to 4: that
+    many tiles of keys in registers, pages of 16 positions or more); all give the same bits.
+    """
     _gpu(q, "queries")
     _gpu(out, "attention output")
     _gpu(k_cache, "k cache")
@@ -760,10 +774,12 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         if part_o.numel() < num_seqs * H * nsplit * Dh or part_ml.numel() < num_seqs * H * nsplit * 2:
             raise InvalidArgument("the buffers for the splits are too small")
     lib = _lib("attention_decode_bf16", Dh)
-    _call(lib.tie_attention_decode_bf16, "attention_decode_bf16",
+    if not 0 <= depth <= 4 or (depth > 1 and bs < 16):
+        raise InvalidArgument(f"attention_decode_bf16: depth {depth} with pages of {bs} positions")
+    _call(lib.tie_attention_decode_bf16_with, "attention_decode_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), nsplit, _stream())
+        block_tables.shape[1], float(scale), int(window or 0), nsplit, depth, _stream())
 
 
 def prefill_items(new_tokens, group_size: int) -> "list":
@@ -857,7 +873,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
-        nsplit = decode_splits(S, KVH, batch.plan_context)
+        nsplit = decode_splits(S, KVH, batch.plan_context, bs)
         part_o = part_ml = None
         if nsplit > 1:
             part_o = scratch("attention.split_o", (S * num_heads * nsplit * Dh,), torch.float32)
@@ -890,7 +906,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 torch.tensor(merge_rows, dtype=torch.int32).to(q.device) if items else None)
         seq_ids, num_single, items, num_items, merge_rows = work
         if num_single:
-            nsplit = decode_splits(num_single, KVH, batch.plan_context)
+            nsplit = decode_splits(num_single, KVH, batch.plan_context, bs)
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = scratch("attention.split_o", (num_single * num_heads * nsplit * Dh,), torch.float32)
