@@ -673,7 +673,7 @@ def test_attention_decode_bf16_one_sequence_past_32k(H, KVH):
 
 
 
-def run_prefill(case, H, KVH, lens_new, window=None, nsplit=1):
+def run_prefill(case, H, KVH, lens_new, window=None, nsplit=1, staging=0):
     from tie_amd import kernels
 
     q = case["q"]
@@ -687,8 +687,27 @@ def run_prefill(case, H, KVH, lens_new, window=None, nsplit=1):
                      part_o=torch.full((rows * H * nsplit * Dh,), float("nan"), dtype=torch.float32, device="cuda"),
                      part_ml=torch.full((rows * H * nsplit * 2,), float("nan"), dtype=torch.float32, device="cuda"))
     kernels.attention_prefill_bf16(q, case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
-                                   case["tables"], items, H, Dh ** -0.5, window, **extra)
+                                   case["tables"], items, H, Dh ** -0.5, window, staging=staging, **extra)
     return out
+
+
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(8, 2, 128, 16), (6, 2, 32, 16), (12, 2, 64, 32), (2, 1, 256, 16), (3, 3, 128, 64),
+                                         (16, 2, 64, 16)])
+@pytest.mark.parametrize("nsplit,window", [(1, None), (3, None), (1, 100), (2, 45)])
+def test_attention_prefill_bf16_tiles_copied_or_loaded_straight(H, KVH, Dh, bs, nsplit, window):
+    """Both ways of staging the key tiles (through registers; straight into LDS, a page's block of 16 keys per
+    wave) against the plain formula: whole prompts, portions over cached prefixes that start and end inside
+    tiles and pages, one-row portions, with a window and with the keys cut into shares."""
+    from tie_amd import kernels
+
+    assert kernels.prefill_loads_straight(Dh, bs)
+    lens_new, lens_ctx = [13, 5, 1, 70, 2, 200, 64, 33], [13, 29, 300, 150, 33, 777, 64, 1000]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=lens_new, lens_ctx=lens_ctx, seed=29, dtype=torch.bfloat16,
+                             window=window)
+    for staging in (1, 2):
+        out = run_prefill(case, H, KVH, lens_new, window=window, nsplit=nsplit, staging=staging)
+        close(out, case["want"], 1e-2, f"prefill attention staging {staging} H={H} KVH={KVH} Dh={Dh} bs={bs} "
+                                      f"splits={nsplit} window={window}")
 
 
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),

@@ -85,6 +85,9 @@ _SIGNATURES = {
         "tie_attention_prefill_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int,
                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void, _c_void,
                                        _c_void, _c_int, _c_void],
+        "tie_attention_prefill_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void,
+                                            _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
@@ -797,12 +800,22 @@ def prefill_items(new_tokens, group_size: int) -> "list":
     return items
 
 
+def prefill_loads_straight(head_dim: int, block_size: int) -> bool:
+    """Whether the prefill attention kernel that loads its tiles straight into LDS takes this geometry
+    (it has no limit on the cache's size: its addresses are 64-bit scalars)."""
+    return head_dim in (32, 64, 128, 256) and block_size >= 16 and mfma_block_size(block_size)
+
+
 def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                            query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                            items: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None,
                            nsplit: int = 1, part_o: Optional[torch.Tensor] = None,
-                           part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None) -> None:
+                           part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None,
+                           staging: int = 0) -> None:
     """Causal attention of the new rows of the sequences ``items`` names over their cached keys.
+
+    ``staging`` picks how key tiles reach LDS: 1 = copied through registers (any page and head size),
+    2 = loaded straight into LDS (``prefill_loads_straight``), 0 = the second where it applies.
 
     ``nsplit`` > 1 cuts every item's keys into that many shares (one workgroup each) for steps with few
     items and long contexts; ``part_o`` / ``part_ml`` (float32, ``rows * H * nsplit * Dh`` and ``* 2``
@@ -823,7 +836,11 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if Dh not in MFMA_HEAD_DIMS or H % KVH or not mfma_block_size(bs):
         raise InvalidArgument(f"attention_prefill_bf16 takes head sizes in steps of 16 up to 256 and block sizes 4, 8, "
                               f"16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
-    if not prefill_addressable(k_cache):
+    if staging not in (0, 1, 2) or (staging == 2 and not prefill_loads_straight(Dh, bs)):
+        raise InvalidArgument(f"attention_prefill_bf16: staging {staging} with head_dim {Dh} and pages of {bs} positions")
+    if staging == 0:
+        staging = 2 if prefill_loads_straight(Dh, bs) else 1
+    if staging == 1 and not prefill_addressable(k_cache):
         raise InvalidArgument(f"attention_prefill_bf16 addresses cache planes under 32 GB (pages under 128 MB, under 2^24 "
                               f"pages); got {NB} pages of {k_cache[0].numel() * k_cache.element_size()} bytes")
     _i32(query_start, "query_start")
@@ -842,11 +859,11 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         if part_o.numel() < rows * H * nsplit * Dh or part_ml.numel() < rows * H * nsplit * 2 or not 0 < num_merge <= 65535:
             raise InvalidArgument("the buffers for the splits are too small, or no (or too many) rows to merge")
     lib = _lib("attention_prefill_bf16", Dh)
-    _call(lib.tie_attention_prefill_bf16, "attention_prefill_bf16",
+    _call(lib.tie_attention_prefill_bf16_with, "attention_prefill_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
         block_tables.shape[1], float(scale), int(window or 0), int(nsplit), _ptr(part_o), _ptr(part_ml),
-        _ptr(merge_rows), num_merge, _stream())
+        _ptr(merge_rows), num_merge, staging, _stream())
 
 
 def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:
@@ -913,7 +930,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids)
-        if items is not None and not prefill_addressable(k_cache):
+        if items is not None and not prefill_loads_straight(Dh, bs) and not prefill_addressable(k_cache):
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
             paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
