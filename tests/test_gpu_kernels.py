@@ -554,6 +554,73 @@ def run_decode(case, S, H, Dh, nsplit, window=None, depth=0):
     return out
 
 
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(8, 2, 128, 16), (6, 2, 32, 16), (64, 8, 128, 16), (2, 1, 256, 32), (12, 4, 64, 64),
+                                         (16, 1, 128, 16)])
+@pytest.mark.parametrize("planes,normed,window", [(1, True, None), (4, True, None), (2, False, None), (4, True, 50)])
+def test_attention_decode_that_prepares_its_own_queries(H, KVH, Dh, bs, planes, normed, window):
+    """A step of single decoded tokens on the kernel that sums the QKV planes, norms and rotates its queries and
+    writes the newest keys and values itself, against the q/k kernel followed by the decode attention: the same
+    bits in both cache planes and the same output up to rounding, at lengths where the newest position opens a
+    tile or a page."""
+    from tie_amd import kernels
+
+    lens = [1, 16, 17, 32, 33, 64, 65, 129, 300, 700, 1000, 2049]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=[1] * len(lens), lens_ctx=lens, seed=43, dtype=torch.bfloat16,
+                             window=window)
+    width = (H + 2 * KVH) * Dh
+    qkv = (rnd(planes, S, width, seed=44) / planes).cuda()
+    qw = (1 + 0.1 * rnd(Dh, seed=45)).cuda() if normed else None
+    kw = (1 + 0.1 * rnd(Dh, seed=46)).cuda() if normed else None
+    eps = 1e-5
+    inv_freq = torch.from_numpy(plain.rope_inv_freq(1e4, Dh)).float().cuda()
+    positions = i32([c - 1 for c in lens])
+    tables = case["tables"]
+    slots = i32([int(tables[s, (c - 1) // bs]) * bs + (c - 1) % bs for s, c in enumerate(lens)])
+    angles = torch.empty(S, Dh, device="cuda")
+    kernels.rope_angles(positions, inv_freq, angles)
+
+    class Batch:
+        all_decode, num_seqs, plan_context = True, S, max(lens)
+        query_start, context_lens = case["query_start"], case["context_lens"]
+
+    class Step:
+        block_tables = tables
+
+    memory = {}
+
+    def scratch(name, shape, dtype):
+        return memory.setdefault((name, tuple(shape), dtype), torch.full(tuple(shape), float("nan"), dtype=dtype, device="cuda"))
+
+    # the two kernels, one after the other
+    kc1, vc1 = case["kc"].clone(), case["vc"].clone()
+    q = torch.empty(S, H * Dh, dtype=torch.bfloat16, device="cuda")
+    kernels.qk_norm_rope_kv_write(qkv[0], q, qw, kw, eps, inv_freq, positions, slots, kc1, vc1, H, KVH, Dh, bs,
+                                  planes=planes, plane_stride=S * width, angles=angles)
+    apart = torch.full_like(q, float("nan"))
+    nsplit = kernels.decode_splits(S, KVH, max(lens), bs)
+    part_o = torch.empty(S * H * nsplit * Dh, device="cuda")
+    part_ml = torch.empty(S * H * nsplit * 2, device="cuda")
+    kernels.attention_decode_bf16(q, kc1, vc1, apart, case["query_start"], case["context_lens"], tables, S, H, Dh ** -0.5,
+                                  window, nsplit, part_o, part_ml)
+    # the one kernel
+    kc2, vc2 = case["kc"].clone(), case["vc"].clone()
+    assert kernels.decode_attention_prepares(Batch, torch.bfloat16, kc2, H)
+    fused = torch.full_like(q, float("nan"))
+    kernels.paged_attention_prepared(qkv, qw, kw, eps, angles, True, kc2, vc2, fused, Step, Batch, H, Dh ** -0.5, window,
+                                     scratch)
+    assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1), "the newest keys or values differ"
+    assert not torch.isnan(fused.float()).any()
+    # the same queries, keys and values; the newest key is attended to by itself, after the tiles, instead of inside
+    # its tile, so the sums round differently
+    close(fused, apart, 1e-2, "the kernel that prepares its queries")
+    # a cache that holds the token already is left alone
+    kc3, vc3 = kc1.clone(), vc1.clone()
+    again = torch.full_like(q, float("nan"))
+    kernels.paged_attention_prepared(qkv * 3, qw, kw, eps, angles, False, kc3, vc3, again, Step, Batch, H, Dh ** -0.5,
+                                     window, scratch)
+    assert torch.equal(kc3, kc1) and torch.equal(vc3, vc1)
+
+
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(6, 2, 32, 16), (5, 5, 80, 16), (8, 2, 128, 16), (2, 1, 256, 32), (4, 4, 112, 64)])
 @pytest.mark.parametrize("nsplit,window", [(1, None), (2, None), (5, None), (1, 100), (3, 77)])
 def test_attention_decode_bf16_with_tiles_in_flight(H, KVH, Dh, bs, nsplit, window):

@@ -22,6 +22,7 @@
 // Formula: src/backend/cpu/cpu_backend.cpp:261-319 (score = scale * q.k, causal by position,
 // online softmax, query head h reads KV head h / (H / KVH)).
 #include "common.h"
+#include "qk_prepare.h"
 
 #include <math.h>
 
@@ -261,13 +262,32 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 // for all lanes and come by scalar loads, which have a counter of their own; the tiles live in a ring of
 // DEPTH register sets that is walked with constant indices, so no set is copied (a copy would wait for its
 // loads). The arithmetic of a tile and the order of the tiles are those of the kernel above: the same bits.
-template <int DEPTH>
+//
+// PREPARE: the kernel makes its queries itself from the projection's planes of partial sums (sum, per-head RMS
+// norm, rotation by the step's table of angles: the q/k kernel's own functions, so the same bits), every wave
+// those of its KV head's group, through LDS into the operand layout; and the wave whose share holds the
+// sequence's newest position first makes that token's key and value and writes them into the cache, waits
+// for the stores, and only then reads its tiles. One kernel less a layer; head sizes 32 to 256 in powers of
+// two (head_dim / 8 lanes a head).
+struct QkSource {
+  const float* qkv;        // [planes][rows][in_row] float32: q heads, k heads, v heads of a row
+  size_t plane_stride;
+  int planes;
+  int in_row;
+  const float* q_weight;   // per-head norm weights, or null for no norm
+  const float* k_weight;
+  float eps;
+  const float* angles;     // [rows][DH]: cos of the DH / 2 angles, then sin
+  int write_kv;            // 0: the cache holds the newest token already (another layer's cache)
+};
+
+template <int DEPTH, bool PREPARE>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const bf16_t* __restrict__ q, bf16_t* k_cache, bf16_t* v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit) {
+    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit, QkSource src) {
   const int lane = threadIdx.x;
   const int col = lane & 15;
   const int quad = lane >> 4;
@@ -286,8 +306,18 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   const int tile_begin = first_tile + split * per_split;
   const int tile_end = min(num_tiles, tile_begin + per_split);
 
+  const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
+  const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
   u32x4_t qf[KSTEPS];
-  {
+  // PREPARE: the wave whose share ends the sequence takes the newest token from the projection itself: it makes
+  // the token's key and value, sends them to the cache for later steps, keeps them (as the cache will hold
+  // them, in bfloat16) in LDS, leaves the newest position out of its last tile and attends to it by itself
+  // after the loop. Nothing it reads from the cache was written in this launch.
+  const bool takes_newest = PREPARE && src.write_kv && tile_end == num_tiles && tile_begin < tile_end;
+  const int last_cached = takes_newest ? pos - 1 : pos;     // the newest position the tiles may show
+  __shared__ __attribute__((aligned(16))) bf16_t newest_lds[PREPARE ? 2 * DH : 8];   // key, then value
+  if constexpr (PREPARE) {
+  } else {
     const bool valid = col < G;
     const bf16_t* qr = q + (static_cast<size_t>(t) * H + static_cast<size_t>(kvh) * G + (valid ? col : 0)) * DH;
 #pragma unroll
@@ -301,8 +331,6 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   for (int dt = 0; dt < DTILES; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
-  const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
   const int krow0 = (col >> 2) * 8 + (col & 3);
   const bool keys_in_upper_half = krow0 >= 16;      // both sub-tiles' rows (krow0, krow0 + 4) lie in one half
   const bool values_in_upper_half = quad >= 2;      // positions quad * 8 .. + 7
@@ -347,22 +375,133 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 #pragma unroll
   for (int j = 0; j < DEPTH - 1; ++j)
     if (tile_begin + j < tile_end) issue(tile_begin + j, ring[j]);
+  if constexpr (PREPARE) {
+    // After the first tiles' loads are on their way: the group's queries, HEADS_AT_ONCE heads at a time with a
+    // head's lanes together, and the newest key (lanes 0 .. LPH - 1) and value (the next LPH lanes).
+    constexpr int LPH = DH / 8, HALF = DH / 2, HEADS_AT_ONCE = TIE_WAVE / LPH;
+    __shared__ __attribute__((aligned(16))) bf16_t q_lds[16 * DH];
+    const float* row = src.qkv + static_cast<size_t>(t) * src.in_row;
+    const float* angles = src.angles + static_cast<size_t>(t) * DH;
+    const int p0 = (lane % LPH) * 4;
+    // All loads first, so that they share one trip to memory: the first HEADS_AT_ONCE query heads (lanes beyond
+    // the group read its last head again) and, in the wave that takes the newest token, its key (the lanes
+    // of even heads-worth) or value (odd), 4 + 4 elements a lane like a query's.
+    const int g_first = lane / LPH;
+    const float* q_in = row + (static_cast<size_t>(kvh) * G + min(g_first, G - 1)) * DH;
+    qk_f4_t qa = load4_planes(q_in + p0, src.plane_stride, src.planes);
+    qk_f4_t qb = load4_planes(q_in + HALF + p0, src.plane_stride, src.planes);
+    qk_f4_t na = {0.f, 0.f, 0.f, 0.f}, nb = na;
+    const bool value_lane = (g_first & 1) != 0;
+    if (takes_newest) {
+      const float* n_in = row + static_cast<size_t>(H + kvh + (value_lane ? KVH : 0)) * DH;
+      na = load4_planes(n_in + p0, src.plane_stride, src.planes);
+      nb = load4_planes(n_in + HALF + p0, src.plane_stride, src.planes);
+    }
+    if (g_first < G) {
+      if (src.q_weight != nullptr) qk_head_norm<LPH>(qa, qb, src.q_weight, src.eps, p0);
+      qk_f4_t o1, o2;
+      qk_rotate_by_table<LPH>(qa, qb, angles, p0, o1, o2);
+      store4(q_lds + g_first * DH + p0, o1);
+      store4(q_lds + g_first * DH + HALF + p0, o2);
+    }
+    if (takes_newest) {
+      const int page = table[pos >> block_shift];
+      const int off = pos & (block_size - 1);
+      if (lane < LPH) {
+        if (src.k_weight != nullptr) qk_head_norm<LPH>(na, nb, src.k_weight, src.eps, p0);
+        qk_f4_t o1, o2;
+        qk_rotate_by_table<LPH>(na, nb, angles, p0, o1, o2);
+        bf16_t* dst = k_cache + static_cast<size_t>(page) * page_stride + head_off + static_cast<size_t>(off) * DH;
+        store4(dst + p0, o1);
+        store4(dst + HALF + p0, o2);
+        store4(newest_lds + p0, o1);
+        store4(newest_lds + HALF + p0, o2);
+      } else if (lane < 2 * LPH) {
+        // In a page the dimensions of a value lie block_size apart.
+        bf16_t* dst = v_cache + static_cast<size_t>(page) * page_stride + head_off + off;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          store_from_float(dst + static_cast<size_t>(p0 + j) * block_size, na[j]);
+          store_from_float(dst + static_cast<size_t>(HALF + p0 + j) * block_size, nb[j]);
+        }
+        store4(newest_lds + DH + p0, na);
+        store4(newest_lds + DH + HALF + p0, nb);
+      }
+    }
+    for (int g0 = HEADS_AT_ONCE; g0 < G; g0 += HEADS_AT_ONCE) {
+      const int g = g0 + lane / LPH;
+      if (g < G) {
+        const float* in = row + (static_cast<size_t>(kvh) * G + g) * DH;
+        qk_f4_t a = load4_planes(in + p0, src.plane_stride, src.planes);
+        qk_f4_t b = load4_planes(in + HALF + p0, src.plane_stride, src.planes);
+        if (src.q_weight != nullptr) qk_head_norm<LPH>(a, b, src.q_weight, src.eps, p0);
+        qk_f4_t o1, o2;
+        qk_rotate_by_table<LPH>(a, b, angles, p0, o1, o2);
+        store4(q_lds + g * DH + p0, o1);
+        store4(q_lds + g * DH + HALF + p0, o2);
+      }
+    }
+    __syncthreads();   // one wave: the writes above are done before the reads below
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+      const int d = st * 32 + quad * 8;
+      qf[st] = (col < G && d < DH) ? *reinterpret_cast<const u32x4_t*>(q_lds + col * DH + d) : u32x4_t{0, 0, 0, 0};
+    }
+  }
   int tile = tile_begin;
   for (; tile + 2 * DEPTH - 2 < tile_end; tile += DEPTH) {
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) {
       issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
-      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, pos, quad, scale_log2e);
+      attend_tile(ring[j].k, ring[j].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad, scale_log2e);
     }
   }
 #pragma unroll
   for (int j = 0; j < 2 * DEPTH - 2; ++j) {
     if (tile + j < tile_end) {
       if (j < DEPTH - 1 && tile + j + DEPTH - 1 < tile_end) issue(tile + j + DEPTH - 1, ring[(j + DEPTH - 1) % DEPTH]);
-      attend_tile(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, pos, quad, scale_log2e);
+      attend_tile(ring[j % DEPTH].k, ring[j % DEPTH].v, qf, acc, m, l, (tile + j) * 32, start, last_cached, quad,
+                    scale_log2e);
     }
   }
 
+  if constexpr (PREPARE) {
+    if (takes_newest) {
+      // The newest key by itself: its score for this lane's column from the 32 dimensions the lane holds of the
+      // query, summed over the four quads; then one step of the online softmax with a single key, the
+      // probability rounded to bfloat16 as the tiles' are.
+      float dot = 0.f;
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) {
+        const int d = st * 32 + quad * 8;
+        if (DH % 32 == 0 || d < DH) {
+          const u32x4_t kq = *reinterpret_cast<const u32x4_t*>(newest_lds + d);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dot = fmaf(__uint_as_float(qf[st][e] << 16), __uint_as_float(kq[e] << 16), dot);
+            dot = fmaf(__uint_as_float(qf[st][e] & 0xffff0000u), __uint_as_float(kq[e] & 0xffff0000u), dot);
+          }
+        }
+      }
+      dot += __shfl_xor(dot, 16, TIE_WAVE);
+      dot += __shfl_xor(dot, 32, TIE_WAVE);
+      const float m_new = fmaxf(m, dot);
+      const float neg_mc = -m_new * scale_log2e;
+      const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
+      const float p = __builtin_amdgcn_exp2f(fmaf(dot, scale_log2e, neg_mc));
+      const float p_rounded = __uint_as_float(pack_bf16x2(p, 0.f) << 16);
+      l = l * corr + (quad == 0 ? p : 0.f);
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt) {
+        const u32x2_t vv = *reinterpret_cast<const u32x2_t*>(newest_lds + DH + dt * 16 + quad * 4);
+        acc[dt][0] = fmaf(p_rounded, __uint_as_float(vv.x << 16), acc[dt][0] * corr);
+        acc[dt][1] = fmaf(p_rounded, __uint_as_float(vv.x & 0xffff0000u), acc[dt][1] * corr);
+        acc[dt][2] = fmaf(p_rounded, __uint_as_float(vv.y << 16), acc[dt][2] * corr);
+        acc[dt][3] = fmaf(p_rounded, __uint_as_float(vv.y & 0xffff0000u), acc[dt][3] * corr);
+      }
+    }
+  }
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
@@ -374,13 +513,12 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 extern "C" int tie_attention_decode_head_dim() { return DH; }
 extern "C" int tie_attention_max_splits() { return MERGE_MAX_SPLITS; }
 
-// depth: 0 = by the rule, 1 = the kernel that looks its pages up per lane (any page size), 2 to 4 = the ring
-// kernel with that many register sets (pages of 16 positions or more); for tests and sweeps.
-extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                              float* part_o, float* part_ml, const int* query_start,
-                                              const int* context_lens, const int* block_tables, const int* seq_ids,
-                                              int num_seqs, int H, int KVH, int block_size, int max_blocks,
-                                              float scale, int window, int nsplit, int depth, hipStream_t stream) {
+constexpr bool PREPARE_HEAD_DIM = DH == 32 || DH == 64 || DH == 128 || DH == 256;
+
+static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out,
+                         float* part_o, float* part_ml, const int* query_start, const int* context_lens,
+                         const int* block_tables, const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
+                         int max_blocks, float scale, int window, int nsplit, int depth, hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
@@ -390,25 +528,73 @@ extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache
   // Measured: the ring of three register sets where the keys are cut into shares, of four where a wave walks
   // a whole sequence.
   if (depth == 0) depth = block_size < 16 ? 1 : (nsplit == 1 ? 4 : 3);
+  if (src != nullptr && (depth < 2 || !PREPARE_HEAD_DIM)) return TIE_BAD_ARGUMENT;
   const dim3 grid(nsplit, KVH, num_seqs);
   const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
-#define LAUNCH(KERNEL)                                                                                          \
-  KERNEL<<<grid, TIE_WAVE, 0, stream>>>(                                                                         \
-      static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),  \
-      static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH,     \
-      block_size, block_shift, max_blocks, scale_log2e, window, nsplit)
-  if (depth == 4) LAUNCH(attention_decode_ring_kernel<4>);
-  else if (depth == 3) LAUNCH(attention_decode_ring_kernel<3>);
-  else if (depth == 2) LAUNCH(attention_decode_ring_kernel<2>);
-  else if (block_size % 8 == 0) LAUNCH(attention_decode_kernel<true>);
-  else LAUNCH(attention_decode_kernel<false>);
-#undef LAUNCH
+#define ARGS out, part_o, part_ml, query_start, context_lens, block_tables, seq_ids, H, KVH, block_size, block_shift, \
+             max_blocks, scale_log2e, window, nsplit
+#define LAUNCH_RING(DEPTH)                                                                                   \
+  {                                                                                                          \
+    if (src == nullptr) {                                                                                    \
+      attention_decode_ring_kernel<DEPTH, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS,   \
+                                                                                QkSource{});                 \
+    } else if constexpr (PREPARE_HEAD_DIM) {                                                                 \
+      attention_decode_ring_kernel<DEPTH, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS, *src); \
+    }                                                                                                        \
+  }
+  if (depth == 4) LAUNCH_RING(4)
+  else if (depth == 3) LAUNCH_RING(3)
+  else if (depth == 2) LAUNCH_RING(2)
+  else if (block_size % 8 == 0) attention_decode_kernel<true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);
+  else attention_decode_kernel<false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);
+#undef LAUNCH_RING
+#undef ARGS
   int status = tie_launch_status();
   if (status != TIE_OK || nsplit == 1) return status;
-  launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), nullptr, query_start, seq_ids, H, nsplit, num_seqs,
-                         stream);
+  launch_attention_merge(part_o, part_ml, out, nullptr, query_start, seq_ids, H, nsplit, num_seqs, stream);
   return tie_launch_status();
+}
+
+// depth: 0 = by the rule, 1 = the kernel that looks its pages up per lane (any page size), 2 to 4 = the ring
+// kernel with that many register sets (pages of 16 positions or more); for tests and sweeps.
+extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              float* part_o, float* part_ml, const int* query_start,
+                                              const int* context_lens, const int* block_tables, const int* seq_ids,
+                                              int num_seqs, int H, int KVH, int block_size, int max_blocks,
+                                              float scale, int window, int nsplit, int depth, hipStream_t stream) {
+  return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
+                       static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
+                       query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
+                       scale, window, nsplit, depth, stream);
+}
+
+// The same for a step of single decoded tokens whose queries, newest keys and values still lie in the QKV
+// projection's output: qkv is float32 [planes][rows][in_row] (plane p at qkv + p * plane_stride; a row holds H
+// query heads, KVH key heads, KVH value heads), summed over the planes by the kernel; q_weight / k_weight (or
+// null) the per-head RMS norm weights with eps; angles [rows][head_dim] the step's table of cos and sin.
+// write_kv = 0 where the cache is another layer's and holds the token already. Pages of 16 positions or more
+// and head sizes 32, 64, 128, 256; refused otherwise (tie_attention_decode_prepares tells).
+extern "C" int tie_attention_decode_prepares(int block_size) { return PREPARE_HEAD_DIM && block_size >= 16 ? 1 : 0; }
+
+extern "C" int tie_attention_decode_prepared_bf16(const float* qkv, long plane_stride, int planes, int in_row,
+                                                  const float* q_weight, const float* k_weight, float eps,
+                                                  const float* angles, int write_kv, void* k_cache, void* v_cache,
+                                                  void* out, float* part_o, float* part_ml, const int* query_start,
+                                                  const int* context_lens, const int* block_tables,
+                                                  const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
+                                                  int max_blocks, float scale, int window, int nsplit, int depth,
+                                                  hipStream_t stream) {
+  if (qkv == nullptr || angles == nullptr || planes < 1 || planes > 8 || plane_stride < 0 || block_size < 16 ||
+      depth == 1 || H <= 0 || KVH <= 0 || in_row < (H + 2 * KVH) * DH || in_row % 4 != 0 || plane_stride % 4 != 0 ||
+      reinterpret_cast<uintptr_t>(qkv) % 16 != 0 || reinterpret_cast<uintptr_t>(angles) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(q_weight) % 16 != 0 || reinterpret_cast<uintptr_t>(k_weight) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(k_cache) % 16 != 0)
+    return TIE_BAD_ARGUMENT;
+  const QkSource src = {qkv, static_cast<size_t>(plane_stride), planes, in_row, q_weight, k_weight, eps, angles, write_kv};
+  return launch_decode(nullptr, &src, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache),
+                       static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids,
+                       num_seqs, H, KVH, block_size, max_blocks, scale, window, nsplit, depth, stream);
 }
 
 extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,

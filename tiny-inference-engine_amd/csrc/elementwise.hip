@@ -3,6 +3,7 @@
 // sampling kernels (argmax, temperature). All arithmetic is float32; only
 // loads and stores convert. One C entry point per operation.
 #include "common.h"
+#include "qk_prepare.h"
 #include "argmax_static.h"
 
 #include <math.h>
@@ -281,25 +282,6 @@ extern "C" int tie_add_partials_rms_norm(float* x, const float* partials, long p
 // apart (a product cut along K): they are added in plane order as they are read.
 #define TIE_MAX_PAIRS 4  // head_dim <= 512
 
-template <typename TX>
-__device__ __forceinline__ float load_planes(const TX* p, size_t plane_stride, int planes) {
-  // The usual cuts (2, 4, 8) have all their loads in flight together; the sum is formed in plane order in every case.
-  if (planes == 2) return load_as_float(p) + load_as_float(p + plane_stride);
-  if (planes == 4 || planes == 8) {
-    float part[8];
-#pragma unroll
-    for (int s = 0; s < 8; ++s) part[s] = s < planes ? load_as_float(p + static_cast<size_t>(s) * plane_stride) : 0.f;
-    float v = part[0];
-#pragma unroll
-    for (int s = 1; s < 8; ++s)
-      if (s < planes) v += part[s];
-    return v;
-  }
-  float v = load_as_float(p);
-  for (int s = 1; s < planes; ++s) v += load_as_float(p + static_cast<size_t>(s) * plane_stride);
-  return v;
-}
-
 template <typename TX, typename TQ, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const float* __restrict__ q_w,
                                              const float* __restrict__ k_w, float eps,
@@ -404,49 +386,6 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
 // first half and the 4 they pair with in the second (16-byte loads and stores where the one-wave-a-head
 // kernel above moves 4 and 2 bytes), head_dim / 8 lanes share a head, four waves of heads a workgroup.
 // The sums of squares meet by shuffles inside the lanes of a head. Whole heads rotated as halves only.
-typedef __attribute__((ext_vector_type(4))) float qk_f4_t;
-
-template <typename T>
-__device__ __forceinline__ qk_f4_t load4(const T* p);
-template <>
-__device__ __forceinline__ qk_f4_t load4<float>(const float* p) { return *reinterpret_cast<const qk_f4_t*>(p); }
-template <>
-__device__ __forceinline__ qk_f4_t load4<bf16_t>(const bf16_t* p) {
-  const uint2 v = *reinterpret_cast<const uint2*>(p);
-  return qk_f4_t{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
-                 __uint_as_float(v.y & 0xffff0000u)};
-}
-template <typename T>
-__device__ __forceinline__ void store4(T* p, qk_f4_t v);
-template <>
-__device__ __forceinline__ void store4<float>(float* p, qk_f4_t v) { *reinterpret_cast<qk_f4_t*>(p) = v; }
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, qk_f4_t v) {
-  uint2 o;
-  o.x = pack_bf16x2(v[0], v[1]);
-  o.y = pack_bf16x2(v[2], v[3]);
-  *reinterpret_cast<uint2*>(p) = o;
-}
-
-template <typename TX>
-__device__ __forceinline__ qk_f4_t load4_planes(const TX* p, size_t plane_stride, int planes) {
-  if (planes == 2) return load4(p) + load4(p + plane_stride);
-  if (planes == 4 || planes == 8) {
-    qk_f4_t part[8];
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
-      part[s] = s < planes ? load4(p + static_cast<size_t>(s) * plane_stride) : qk_f4_t{0.f, 0.f, 0.f, 0.f};
-    qk_f4_t v = part[0];
-#pragma unroll
-    for (int s = 1; s < 8; ++s)
-      if (s < planes) v += part[s];
-    return v;
-  }
-  qk_f4_t v = load4(p);
-  for (int s = 1; s < planes; ++s) v += load4(p + static_cast<size_t>(s) * plane_stride);
-  return v;
-}
-
 #define QK4_THREADS 256
 
 template <typename TX, typename TQ, typename TC, int LPH>   // LPH: lanes per head = head_dim / 8
@@ -481,21 +420,10 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
   qk_f4_t b = load4_planes(in + half + p0, plane_stride, planes);
 
   const float* w = is_q ? q_w : k_w;
-  if (w != nullptr) {
-    float ss = (a[0] * a[0] + b[0] * b[0]) + (a[1] * a[1] + b[1] * b[1]) + (a[2] * a[2] + b[2] * b[2]) +
-               (a[3] * a[3] + b[3] * b[3]);
-#pragma unroll
-    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, TIE_WAVE);
-    const float inv = 1.0f / sqrtf(ss / static_cast<float>(Dh) + eps);
-    a = (a * inv) * load4(w + p0);
-    b = (b * inv) * load4(w + half + p0);
-  }
+  if (w != nullptr) qk_head_norm<LPH>(a, b, w, eps, p0);
   qk_f4_t o1 = a, o2 = b;
   if (angles != nullptr) {
-    const qk_f4_t cs = load4(angles + static_cast<size_t>(t) * Dh + p0);
-    const qk_f4_t sn = load4(angles + static_cast<size_t>(t) * Dh + half + p0);
-    o1 = a * cs - b * sn;
-    o2 = b * cs + a * sn;
+    qk_rotate_by_table<LPH>(a, b, angles + static_cast<size_t>(t) * Dh, p0, o1, o2);
   } else if (inv_freq != nullptr) {
     const float pos = static_cast<float>(positions[t]);
 #pragma unroll

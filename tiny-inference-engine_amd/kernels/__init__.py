@@ -95,6 +95,11 @@ _SIGNATURES = {
         "tie_attention_decode_bf16": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                       _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                       _c_void],
+        "tie_attention_decode_prepares": [_c_int],
+        "tie_attention_decode_prepared_bf16": [_c_void, _c_long, _c_int, _c_int, _c_void, _c_void, _c_float, _c_void,
+                                               _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                               _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                               _c_int, _c_int, _c_int, _c_void],
         "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                            _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                                            _c_int, _c_int, _c_void],
@@ -783,6 +788,52 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
         block_tables.shape[1], float(scale), int(window or 0), nsplit, depth, _stream())
+
+
+def decode_attention_prepares(batch, q_dtype: torch.dtype, k_cache: torch.Tensor, num_heads: int) -> bool:
+    """Whether a step runs on the decode attention kernel that makes its own queries, newest keys and values
+    from the QKV projection's planes: single decoded tokens only, bfloat16, pages of 16 positions or more,
+    head sizes 32, 64, 128 or 256, at most 16 query heads a KV head."""
+    NB, KVH, bs, Dh = k_cache.shape
+    return (batch.all_decode and q_dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
+            and Dh in (32, 64, 128, 256) and bs >= 16 and mfma_block_size(bs)
+            and num_heads % KVH == 0 and num_heads // KVH <= 16)
+
+
+def paged_attention_prepared(planes: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                             eps: float, angles: torch.Tensor, write_kv: bool, k_cache: torch.Tensor,
+                             v_cache: torch.Tensor, out: torch.Tensor, step, batch, num_heads: int, scale: float,
+                             window: Optional[int], scratch) -> None:
+    """Attention of a step of single decoded tokens straight from the QKV projection's planes of partial sums
+    (``planes`` float32 ``[P, rows, (H + 2 KVH) * Dh]``): the kernel sums the planes, applies the per-head
+    RMS norm (weights or None) and the rotation by ``angles`` (``[rows, Dh]``: cos, then sin), writes the newest
+    key and value into the cache (unless ``write_kv`` is false) and attends; see ``decode_attention_prepares``."""
+    NB, KVH, bs, Dh = k_cache.shape
+    _check_cache(k_cache, v_cache, KVH, bs, Dh)
+    H, S = num_heads, batch.num_seqs
+    if not decode_attention_prepares(batch, out.dtype, k_cache, H):
+        raise InvalidArgument("this step does not run on the decode attention kernel that prepares its own queries")
+    _f32(planes, "QKV planes")
+    _f32(angles, "rotation angles")
+    _gpu(out, "attention output")
+    P, rows, width = planes.shape
+    if not planes.is_contiguous() or width < (H + 2 * KVH) * Dh or rows != out.shape[0] or out.shape[1] != H * Dh:
+        raise InvalidArgument(f"QKV planes {list(planes.shape)} / out {list(out.shape)} do not fit {H} + 2 x {KVH} heads of {Dh}")
+    if angles.shape != (rows, Dh) or not angles.is_contiguous() or not 1 <= P <= 8:
+        raise InvalidArgument(f"angles {list(angles.shape)} for {rows} rows of head_dim {Dh}, {P} planes")
+    for w, name in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
+        if w is not None:
+            _f32(w, name, (Dh,))
+    nsplit = decode_splits(S, KVH, batch.plan_context, bs)
+    part_o = part_ml = None
+    if nsplit > 1:
+        part_o = scratch("attention.split_o", (S * H * nsplit * Dh,), torch.float32)
+        part_ml = scratch("attention.split_ml", (S * H * nsplit * 2,), torch.float32)
+    _call(_lib("attention_decode_bf16", Dh).tie_attention_decode_prepared_bf16, "attention_decode_prepared_bf16",
+          planes.data_ptr(), rows * width, P, width, _ptr(q_weight), _ptr(k_weight), float(eps), angles.data_ptr(),
+          int(bool(write_kv)), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
+          batch.query_start.data_ptr(), batch.context_lens.data_ptr(), step.block_tables.data_ptr(), None, S, H, KVH,
+          bs, step.block_tables.shape[1], float(scale), int(window or 0), nsplit, 0, _stream())
 
 
 def prefill_items(new_tokens, group_size: int) -> "list":
