@@ -551,10 +551,12 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int first16 = wg_first & ~15, last16 = wg_last & ~15;
   const size_t page_elems = static_cast<size_t>(KVH) * block_size * DH;
   const size_t head_elems = static_cast<size_t>(kvh) * block_size * DH;
-  // Block `wave` of tile `tile` into buffer `buf`.
-  auto issue = [&](int tile, int buf) {
+  // The page of block `wave` of tile `tile` (a scalar load), looked up one tile before the block is loaded
+  // so that no load waits for it.
+  auto page_of_block = [&](int tile) { return table[min(max(tile * KT + wave * 16, first16), last16) >> block_shift]; };
+  // Block `wave` of tile `tile`, which lies in `page`, into buffer `buf`.
+  auto issue = [&](int tile, int buf, int page) {
     const int p16 = min(max(tile * KT + wave * 16, first16), last16);
-    const int page = table[p16 >> block_shift];
     const int off = p16 & (block_size - 1);
     const bf16_t* kb = k_cache + static_cast<size_t>(page) * page_elems + head_elems + static_cast<size_t>(off) * DH;
     const bf16_t* vb = v_cache + static_cast<size_t>(page) * page_elems + head_elems + off;
@@ -577,7 +579,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   for (int ks = 0; ks < KS; ++ks) k_frag[ks] = r32 * DH + (((ks * 2 + hi) ^ swz) * 8);
   const int v_frag = r32 * 16 + ((hi ^ ((r32 >> 3) & 1)) * 8);
 
-  if (!empty) issue(tile_begin, 0);
+  int next_page = 0;
+  if (!empty) {
+    issue(tile_begin, 0, page_of_block(tile_begin));
+    if (tile_begin < tile_end) next_page = page_of_block(tile_begin + 1);
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
@@ -585,7 +591,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const int buf = (tile - tile_begin) & 1;
     const bf16_t* k_lds = lds + buf * DMA_TILE;
     const bf16_t* v_lds = k_lds + KT * DH;
-    if (tile < tile_end) issue(tile + 1, buf ^ 1);   // that buffer was last read before the barrier below
+    if (tile < tile_end) {
+      issue(tile + 1, buf ^ 1, next_page);           // that buffer was last read before the barrier below
+      if (tile + 1 < tile_end) next_page = page_of_block(tile + 2);
+    }
 
     const int base = tile * KT;
     if (wave_active && base <= wave_last) {
