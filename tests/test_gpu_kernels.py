@@ -758,6 +758,74 @@ def run_prefill(case, H, KVH, lens_new, window=None, nsplit=1, staging=0):
     return out
 
 
+def test_attention_kernels_over_cache_planes_beyond_4_gb():
+    """Pages that lie more than 4 GB into a cache plane of 4.5 GB (byte offsets that no 32-bit number holds): the
+    prefill kernel that loads straight into LDS, the decode kernel with its tiles in flight, and the same kernel
+    making its own queries and writing the newest key and value there."""
+    from tie_amd import kernels
+
+    H, KVH, Dh, bs = 8, 8, 128, 16
+    NB = (9 << 29) // (KVH * bs * Dh * 2)                   # 4.5 GB a plane
+    kc = torch.zeros(NB, KVH, bs, Dh, dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros(NB, KVH, Dh, bs, dtype=torch.bfloat16, device="cuda")
+    lens = [70, 300]
+    rng = np.random.RandomState(5)
+    far = list(NB - 1 - rng.permutation(64))                # the last pages of the plane
+    assert min(far) * KVH * bs * Dh * 2 > 1 << 32
+    tables = np.zeros((len(lens), 32), dtype=np.int32)
+    qs, ks, vs = [], [], []
+    for s, ctx in enumerate(lens):
+        q, k, v = (rnd(ctx, n, Dh, seed=60 + 3 * s + i).to(torch.bfloat16) for i, n in enumerate((H, KVH, KVH)))
+        for j in range(math.ceil(ctx / bs)):
+            page = int(far.pop())
+            tables[s, j] = page
+            rows = slice(j * bs, min(ctx, (j + 1) * bs))
+            kc[page, :, :rows.stop - rows.start] = k[rows].transpose(0, 1).cuda()
+            vc[page, :, :, :rows.stop - rows.start] = v[rows].permute(1, 2, 0).cuda()
+        qs.append(q), ks.append(k), vs.append(v)
+    tables = torch.from_numpy(tables).cuda()
+    scale = Dh ** -0.5
+    whole = [plain.causal_attention(q.float(), k.float(), v.float(), scale) for q, k, v in zip(qs, ks, vs)]
+    # the prompts whole
+    q_all = torch.cat([q.reshape(len(q), H * Dh) for q in qs]).cuda()
+    out = torch.full_like(q_all, float("nan"))
+    items = torch.tensor(kernels.prefill_items(lens, H // KVH), dtype=torch.int32).cuda()
+    kernels.attention_prefill_bf16(q_all, kc, vc, out, i32([0, lens[0], sum(lens)]), i32(lens), tables, items, H, scale,
+                                   staging=2)
+    close(out, torch.cat([w.reshape(len(w), H * Dh) for w in whole]), 1e-2, "prefill attention beyond 4 GB")
+    # the last rows as decoded tokens
+    q_last = torch.stack([q[-1].reshape(H * Dh) for q in qs]).cuda()
+    want_last = torch.stack([w[-1].reshape(H * Dh) for w in whole])
+    for nsplit in (1, 2):
+        got = torch.full_like(q_last, float("nan"))
+        kernels.attention_decode_bf16(q_last, kc, vc, got, i32([0, 1, 2]), i32(lens), tables, 2, H, scale, None, nsplit,
+                                      torch.empty(2 * H * nsplit * Dh, device="cuda"),
+                                      torch.empty(2 * H * nsplit * 2, device="cuda"), depth=3)
+        close(got, want_last, 1e-2, f"decode attention beyond 4 GB, {nsplit} shares")
+    # the same rows from a projection's output: no norm, angles of position 0 (cos 1, sin 0) leave q and k as they are
+    width = (H + 2 * KVH) * Dh
+    qkv = torch.stack([torch.cat([q[-1].reshape(-1), k[-1].reshape(-1), v[-1].reshape(-1)]).float() for q, k, v in zip(qs, ks, vs)])
+    angles = torch.cat([torch.ones(2, Dh // 2), torch.zeros(2, Dh // 2)], dim=1).cuda()
+    for s, ctx in enumerate(lens):                          # the kernel has to write these itself
+        kc[tables[s, (ctx - 1) // bs], :, (ctx - 1) % bs] = 7.0
+        vc[tables[s, (ctx - 1) // bs], :, :, (ctx - 1) % bs] = 7.0
+
+    class Batch:
+        all_decode, num_seqs, plan_context = True, 2, 4096
+        query_start, context_lens = i32([0, 1, 2]), i32(lens)
+
+    class Step:
+        block_tables = tables
+
+    got = torch.full_like(q_last, float("nan"))
+    kernels.paged_attention_prepared(qkv.view(1, 2, width).cuda().contiguous(), None, None, 0.0, angles, True, kc, vc, got,
+                                     Step, Batch, H, scale, None, lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device="cuda"))
+    close(got, want_last, 1e-2, "decode attention that prepares its queries, beyond 4 GB")
+    for s, ctx in enumerate(lens):
+        page, off = int(tables[s, (ctx - 1) // bs]), (ctx - 1) % bs
+        assert torch.equal(kc[page, :, off].cpu(), ks[s][-1]) and torch.equal(vc[page, :, :, off].cpu(), vs[s][-1])
+
+
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(8, 2, 128, 16), (6, 2, 32, 16), (12, 2, 64, 32), (2, 1, 256, 16), (3, 3, 128, 64),
                                          (16, 2, 64, 16)])
 @pytest.mark.parametrize("nsplit,window", [(1, None), (3, None), (1, 100), (2, 45)])
