@@ -105,6 +105,43 @@ def test_single_rows_beside_portions_on_either_attention_kernel(folders, name, m
         check(got[ride_along], want, "bfloat16", f"{name}/bfloat16/mixed, single rows riding along up to {ride_along}")
 
 
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_decode_steps_with_and_without_the_attention_kernel_that_prepares(folders, monkeypatch, use_graphs):
+    """Steps of single decoded tokens run on the attention kernel that makes its own queries and newest keys
+    (heads of 32, pages of 16: configuration B); switched off, the q/k kernel runs before the decode attention.
+    Both against the plain implementation, the last 32 tokens of every request decoded one by one, and the
+    keys and values the first way left in the cache serve the second way's later steps just as well."""
+    import tie_amd.parts.attention as attention_part
+    from tie_amd import kernels
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["bfloat16"]["B"]
+    requests = th.make_requests(cfg["vocab_size"], LENGTHS["B"], seed=9)
+    want = reference_logits(folder, cfg, requests)
+    steps = th.prefill_then_decode(requests)
+    biggest = max(th.round64(len(t)) for t in requests.values())
+    calls = {"prepared": 0}
+    prepared = kernels.paged_attention_prepared
+
+    def counted(*args, **kwargs):
+        calls["prepared"] += 1
+        return prepared(*args, **kwargs)
+
+    monkeypatch.setattr(attention_part.kernels, "paged_attention_prepared", counted)
+    on = th.collect(TraceReplayer.from_folder(folder, "bfloat16", biggest, block_size=16, use_graphs=use_graphs), steps)
+    assert calls["prepared"] > 0, "no decode step took the kernel that prepares its own queries"
+    check(on, want, "bfloat16", "B/bfloat16/decode steps on the kernel that prepares")
+    monkeypatch.setattr(attention_part.kernels, "decode_attention_prepares", lambda *a, **k: False)
+    before = calls["prepared"]
+    off = th.collect(TraceReplayer.from_folder(folder, "bfloat16", biggest, block_size=16, use_graphs=use_graphs), steps)
+    assert calls["prepared"] == before
+    check(off, want, "bfloat16", "B/bfloat16/decode steps on the q/k kernel and the decode attention")
+    for rid in requests:
+        a = torch.stack([on[rid][p] for p in sorted(on[rid])])
+        b = torch.stack([off[rid][p] for p in sorted(off[rid])])
+        assert float((a - b).abs().max() / b.abs().max()) < 2e-2, f"request {rid}: the two ways differ by more than rounding"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("use_graphs", [False, True])
 def test_layers_of_one_shape_run_from_one_layers_launch_list(tmp_path, dtype, use_graphs):

@@ -89,14 +89,14 @@ class PagedAttention(Mixer):
             self.qkv(h, qkv)
         if table is not None:
             inv_freq, rotary_dim, pairing = table
-            if (planes is not None and inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half"
+            if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half"
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
                 # A step of single decoded tokens: the attention kernel sums the planes, norms and rotates its own
                 # queries and writes the newest keys and values itself: one kernel less.
                 attn = ctx.scratch("attention.out", (T, self.q_dim))
                 kernels.paged_attention_prepared(
-                    planes, self.q_norm_weight if self.qk_norm else None, self.k_norm_weight if self.qk_norm else None,
-                    eps, self.position.angles(ctx), cache.writes, cache.k_cache, cache.v_cache, attn, step, ctx.batch,
+                    planes if planes is not None else qkv.unsqueeze(0),
+                    self.q_norm_weight if self.qk_norm else None, self.k_norm_weight if self.qk_norm else None, eps, self.position.angles(ctx), cache.writes, cache.k_cache, cache.v_cache, attn, step, ctx.batch,
                     H, self.scale, self.window, ctx.scratch)
                 self.out(attn, residual, accumulate=True, ctx=ctx)
                 return
