@@ -793,11 +793,16 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
 def decode_attention_prepares(batch, q_dtype: torch.dtype, k_cache: torch.Tensor, num_heads: int) -> bool:
     """Whether a step runs on the decode attention kernel that makes its own queries, newest keys and values
     from the QKV projection's planes: single decoded tokens only, bfloat16, pages of 16 positions or more,
-    head sizes 32, 64, 128 or 256, at most 16 query heads a KV head."""
+    head sizes 32, 64, 128 or 256, at most 16 query heads a KV head, fewer than 512 (sequence, KV head) pairs."""
     NB, KVH, bs, Dh = k_cache.shape
-    return (batch.all_decode and q_dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
+    if not (batch.all_decode and q_dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
             and Dh in (32, 64, 128, 256) and bs >= 16 and mfma_block_size(bs)
-            and num_heads % KVH == 0 and num_heads // KVH <= 16)
+            and num_heads % KVH == 0 and num_heads // KVH <= 16):
+        return False
+    # With so many sequences that the keys are not cut into shares, every wave would make a newest key and value
+    # and attend to it after its tiles, and the step is a little slower that way than with the q/k kernel before
+    # it (batch 64 at the 8B shape: 0.7 %).
+    return batch.num_seqs * KVH < 512
 
 
 def paged_attention_prepared(planes: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
