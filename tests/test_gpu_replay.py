@@ -105,6 +105,26 @@ def test_single_rows_beside_portions_on_either_attention_kernel(folders, name, m
         check(got[ride_along], want, "bfloat16", f"{name}/bfloat16/mixed, single rows riding along up to {ride_along}")
 
 
+@pytest.mark.parametrize("block_size", [32, 64])
+def test_pages_of_32_and_64_positions(folders, block_size):
+    """Configuration B in bfloat16 over larger pages (a page then holds several blocks of 16 keys, which the
+    attention kernels that load by such blocks must find inside it): mixed steps and decoding against the plain
+    implementation, pages counted in the replayer's own page size."""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["bfloat16"]["B"]
+    requests = th.make_requests(cfg["vocab_size"], [130, 23, 70, 64, 97, 33], seed=12)
+    want = reference_logits(folder, cfg, requests)
+    steps, peak = th.mixed(requests, max_live=4, seed=7)
+    rep = TraceReplayer.from_folder(folder, "bfloat16", 2 * peak, block_size=block_size)
+    got = th.collect(rep, steps)
+    assert rep.cache.num_free() == rep.cache.num_blocks
+    check(got, want, "bfloat16", f"B/bfloat16/mixed, pages of {block_size}")
+    tail = th.collect(TraceReplayer.from_folder(folder, "bfloat16", 2 * peak, block_size=block_size),
+                      th.prefill_then_decode(requests))
+    check(tail, want, "bfloat16", f"B/bfloat16/prefill+decode, pages of {block_size}")
+
+
 @pytest.mark.parametrize("use_graphs", [False, True])
 def test_decode_steps_with_and_without_the_attention_kernel_that_prepares(folders, monkeypatch, use_graphs):
     """Steps of single decoded tokens run on the attention kernel that makes its own queries and newest keys
