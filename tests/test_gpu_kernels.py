@@ -926,6 +926,108 @@ def test_argmax_and_sample_kernels():
     assert (drawn.cpu().long() == want).float().mean() > 0.999
 
 
+@pytest.mark.parametrize("vocab", [7, 1537, 50257, 151936])
+def test_temperature_sampling_kernel_draws_what_the_host_rule_draws(vocab):
+    """The walk in index order, against ``sample`` with the same uniform numbers: vocabularies that are no
+    multiple of the kernel's pieces of 256 (and rows that start off 16 bytes), -inf logits, temperatures; the
+    odd rows; only the rows listed, with the maxima given."""
+    import numpy as np
+    from tie_amd import kernels
+    from tie_amd.sampling import RandomStream, SamplingParams, sample
+
+    g = torch.Generator().manual_seed(vocab)
+    temperatures = [1.0, 0.5, 3.0, 0.05, 1.0, 0.8]
+    R = len(temperatures)
+    logits = torch.randn(R, vocab, generator=g) * 3
+    logits[4, torch.randperm(vocab, generator=g)[:vocab // 2]] = float("-inf")
+    logits[5, -1] = logits[5].max() + 3                       # most of the weight on the row's last logit
+    dev = logits.cuda()
+    inv_t = torch.tensor([float(np.float32(1.0) / np.float32(t)) for t in temperatures], device="cuda")
+    streams, host_streams = [RandomStream(i) for i in range(R)], [RandomStream(i) for i in range(R)]
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    host = logits.numpy()
+    for d in range(40):
+        uniform = torch.tensor([s.unit() for s in streams], dtype=torch.float64).cuda()
+        kernels.sample_rows(dev, inv_t, uniform, out)
+        want = [sample(host[i], SamplingParams(temperature=temperatures[i]), host_streams[i]) for i in range(R)]
+        assert out.tolist() == want, f"draw {d}"
+    listed = torch.tensor([4, 1], dtype=torch.int32, device="cuda")
+    again = torch.full((R,), -7, dtype=torch.int32, device="cuda")
+    kernels.sample_rows(dev, inv_t, uniform, again, listed, dev.max(dim=1).values.contiguous())
+    assert again.tolist() == [-7, want[1], -7, -7, want[4], -7]
+    odd = torch.randn(3, vocab, generator=g)
+    odd[0, vocab // 2] = float("nan")
+    odd[1] = float("-inf")
+    odd[2, 5] = odd[2, 2] = float("inf")
+    three = torch.empty(3, dtype=torch.int32, device="cuda")
+    kernels.sample_rows(odd.cuda(), inv_t[:3].contiguous(), uniform[:3].contiguous(), three)
+    assert three.tolist() == [-1, -2, 2]
+
+
+@pytest.mark.parametrize("vocab", [1000, 151936])
+def test_sampling_kernel_with_top_k_and_top_p_draws_what_the_host_rule_draws(vocab):
+    """The kernel that selects instead of sorting, against ``sample`` (sort, sums in double precision), draw by
+    draw with the same uniform numbers: every combination of top-k and top-p, logits with many exact ties (steps
+    of 0.25, so that the k-th value and the top-p boundary fall among equals and the ids decide), -inf logits,
+    a tiny temperature, all logits equal. Rows not listed keep what the output held."""
+    import numpy as np
+    from tie_amd import kernels
+    from tie_amd.sampling import RandomStream, SamplingParams, sample
+
+    g = torch.Generator().manual_seed(vocab)
+    smooth = torch.randn(vocab, generator=g) * 3
+    stepped = (torch.randn(vocab, generator=g) * 2 / 0.25).round() * 0.25
+    holes = smooth.clone()
+    holes[torch.randperm(vocab, generator=g)[:vocab // 3]] = float("-inf")
+    flat = torch.full((vocab,), 1.5)
+    cases = []
+    for name, row in (("smooth", smooth), ("stepped", stepped), ("holes", holes), ("flat", flat)):
+        for temperature in (1.0, 0.6, 2.5, 1e-3):
+            for top_k in (0, 1, 7, 50, vocab - 1, vocab + 5):
+                for top_p in (1.0, 0.95, 0.5, 0.02):
+                    if top_k in (0, vocab + 5) and top_p == 1.0:
+                        continue
+                    cases.append((name, row, temperature, top_k, top_p))
+    cases, draws = (cases[::7], 4) if vocab > 10000 else (cases, 6)     # the host rule sorts every large row: fewer of them
+    R = len(cases)
+    logits = torch.stack([c[1] for c in cases]).cuda()
+    inv_t = torch.tensor([float(np.float32(1.0) / np.float32(c[2])) for c in cases], device="cuda")
+    top_k = torch.tensor([c[3] for c in cases], dtype=torch.int32, device="cuda")
+    top_p = torch.tensor([c[4] for c in cases], dtype=torch.float32, device="cuda")
+    streams = [RandomStream(i) for i in range(R)]
+    host_streams = [RandomStream(i) for i in range(R)]
+    host_rows = {name: row.numpy() for name, row, *_ in cases}
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    for d in range(draws):
+        uniform = torch.tensor([s.unit() for s in streams], dtype=torch.float64).cuda()
+        out.fill_(-7)
+        kernels.sample_rows_filtered(logits, inv_t, uniform, top_k, top_p, out)
+        got = out.tolist()
+        for i, (name, _, temperature, k, p) in enumerate(cases):
+            want = sample(host_rows[name], SamplingParams(temperature=temperature, top_k=k, top_p=p), host_streams[i])
+            assert got[i] == want, f"{name} T={temperature} top_k={k} top_p={p} draw {d}: {got[i]} != {want}"
+    # only the rows listed
+    listed = torch.tensor([3, 0, R - 1], dtype=torch.int32, device="cuda")
+    again = torch.full((R,), -7, dtype=torch.int32, device="cuda")
+    kernels.sample_rows_filtered(logits, inv_t, uniform, top_k, top_p, again, listed)
+    again = again.tolist()
+    assert [again[i] for i in (3, 0, R - 1)] == [got[i] for i in (3, 0, R - 1)]
+    # the maxima given by the caller (the sampler has them from the argmax kernel)
+    given = torch.empty(R, dtype=torch.int32, device="cuda")
+    kernels.sample_rows_filtered(logits, inv_t, uniform, top_k, top_p, given, row_max=logits.max(dim=1).values.contiguous())
+    assert given.tolist() == got
+    assert all(t == -7 for i, t in enumerate(again) if i not in (3, 0, R - 1))
+    # a NaN and a row of -inf are reported, a +inf logit wins
+    odd = torch.randn(3, vocab, generator=g)
+    odd[0, 11] = float("nan")
+    odd[1] = float("-inf")
+    odd[2, 40] = odd[2, 90] = float("inf")
+    three = torch.empty(3, dtype=torch.int32, device="cuda")
+    kernels.sample_rows_filtered(odd.cuda(), inv_t[:3].contiguous(), uniform[:3].contiguous(), top_k[:3].contiguous(),
+                                 top_p[:3].contiguous(), three)
+    assert three.tolist() == [-1, -2, 40]
+
+
 def test_kernels_refuse_what_they_cannot_take():
     from tie_amd import kernels
     from tie_amd.errors import InvalidArgument, KernelUnavailable

@@ -680,91 +680,156 @@ extern "C" int tie_argmax_static(const float* logits, int* out, float* max_out, 
 // first index at which the running remainder turns negative
 // (src/sampling/sampler.cpp:35-39,56-60,75-80 without top-k / top-p).
 // out[r] = -1 for a row with a NaN, -2 for a row that is all -inf; a +inf logit wins outright.
+//
+// One workgroup a row, one pass for the sums: the waves own consecutive stretches of the row and read them in
+// pieces of 256 logits (four in a row per lane, so the loads are whole lines); the sum of every piece goes to
+// LDS. One thread then finds the piece in which u * total falls, walking the waves' sums and then that wave's
+// pieces in index order, and a wave reads this one piece again and finds the lane and the logit.
 #define SAMPLE_THREADS 1024
-__global__ void sample_kernel(const float* __restrict__ logits, const float* __restrict__ inv_temperature,
-                              const double* __restrict__ uniform, int* __restrict__ out, int V) {
+#define SAMPLE_WAVES (SAMPLE_THREADS / TIE_WAVE)
+#define SAMPLE_PIECE (4 * TIE_WAVE)
+#define SAMPLE_MAX_PIECES 4096          // rows of up to 2^20 logits
+
+__device__ __forceinline__ double sample_wave_sum(double v) {
+  for (int d = TIE_WAVE / 2; d > 0; d >>= 1) v += __shfl_xor(v, d);
+  return v;
+}
+
+// Four logits from index i on; beyond the row -inf, which weighs nothing.
+__device__ __forceinline__ float4 sample_load4(const float* row, int i, int V, bool by_four) {
+  if (by_four && i + 3 < V) return *reinterpret_cast<const float4*>(row + i);
+  float4 v;
+  v.x = i < V ? row[i] : -INFINITY;
+  v.y = i + 1 < V ? row[i + 1] : -INFINITY;
+  v.z = i + 2 < V ? row[i + 2] : -INFINITY;
+  v.w = i + 3 < V ? row[i + 3] : -INFINITY;
+  return v;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits,
+                                                                const float* __restrict__ row_max,
+                                                                const float* __restrict__ inv_temperature,
+                                                                const double* __restrict__ uniform,
+                                                                const int* __restrict__ rows, int* __restrict__ out,
+                                                                int V) {
   __shared__ float fscratch[16];
-  __shared__ double sums[SAMPLE_THREADS];
-  __shared__ int flag_nan;
-  __shared__ int chosen;
-  const int r = blockIdx.x;
-  const int tid = threadIdx.x;
+  __shared__ double piece_sums[SAMPLE_MAX_PIECES];
+  __shared__ double wave_sums[SAMPLE_WAVES];
+  __shared__ double remainder;
+  __shared__ int flag_nan, chosen, owner_piece;
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & (TIE_WAVE - 1), wave = tid / TIE_WAVE;
   const float* row = logits + static_cast<size_t>(r) * V;
-  if (tid == 0) {
-    flag_nan = 0;
-    chosen = V;
-  }
-  __syncthreads();
-  float mx = -INFINITY;
-  bool nan = false;
-  for (int i = tid; i < V; i += SAMPLE_THREADS) {
-    const float v = row[i];
-    nan |= (v != v);
-    mx = fmaxf(mx, v);
-  }
-  if (nan) flag_nan = 1;
-  mx = block_max(mx, fscratch);
-  __syncthreads();
-  if (flag_nan) {
-    if (tid == 0) out[r] = -1;
-    return;
-  }
-  if (mx == -INFINITY) {
-    if (tid == 0) out[r] = -2;
-    return;
+  const bool by_four = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  const int pieces = (V + SAMPLE_PIECE - 1) / SAMPLE_PIECE;
+  const int per_wave = (pieces + SAMPLE_WAVES - 1) / SAMPLE_WAVES;
+  const int first_piece = wave * per_wave;
+  float mx;
+  if (row_max) {
+    mx = row_max[r];         // the caller has looked at the row: no NaN, a finite maximum
+  } else {
+    if (tid == 0) {
+      flag_nan = 0;
+      chosen = V;
+    }
+    __syncthreads();
+    mx = -INFINITY;
+    bool nan = false;
+    for (int i = tid; i < V; i += SAMPLE_THREADS) {
+      const float v = row[i];
+      nan |= (v != v);
+      mx = fmaxf(mx, v);
+    }
+    if (nan) flag_nan = 1;
+    mx = block_max(mx, fscratch);
+    __syncthreads();
+    if (flag_nan || mx == -INFINITY) {
+      if (tid == 0) out[r] = flag_nan ? -1 : -2;
+      return;
+    }
+    if (mx == INFINITY) {  // the lowest +inf index wins without a draw
+      int first = V;
+      for (int i = tid; i < V; i += SAMPLE_THREADS)
+        if (row[i] == INFINITY) first = min(first, i);
+      if (first < V) atomicMin(&chosen, first);
+      __syncthreads();
+      if (tid == 0) out[r] = chosen;
+      return;
+    }
   }
   const float inv_t = inv_temperature[r];
-  // Each thread owns one contiguous segment so that the walk is in index order.
-  const int seg = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int begin = min(tid * seg, V);
-  const int end = min(begin + seg, V);
-  if (mx == INFINITY) {  // the lowest +inf index wins without a draw
-    int first = V;
-    for (int i = begin; i < end; ++i) {
-      if (row[i] == INFINITY) {
-        first = i;
-        break;
-      }
+  double of_wave = 0.0;
+  for (int p0 = 0; p0 < per_wave; p0 += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = sample_load4(row, (first_piece + p0 + u) * SAMPLE_PIECE + 4 * lane, V, by_four);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (p0 + u >= per_wave || first_piece + p0 + u >= pieces) break;
+      double mine = static_cast<double>(expf((v[u].x - mx) * inv_t));
+      mine += static_cast<double>(expf((v[u].y - mx) * inv_t));
+      mine += static_cast<double>(expf((v[u].z - mx) * inv_t));
+      mine += static_cast<double>(expf((v[u].w - mx) * inv_t));
+      const double piece = sample_wave_sum(mine);
+      if (lane == 0) piece_sums[first_piece + p0 + u] = piece;
+      of_wave += piece;
     }
-    if (first < V) atomicMin(&chosen, first);
-    __syncthreads();
-    if (tid == 0) out[r] = chosen;
-    return;
   }
-  double local = 0.0;
-  for (int i = begin; i < end; ++i) local += static_cast<double>(expf((row[i] - mx) * inv_t));
-  sums[tid] = local;
+  if (lane == 0) wave_sums[wave] = of_wave;
   __syncthreads();
   if (tid == 0) {
     double total = 0.0;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) total += sums[i];
+    for (int w = 0; w < SAMPLE_WAVES; ++w) total += wave_sums[w];
     double rem = uniform[r] * total;
-    int owner = SAMPLE_THREADS - 1;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) {
-      if (rem - sums[i] < 0.0) {
-        owner = i;
-        break;
-      }
-      rem -= sums[i];
+    int w = 0;
+    for (; w < SAMPLE_WAVES - 1; ++w) {
+      if (rem - wave_sums[w] < 0.0) break;
+      rem -= wave_sums[w];
     }
-    // Walk the owner's segment; fall back to the last index with weight if rounding leaves a remainder.
-    const int b = min(owner * seg, V), e = min(b + seg, V);
-    int pick = -1;
-    for (int i = b; i < e; ++i) {
-      rem -= static_cast<double>(expf((row[i] - mx) * inv_t));
-      if (rem < 0.0) {
-        pick = i;
-        break;
-      }
+    int p = w * per_wave;
+    const int last = min(p + per_wave, pieces) - 1;
+    if (p > last) p = pieces - 1;         // rounding left a remainder beyond the last piece with logits
+    for (; p < last; ++p) {
+      if (rem - piece_sums[p] < 0.0) break;
+      rem -= piece_sums[p];
     }
-    if (pick < 0) pick = V - 1;
-    out[r] = pick;
+    owner_piece = p;
+    remainder = rem;
   }
+  __syncthreads();
+  if (wave != 0) return;
+  const int base = owner_piece * SAMPLE_PIECE + 4 * lane;
+  const float4 v = sample_load4(row, base, V, by_four);
+  const double w0 = static_cast<double>(expf((v.x - mx) * inv_t)), w1 = static_cast<double>(expf((v.y - mx) * inv_t));
+  const double w2 = static_cast<double>(expf((v.z - mx) * inv_t)), w3 = static_cast<double>(expf((v.w - mx) * inv_t));
+  const double mine = ((w0 + w1) + w2) + w3;
+  double upto = mine;                     // of this lane and the lanes before it
+  for (int d = 1; d < TIE_WAVE; d <<= 1) {
+    const double other = __shfl_up(upto, d);
+    if (lane >= d) upto += other;
+  }
+  const unsigned long long reached = __ballot(remainder - upto < 0.0);
+  // Rounding may leave a remainder: then the last logit of the piece, as the walk would end at the row's last.
+  int pick = min(owner_piece * SAMPLE_PIECE + SAMPLE_PIECE, V) - 1;
+  const int who = reached ? __ffsll(reached) - 1 : -1;
+  if (lane == who) {
+    double rem = remainder - (upto - mine);
+    pick = base + 3;
+    if ((rem -= w0) < 0.0) pick = base;
+    else if ((rem -= w1) < 0.0) pick = base + 1;
+    else if ((rem -= w2) < 0.0) pick = base + 2;
+    pick = min(pick, V - 1);
+  }
+  if (who < 0 ? lane == 0 : lane == who) out[r] = pick;
 }
 
-extern "C" int tie_sample(const float* logits, const float* inv_temperature, const double* uniform, int* out,
-                          int R, int V, hipStream_t stream) {
-  if (R <= 0 || V <= 0) return TIE_BAD_ARGUMENT;
-  sample_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, inv_temperature, uniform, out, V);
+// With `rows` only the `num_rows` rows it lists are drawn, and out[] of the others is left as it is. With `row_max`
+// (the rows' maxima, which the caller has found finite, in rows without a NaN) the kernel does not look for them.
+extern "C" int tie_sample(const float* logits, const float* row_max, const float* inv_temperature, const double* uniform,
+                          const int* rows, int num_rows, int* out, int R, int V, hipStream_t stream) {
+  if (R <= 0 || V <= 0 || (rows && (num_rows <= 0 || num_rows > R))) return TIE_BAD_ARGUMENT;
+  if (V > SAMPLE_MAX_PIECES * SAMPLE_PIECE) return TIE_BAD_ARGUMENT;
+  sample_kernel<<<rows ? num_rows : R, SAMPLE_THREADS, 0, stream>>>(logits, row_max, inv_temperature, uniform, rows, out,
+                                                                    V);
   return tie_launch_status();
 }

@@ -29,6 +29,7 @@ _SOURCES = {
     "attention_generic": ("tie_attention_generic", "attention_generic.hip"),
     "skinny_gemm_bf16": ("tie_skinny_gemm_bf16", "skinny_gemm_bf16.hip"),
     "gemm_bf16": ("tie_gemm_bf16", "gemm_bf16.hip"),
+    "sample_filtered": ("tie_sample_filtered", "sample_filtered.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -41,6 +42,10 @@ MAX_HEAD_DIM = 512        # the largest head size any attention kernel takes (th
 MAX_STEP_TOKENS = 65535   # rows of one step: a grid dimension of the row-wise kernels
 
 _SIGNATURES = {
+    "sample_filtered": {
+        "tie_sample_filtered": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int,
+                                _c_int, _c_void],
+    },
     "elementwise": {
         "tie_embed": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
@@ -54,7 +59,7 @@ _SIGNATURES = {
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
                                       _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
-        "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_argmax_static": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
@@ -685,18 +690,74 @@ def argmax_rows_static(logits: torch.Tensor, out: torch.Tensor, max_out: Optiona
                                                      _stream())
 
 
-def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
-                out: torch.Tensor) -> None:
-    """Draws one token per row from softmax(logits * inv_temperature) with the given uniform numbers."""
+MAX_SAMPLED_VOCAB = 1 << 20      # rows the temperature sampling kernel takes (the sums of its pieces fit LDS)
+
+
+def _row_selection(rows: Optional[torch.Tensor], row_max: Optional[torch.Tensor], R: int) -> int:
+    count = 0
+    if rows is not None:
+        _i32(rows, "row numbers")
+        count = rows.numel()
+        if not 0 < count <= R:
+            raise InvalidArgument(f"{count} row numbers for {R} rows")
+    if row_max is not None:
+        _f32(row_max, "row maxima", (R,))
+    return count
+
+
+def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor,
+                rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None) -> None:
+    """Draws one token per row from softmax(logits * inv_temperature) with the given uniform numbers, walking the
+    tokens in index order. ``out[r]`` is -1 for a row with a NaN and -2 for a row that is all -inf. With ``rows``
+    (int32 row numbers) only those rows are drawn; the other entries of ``out`` stay as they are. With ``row_max``
+    (the rows' maxima, which the caller has found to be finite, in rows without a NaN) the kernel does not look
+    for them."""
     _f32(logits, "logits")
+    if logits.dim() != 2:
+        raise InvalidArgument("logits must be [rows, vocabulary]")
     R, V = logits.shape
+    if V > MAX_SAMPLED_VOCAB:
+        raise InvalidArgument(f"the sampling kernel takes rows of up to {MAX_SAMPLED_VOCAB} logits, got {V}")
     _f32(inv_temperature, "inverse temperatures", (R,))
     _gpu(uniform, "uniform numbers")
     if uniform.dtype != torch.float64 or uniform.numel() != R:
         raise InvalidArgument("uniform numbers must be float64, one per row")
     _i32(out, "sample output", R)
-    _call(_lib("elementwise").tie_sample, "sample", logits.data_ptr(), inv_temperature.data_ptr(), uniform.data_ptr(),
-                                          out.data_ptr(), R, V, _stream())
+    count = _row_selection(rows, row_max, R)
+    _call(_lib("elementwise").tie_sample, "sample", logits.data_ptr(), _ptr(row_max), inv_temperature.data_ptr(),
+          uniform.data_ptr(), _ptr(rows), count, out.data_ptr(), R, V, _stream())
+
+
+MAX_FILTERED_VOCAB = 1 << 19     # rows the top-k / top-p sampling kernel takes (its integer sums fit 64 bits)
+
+
+def sample_rows_filtered(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
+                         top_k: torch.Tensor, top_p: torch.Tensor, out: torch.Tensor,
+                         rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None) -> None:
+    """Draws one token per row with top-k and top-p: ``top_k[r]`` most likely kept (0: all), then the smallest
+    prefix by likelihood whose weight reaches ``top_p[r]`` of the total (1: all), one uniform number a row, which
+    walks the candidates in the order of likelihood also where neither filter removes any (``sample_rows`` walks
+    them in index order, as the rule is without filters).
+    ``out[r]`` is -1 for a row with a NaN and -2 for a row that is all -inf. With ``rows`` (int32 row numbers)
+    only those rows are drawn; the other entries of ``out`` stay as they are. With ``row_max`` (the rows' maxima,
+    which the caller has found to be finite, in rows without a NaN) the kernel does not look for them."""
+    _f32(logits, "logits")
+    if logits.dim() != 2:
+        raise InvalidArgument("logits must be [rows, vocabulary]")
+    R, V = logits.shape
+    if V > MAX_FILTERED_VOCAB:
+        raise InvalidArgument(f"the top-k / top-p kernel takes rows of up to {MAX_FILTERED_VOCAB} logits, got {V}")
+    _f32(inv_temperature, "inverse temperatures", (R,))
+    _f32(top_p, "top_p", (R,))
+    _i32(top_k, "top_k", R)
+    _gpu(uniform, "uniform numbers")
+    if uniform.dtype != torch.float64 or uniform.numel() != R:
+        raise InvalidArgument("uniform numbers must be float64, one per row")
+    _i32(out, "sample output", R)
+    count = _row_selection(rows, row_max, R)
+    _call(_lib("sample_filtered").tie_sample_filtered, "sample_filtered", logits.data_ptr(), _ptr(row_max),
+          inv_temperature.data_ptr(), uniform.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), _ptr(rows), count,
+          out.data_ptr(), R, V, _stream())
 
 
 # Up to this many workgroups of single decoded rows run in the prefill attention kernel beside a step's prompt

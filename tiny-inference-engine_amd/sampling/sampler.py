@@ -11,9 +11,11 @@ The rules are the reference's (``src/sampling/sampler.cpp:18-81``):
   smallest prefix whose weight reaches ``top_p * total`` kept, one uniform draw in [0, total) and a
   walk over the kept candidates.
 
-``sample`` works on the host from a float32 row. ``DeviceSampler`` handles whole steps: greedy rows
-and plain temperature rows are drawn by GPU kernels (only the token ids come back, and the uniform
-numbers still come from each request's own stream); rows with top-k or top-p go through ``sample``.
+``sample`` works on the host from a float32 row: it is the rule written out, for single rows and for checking.
+``DeviceSampler`` handles whole steps on the GPU: greedy rows, plain temperature rows and rows with top-k or
+top-p each have a kernel; only the token ids come back, and the uniform numbers still come from each request's
+own stream. The top-k / top-p kernel sums its weights as integers in units of 2^-44 of the largest, where
+``sample`` sums in double precision: the two differ only for a draw within 1e-8 of a boundary.
 """
 
 from __future__ import annotations
@@ -92,7 +94,7 @@ class DeviceSampler:
     into asking and reading, so that a caller may queue the next step (whose tokens it takes from
     ``ticket.device_tokens``) before it reads this one's; two sets of buffers alternate for that."""
 
-    GREEDY, PLAIN, HOST = 0, 1, 2      # argmax kernel / temperature kernel / top-k or top-p on the host
+    GREEDY, PLAIN, FILTERED = 0, 1, 2      # argmax kernel / temperature kernel / top-k and top-p kernel
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -101,10 +103,11 @@ class DeviceSampler:
         self._turn = 0
 
     def _buffers(self, rows: int):
+        """Device words and pinned host words: 3 R of results (argmax, maxima, draws), then 6 R of parameters."""
         if rows > self._rows:
             self._rows = max(64, 2 * rows)
-            self._sets = [(torch.empty(3 * self._rows, dtype=torch.int32, device=self.device),
-                           torch.empty(3 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
+            self._sets = [(torch.empty(9 * self._rows, dtype=torch.int32, device=self.device),
+                           torch.empty(9 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
                           for _ in range(2)]
         self._turn ^= 1
         return self._sets[self._turn]
@@ -151,35 +154,56 @@ class DeviceSampler:
         R = logits.shape[0]
         if R != len(params) or R != len(rngs):
             raise InvalidArgument("one set of sampling parameters and one random stream per row")
-        kinds = np.fromiter((self.GREEDY if p.greedy else (self.PLAIN if p.top_k == 0 and p.top_p >= 1.0 else self.HOST)
+        V = logits.shape[1]
+        # Without a filter the reference walks the candidates in index order, with one in the order of likelihood
+        # (src/sampling/sampler.cpp:41-54): the same uniform number picks different tokens, so each has its kernel.
+        kinds = np.fromiter((self.GREEDY if p.greedy else (self.FILTERED if 0 < p.top_k < V or p.top_p < 1.0 else self.PLAIN)
                              for p in params), dtype=np.int8, count=R)
         if not kinds.any():
             return self.collect(self.launch_greedy(logits))
-        out = np.zeros(R, dtype=np.int64)
-        on_device = kinds != self.HOST
-        if on_device.any():
-            # Both kernels work on all rows at once; each kind's result is read where it applies. Index and
-            # maximum lie side by side, so one copy brings both.
-            dev, host = self._buffers(R)
-            kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
-            fetched = self._fetch(dev, host, 2 * R)
-            best, top = fetched[:R], fetched[R:].view(np.float32)
-            if (best[on_device] < 0).any():
-                raise InvalidArgument(f"a logit of row {int(np.flatnonzero(on_device & (best < 0))[0])} is NaN")
-            if (top[on_device] == -np.inf).any():
-                raise InvalidArgument(f"all logits of row {int(np.flatnonzero(on_device & (top == -np.inf))[0])} are -inf")
-            out[on_device] = best[on_device]
-            # A +inf logit is certain and consumes no random number; every other temperature row draws one.
-            drawing = np.flatnonzero((kinds == self.PLAIN) & (top != np.inf))
-            if drawing.size:
-                inv_t = np.ones(R, dtype=np.float32)
-                uniform = np.zeros(R, dtype=np.float64)
-                for i in drawing:
-                    inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
-                    uniform[i] = rngs[i].unit()
-                kernels.sample_rows(logits, torch.from_numpy(inv_t).to(logits.device),
-                                    torch.from_numpy(uniform).to(logits.device), dev[2 * R:3 * R])
-                out[drawing] = self._fetch(dev[2 * R:], host[2 * R:], R)[drawing]
-        for i in np.flatnonzero(kinds == self.HOST):
-            out[i] = sample(logits[i].cpu().numpy(), params[i], rngs[i])
+        # The argmax kernel works on all rows: it answers the greedy rows, finds NaN and all -inf rows, and a
+        # +inf logit, which is certain and consumes no random number. Index and maximum lie side by side, so one
+        # copy brings both.
+        dev, host = self._buffers(R)
+        kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
+        fetched = self._fetch(dev, host, 2 * R)
+        best, top = fetched[:R], fetched[R:].view(np.float32)
+        if (best < 0).any():
+            raise InvalidArgument(f"a logit of row {int(np.flatnonzero(best < 0)[0])} is NaN")
+        if (top == -np.inf).any():
+            raise InvalidArgument(f"all logits of row {int(np.flatnonzero(top == -np.inf)[0])} are -inf")
+        out = best.astype(np.int64)
+        plain = np.flatnonzero((kinds == self.PLAIN) & (top != np.inf))
+        filtered = np.flatnonzero((kinds == self.FILTERED) & (top != np.inf))
+        if not plain.size and not filtered.size:
+            return out.tolist()
+        # The parameters of the drawing rows go up in one copy: 1 / temperature, top_p, top_k, the numbers of the
+        # drawing rows, those with a filter first (one word a row each), one uniform number a row (two words).
+        P = R + (R & 1)                                    # the float64 numbers start on 8 bytes
+        at = 3 * self._rows
+        words = host[at:at + 6 * P].numpy()
+        inv_t, top_p = words[:R].view(np.float32), words[P:P + R].view(np.float32)
+        top_k, rows, uniform = words[2 * P:2 * P + R], words[3 * P:3 * P + R], words[4 * P:6 * P].view(np.float64)[:R]
+        inv_t[:], top_p[:], top_k[:], uniform[:] = 1.0, 1.0, 0, 0.0
+        for i in np.concatenate([plain, filtered]):
+            inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
+            uniform[i] = rngs[i].unit()
+        for i in filtered:
+            top_p[i], top_k[i] = params[i].top_p, min(params[i].top_k, V)
+        rows[:filtered.size] = filtered
+        rows[filtered.size:filtered.size + plain.size] = plain
+        up = dev[at:at + 6 * P]
+        up.copy_(host[at:at + 6 * P], non_blocking=True)
+        d_inv_t, d_uniform = up[:R].view(torch.float32), up[4 * P:6 * P].view(torch.float64)[:R]
+        drawn = dev[2 * R:3 * R]
+        maxima = dev[R:2 * R].view(torch.float32)
+        if plain.size:
+            kernels.sample_rows(logits, d_inv_t, d_uniform, drawn,
+                                up[3 * P + filtered.size:3 * P + filtered.size + plain.size], maxima)
+        if filtered.size:
+            kernels.sample_rows_filtered(logits, d_inv_t, d_uniform, up[2 * P:2 * P + R], up[P:P + R].view(torch.float32),
+                                         drawn, up[3 * P:3 * P + filtered.size], maxima)
+        got = self._fetch(dev[2 * R:], host[2 * R:], R)
+        out[plain] = got[plain]
+        out[filtered] = got[filtered]
         return out.tolist()
