@@ -117,7 +117,7 @@ def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True):
                          max_seq_len=context, launch_ahead=launch_ahead)
 
 
-def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
+def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=None):
     """Times ``steps`` decode steps of ``batch`` sequences whose contexts end at (just below) ``context`` tokens.
 
     The prompts are prefilled through the engine first (untimed). Sequences that finish their prompt
@@ -137,7 +137,8 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk):
     prompt_len = context - (steps + warmup) - slack - 1
     assert prompt_len > 0, "context too short for this many steps"
     ids = [engine.add_request([rng.randrange(cfg["vocab_size"]) for _ in range(prompt_len)],
-                              SamplingParams(max_tokens=steps + warmup + slack + 1)) for _ in range(batch)]
+                              SamplingParams(max_tokens=steps + warmup + slack + 1, seed=i, **(sampling or {})))
+           for i in range(batch)]
     started = time.perf_counter()
     last_log = started
     while any(engine.sequence(i).state != SeqState.DECODING for i in ids):
@@ -209,6 +210,9 @@ def main():
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
     parser.add_argument("--kv-mem", type=int, default=2 << 30, help="stress: bytes of cache")
     parser.add_argument("--skip-points", action="store_true", help="skip batch 1, batch 64 and the prefill")
+    parser.add_argument("--temperature", type=float, default=0.0, help="decode: sampling temperature (0 = greedy)")
+    parser.add_argument("--top-k", type=int, default=0, help="decode: with a temperature, keep the k most likely (0 = all)")
+    parser.add_argument("--top-p", type=float, default=1.0, help="decode: with a temperature, nucleus mass (1 = all)")
     parser.add_argument("--prefill-only", action="store_true",
                         help="run only the 2048-token prefill (for profiling); prints its figures alone")
     args = parser.parse_args()
@@ -257,7 +261,11 @@ def main():
         return 0
 
     chunk = 8192
-    seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk)
+    sampling = None
+    if args.temperature > 0:
+        sampling = {"temperature": args.temperature, "top_k": args.top_k, "top_p": args.top_p}
+    seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk,
+                                                    sampling)
     ms_per_step = seconds / args.steps * 1e3
     value = args.batch * args.steps / seconds
     step_bytes = weight_bytes_per_step(cfg, args.batch) + args.batch * mean_context * kv_bytes_per_token(cfg)
@@ -274,7 +282,8 @@ def main():
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
             "global_batch": args.batch, "seq_len": args.context, "kv_block": BLOCK_SIZE, "kv_dtype": "bf16",
-            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU", "sampling": "greedy",
+            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
+            "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
@@ -288,7 +297,7 @@ def main():
             f"{flops / t / 1e12:.1f} TFLOP/s")
         points = {}
         for b in (1, 64):
-            s, _, _ = measure_decode(model, cfg, b, args.context, max(8, args.steps // 2), args.warmup, chunk)
+            s, _, _ = measure_decode(model, cfg, b, args.context, max(8, args.steps // 2), args.warmup, chunk, sampling)
             points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 2)
             log(f"decode batch {b}: {points[f'decode_b{b}']:.1f} tok/s")
         result["points"] = points

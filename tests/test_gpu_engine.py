@@ -361,13 +361,54 @@ def test_device_sampling_matches_the_host_sampler():
         sampler.sample_rows(bad, params, dev_rngs)
 
 
+def test_steps_queued_before_the_one_before_is_read_draw_the_same_tokens():
+    """``launch`` with the ticket of the step before, collected one step late, against the host rule row by row:
+    greedy, temperature and top-k / top-p rows side by side, over steps whose logits change, one of them with a
+    +inf logit in a drawing row - that row takes no number from its stream, which the next step, already
+    queued, can only know on the GPU."""
+    from tie_amd.sampling import DeviceSampler, RandomStream, SamplingParams, sample
+
+    g = torch.Generator().manual_seed(12)
+    steps = [(torch.randn(5, 3000, generator=g) * 3) for _ in range(12)]
+    steps[3][1, 77] = float("inf")           # a temperature row
+    steps[4][3, 5] = float("inf")            # a top-k / top-p row, in the step right after
+    steps[4][3, 2000] = float("inf")
+    steps[8][1, 9] = steps[8][3, 9] = float("inf")
+    steps[9][1, 9] = float("inf")            # twice in a row
+    params = [SamplingParams(), SamplingParams(temperature=0.9, seed=1), SamplingParams(temperature=0.7, top_k=40, seed=2),
+              SamplingParams(temperature=1.3, top_p=0.6, seed=3), SamplingParams(temperature=0.5, top_k=3000, seed=4)]
+    host_rngs = [RandomStream(p.seed) for p in params]
+    want = [[sample(step[i].numpy(), params[i], host_rngs[i]) for i in range(5)] for step in steps]
+    sampler = DeviceSampler("cuda:0")
+    rngs = [RandomStream(p.seed) for p in params]
+    got, waiting = [], None
+    for step in steps:
+        ticket = sampler.launch(step.cuda(), params, rngs, waiting)
+        if waiting is not None:
+            got.append(sampler.collect(waiting))
+        waiting = ticket
+    got.append(sampler.collect(waiting))
+    assert got == want
+    assert [r.unit() for r in rngs] == [r.unit() for r in host_rngs]        # the streams stand where the host's do
+    # read at once, as a step outside the steady state is
+    rngs = [RandomStream(p.seed) for p in params]
+    assert [sampler.sample_rows(step.cuda(), params, rngs) for step in steps] == want
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("kv_blocks", [256, 14])
-def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_folders_bf16, dtype, kv_blocks):
-    """Greedy requests with the next step queued before the last one's tokens are read, against the same engine
+@pytest.mark.parametrize("drawing", [False, True])
+def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_folders_bf16, dtype, kv_blocks, drawing):
+    """Requests with the next step queued before the last one's tokens are read, against the same engine
     reading every step at once: equal tokens, through stop tokens (a sequence then ran one token too many,
-    which must leave no trace), ends by length, a cancellation and, with 14 pages, evictions."""
+    which must leave no trace), ends by length, a cancellation and, with 14 pages, evictions. ``drawing``: the
+    requests sample, each in its own way (temperature, top-k, top-p, one greedy) from its own stream."""
     import tie_amd
+
+    ways = [dict(temperature=0.8, seed=3), dict(temperature=0.7, top_k=20, top_p=0.8, seed=4), dict(),
+            dict(temperature=1.4, top_p=0.9, seed=5), dict(temperature=0.6, top_k=5, seed=6), dict(temperature=1.0, seed=7)]
+    if not drawing:
+        ways = [dict()] * 6
 
     folder, cfg = (model_folders_bf16 if dtype == "bfloat16" else model_folders)["A"]
     vocab = cfg["vocab_size"]
@@ -379,7 +420,7 @@ def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_fold
                              launch_ahead=ahead, stop_tokens=stop_tokens)
         seen = []
         engine.on_token = lambda seq_id, token: seen.append((seq_id, token))
-        ids = [engine.add_request(p, tie_amd.SamplingParams(max_tokens=m)) for p, m in reqs]
+        ids = [engine.add_request(p, tie_amd.SamplingParams(max_tokens=m, **way)) for (p, m), way in zip(reqs, ways)]
         steps = 0
         while engine.has_work():
             engine.step()

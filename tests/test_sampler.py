@@ -132,3 +132,19 @@ def test_draw_for_draw_agreement_with_the_plain_sampler(top_k, top_p):
         p = SamplingParams(temperature=t, top_k=top_k, top_p=top_p)
         for _ in range(25):
             assert sample(logits, p, mine) == plain.sample(list(logits), t, top_k, top_p, theirs)
+
+
+def test_looking_ahead_in_the_stream_takes_nothing_from_it():
+    """``peek_unit`` shows what ``unit`` will return, any number of outputs ahead and across the generator's
+    refill (312 outputs), and ``skip`` moves on as ``unit`` does."""
+    a, b = RandomStream(9), RandomStream(9)
+    want = [b.unit() for _ in range(700)]
+    got = []
+    for i in range(0, 700, 7):
+        assert a.peek_unit(3) == want[i + 3] and a.peek_unit(0) == want[i] and a.peek_unit(1) == want[i + 1]
+        got.append(a.unit())
+        a.skip(2)
+        assert a.peek_unit() == want[i + 3]
+        got += [a.unit() for _ in range(4)]
+    assert got == [w for i, w in enumerate(want) if i % 7 not in (1, 2)]
+    assert a.uniform(0.0, 3.0) == b.uniform(0.0, 3.0)

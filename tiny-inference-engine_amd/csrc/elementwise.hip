@@ -710,6 +710,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
                                                                 const float* __restrict__ row_max,
                                                                 const float* __restrict__ inv_temperature,
                                                                 const double* __restrict__ uniform,
+                                                                const double* __restrict__ other_uniform,
+                                                                const int* __restrict__ take_other,
+                                                                int* __restrict__ drew_none,
                                                                 const int* __restrict__ rows, int* __restrict__ out,
                                                                 int V) {
   __shared__ float fscratch[16];
@@ -726,7 +729,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   const int first_piece = wave * per_wave;
   float mx;
   if (row_max) {
-    mx = row_max[r];         // the caller has looked at the row: no NaN, a finite maximum
+    // The caller looks at the maxima too: a row with a NaN or of -inf is its to report, and where the maximum
+    // is +inf the argmax stands; none of them draws.
+    mx = row_max[r];
+    if (tid == 0 && drew_none) drew_none[r] = !(mx > -INFINITY && mx < INFINITY);
+    if (!(mx > -INFINITY && mx < INFINITY)) return;
   } else {
     if (tid == 0) {
       flag_nan = 0;
@@ -743,6 +750,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (nan) flag_nan = 1;
     mx = block_max(mx, fscratch);
     __syncthreads();
+    if (tid == 0 && drew_none) drew_none[r] = !(mx > -INFINITY && mx < INFINITY) || flag_nan;
     if (flag_nan || mx == -INFINITY) {
       if (tid == 0) out[r] = flag_nan ? -1 : -2;
       return;
@@ -780,7 +788,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   if (tid == 0) {
     double total = 0.0;
     for (int w = 0; w < SAMPLE_WAVES; ++w) total += wave_sums[w];
-    double rem = uniform[r] * total;
+    double rem = (take_other && take_other[r] ? other_uniform[r] : uniform[r]) * total;
     int w = 0;
     for (; w < SAMPLE_WAVES - 1; ++w) {
       if (rem - wave_sums[w] < 0.0) break;
@@ -824,12 +832,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
 }
 
 // With `rows` only the `num_rows` rows it lists are drawn, and out[] of the others is left as it is. With `row_max`
-// (the rows' maxima, which the caller has found finite, in rows without a NaN) the kernel does not look for them.
+// (the rows' maxima) the kernel does not look for them, and leaves out[] of a row whose maximum is not finite as
+// it is. `drew_none` (optional): 1 for a row that took no uniform number (no finite maximum), else 0.
+// `take_other` (optional): where it is not 0 the row's number is other_uniform[r]; a caller that queues a step
+// before it has read the one before passes that step's `drew_none` here, and both numbers the row's stream may
+// be at.
 extern "C" int tie_sample(const float* logits, const float* row_max, const float* inv_temperature, const double* uniform,
-                          const int* rows, int num_rows, int* out, int R, int V, hipStream_t stream) {
+                          const double* other_uniform, const int* take_other, int* drew_none, const int* rows,
+                          int num_rows, int* out, int R, int V, hipStream_t stream) {
   if (R <= 0 || V <= 0 || (rows && (num_rows <= 0 || num_rows > R))) return TIE_BAD_ARGUMENT;
-  if (V > SAMPLE_MAX_PIECES * SAMPLE_PIECE) return TIE_BAD_ARGUMENT;
-  sample_kernel<<<rows ? num_rows : R, SAMPLE_THREADS, 0, stream>>>(logits, row_max, inv_temperature, uniform, rows, out,
-                                                                    V);
+  if (V > SAMPLE_MAX_PIECES * SAMPLE_PIECE || (take_other && !other_uniform)) return TIE_BAD_ARGUMENT;
+  sample_kernel<<<rows ? num_rows : R, SAMPLE_THREADS, 0, stream>>>(logits, row_max, inv_temperature, uniform,
+                                                                    other_uniform, take_other, drew_none, rows, out, V);
   return tie_launch_status();
 }

@@ -246,6 +246,9 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
                                                                      const float* __restrict__ row_max,
                                                                      const float* __restrict__ inv_temperature,
                                                                      const double* __restrict__ uniform,
+                                                                     const double* __restrict__ other_uniform,
+                                                                     const int* __restrict__ take_other,
+                                                                     int* __restrict__ drew_none,
                                                                      const int* __restrict__ top_k,
                                                                      const float* __restrict__ top_p,
                                                                      const int* __restrict__ rows,
@@ -263,7 +266,13 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
   r.mx = 0.f;
   r.inv_t = 1.f;
   if (row_max) {
-    r.mx = row_max[rix];       // the caller has looked at the row: no NaN, a finite maximum
+    // The caller looks at the maxima too: a row with a NaN or of -inf is its to report, and where the maximum
+    // is +inf the argmax stands; none of them draws.
+    r.mx = row_max[rix];
+    if (!(r.mx > -INFINITY && r.mx < INFINITY)) {
+      if (tid == 0 && drew_none) drew_none[rix] = 1;
+      return;
+    }
   } else {
     if (tid == 0) {
       flag_nan = 0;
@@ -280,6 +289,7 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
     if (nan) flag_nan = 1;
     mx = block_max(mx, fscratch);
     __syncthreads();
+    if (tid == 0 && drew_none) drew_none[rix] = !(mx > -INFINITY && mx < INFINITY) || flag_nan;
     if (flag_nan || mx == -INFINITY) {
       if (tid == 0) out[rix] = flag_nan ? -1 : -2;
       return;
@@ -297,6 +307,7 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
     r.mx = mx;
   }
   r.inv_t = inv_temperature[rix];
+  if (row_max && tid == 0 && drew_none) drew_none[rix] = 0;
 
   SfCandidates cand;
   cand.limit = ~0ull;
@@ -322,19 +333,26 @@ __global__ __launch_bounds__(SF_THREADS) void sample_filtered_kernel(const float
     }
   }
   sf_u64 drawn;
-  sf_search<false>(r, cand, SF_DRAW, uniform[rix], hist, list, &list_n, shared, &drawn, &sum);
+  const double u = take_other && take_other[rix] ? other_uniform[rix] : uniform[rix];
+  sf_search<false>(r, cand, SF_DRAW, u, hist, list, &list_n, shared, &drawn, &sum);
   if (tid == 0) out[rix] = static_cast<int>(drawn & ((1u << SF_ID_BITS) - 1));
 }
 
 // top_k[r] <= 0 or >= V: no top-k; top_p[r] >= 1: no top-p. uniform[r] in [0, 1). The arrays have an entry for
 // each of the R rows of `logits`; with `rows` only the `num_rows` rows it lists are drawn, and out[] of the
-// others is left as it is. With `row_max` (the rows' maxima, which the caller has found finite, in rows without
-// a NaN) the kernel does not look for them.
+// others is left as it is. With `row_max` (the rows' maxima) the kernel does not look for them, and leaves out[]
+// of a row whose maximum is not finite as it is. `drew_none` (optional): 1 for a row that took no uniform number
+// (no finite maximum), else 0. `take_other` (optional): where it is not 0 the row's number is other_uniform[r];
+// a caller that queues a step before it has read the one before passes that step's `drew_none` here, and both
+// numbers the row's stream may be at.
 extern "C" int tie_sample_filtered(const float* logits, const float* row_max, const float* inv_temperature,
-                                   const double* uniform, const int* top_k, const float* top_p, const int* rows,
-                                   int num_rows, int* out, int R, int V, hipStream_t stream) {
+                                   const double* uniform, const double* other_uniform, const int* take_other,
+                                   int* drew_none, const int* top_k, const float* top_p, const int* rows, int num_rows,
+                                   int* out, int R, int V, hipStream_t stream) {
   if (R <= 0 || V <= 0 || V > (1 << SF_ID_BITS) || (rows && (num_rows <= 0 || num_rows > R))) return TIE_BAD_ARGUMENT;
+  if (take_other && !other_uniform) return TIE_BAD_ARGUMENT;
   sample_filtered_kernel<<<rows ? num_rows : R, SF_THREADS, 0, stream>>>(logits, row_max, inv_temperature, uniform,
-                                                                         top_k, top_p, rows, out, V);
+                                                                         other_uniform, take_other, drew_none, top_k,
+                                                                         top_p, rows, out, V);
   return tie_launch_status();
 }

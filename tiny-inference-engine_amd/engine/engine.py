@@ -15,10 +15,11 @@ reference engine's (``src/engine/engine.cpp:26-235``):
 
 Reading ahead (``launch_ahead``, not in the reference). A decode step's host work - planning, the batch
 arrays, the launch - lies between two steps while the GPU idles, because the next step's tokens are the
-ones just sampled. With ``launch_ahead`` a step of greedy rows only queues its argmax and leaves the
+ones just sampled. With ``launch_ahead`` a step only queues its sampling kernels and leaves the
 tokens unread; if the next call to ``step()`` finds the steady state (nobody waiting, the very same
 sequences decoding, none at its last token), it queues the next step first - whose tokens the GPU
-takes from the argmax's own output - and reads the earlier step's tokens while that one runs. A
+takes from the sampling kernels' own output - and reads the earlier step's tokens while that one runs
+(rows that draw carry both uniform numbers their stream may be at, see ``DeviceSampler``). A
 sequence that turns out to have met a stop token has then run one token too many, which is dropped.
 In every other situation the unread tokens are read before anything is planned, and the engine behaves
 as without the option. Tokens (and callbacks) appear one ``step()`` later; ``has_work()`` stays true
@@ -269,9 +270,13 @@ class Engine:
         if unread is not None:
             self.steps_launched_ahead += 1
         tokens: List[int] = []
-        if sampling and self.launch_ahead and all(s.params.greedy for s in sampling):
+        if sampling and self.launch_ahead:
             try:
-                ticket = self.sampler.launch_greedy(logits)
+                if all(s.params.greedy for s in sampling):
+                    ticket = self.sampler.launch_greedy(logits)
+                else:
+                    ticket = self.sampler.launch(logits, [s.params for s in sampling], [s.rng for s in sampling],
+                                                 None if unread is None else unread.ticket)
             except BaseException:
                 self._end_all(sampling, FinishReason.ERROR)
                 raise

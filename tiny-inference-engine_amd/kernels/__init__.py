@@ -43,8 +43,8 @@ MAX_STEP_TOKENS = 65535   # rows of one step: a grid dimension of the row-wise k
 
 _SIGNATURES = {
     "sample_filtered": {
-        "tie_sample_filtered": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int,
-                                _c_int, _c_void],
+        "tie_sample_filtered": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                _c_int, _c_void, _c_int, _c_int, _c_void],
     },
     "elementwise": {
         "tie_embed": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -59,7 +59,8 @@ _SIGNATURES = {
         "tie_add_partials_rms_norm": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int,
                                       _c_int, _c_void],
         "tie_argmax": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
-        "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
+        "tie_sample": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_int,
+                       _c_int, _c_void],
         "tie_argmax_static": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "gemm_generic": {
@@ -705,13 +706,32 @@ def _row_selection(rows: Optional[torch.Tensor], row_max: Optional[torch.Tensor]
     return count
 
 
+def _uniform_numbers(uniform: torch.Tensor, other_uniform, take_other, drew_none, R: int) -> None:
+    for t, name in ((uniform, "uniform numbers"), (other_uniform, "the other uniform numbers")):
+        if t is None:
+            continue
+        _gpu(t, name)
+        if t.dtype != torch.float64 or t.numel() != R:
+            raise InvalidArgument(f"{name} must be float64, one per row")
+    if (take_other is None) != (other_uniform is None):
+        raise InvalidArgument("the other uniform numbers and the marks of the rows that take them come together")
+    if take_other is not None:
+        _i32(take_other, "marks of the rows that take the other number", R)
+    if drew_none is not None:
+        _i32(drew_none, "marks of the rows that drew nothing", R)
+
+
 def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor,
-                rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None) -> None:
+                rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None,
+                other_uniform: Optional[torch.Tensor] = None, take_other: Optional[torch.Tensor] = None,
+                drew_none: Optional[torch.Tensor] = None) -> None:
     """Draws one token per row from softmax(logits * inv_temperature) with the given uniform numbers, walking the
     tokens in index order. ``out[r]`` is -1 for a row with a NaN and -2 for a row that is all -inf. With ``rows``
     (int32 row numbers) only those rows are drawn; the other entries of ``out`` stay as they are. With ``row_max``
-    (the rows' maxima, which the caller has found to be finite, in rows without a NaN) the kernel does not look
-    for them."""
+    (the rows' maxima) the kernel does not look for them and leaves ``out`` of a row without a finite maximum as
+    it is. ``drew_none[r]`` becomes 1 where the row took no uniform number (no finite maximum), else 0;
+    where ``take_other[r]`` is not 0 the row's number is ``other_uniform[r]`` (a step queued before the one
+    before it is read passes that step's ``drew_none``, and both numbers its stream may be at)."""
     _f32(logits, "logits")
     if logits.dim() != 2:
         raise InvalidArgument("logits must be [rows, vocabulary]")
@@ -719,13 +739,12 @@ def sample_rows(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: to
     if V > MAX_SAMPLED_VOCAB:
         raise InvalidArgument(f"the sampling kernel takes rows of up to {MAX_SAMPLED_VOCAB} logits, got {V}")
     _f32(inv_temperature, "inverse temperatures", (R,))
-    _gpu(uniform, "uniform numbers")
-    if uniform.dtype != torch.float64 or uniform.numel() != R:
-        raise InvalidArgument("uniform numbers must be float64, one per row")
+    _uniform_numbers(uniform, other_uniform, take_other, drew_none, R)
     _i32(out, "sample output", R)
     count = _row_selection(rows, row_max, R)
     _call(_lib("elementwise").tie_sample, "sample", logits.data_ptr(), _ptr(row_max), inv_temperature.data_ptr(),
-          uniform.data_ptr(), _ptr(rows), count, out.data_ptr(), R, V, _stream())
+          uniform.data_ptr(), _ptr(other_uniform), _ptr(take_other), _ptr(drew_none), _ptr(rows), count, out.data_ptr(),
+          R, V, _stream())
 
 
 MAX_FILTERED_VOCAB = 1 << 19     # rows the top-k / top-p sampling kernel takes (its integer sums fit 64 bits)
@@ -733,14 +752,16 @@ MAX_FILTERED_VOCAB = 1 << 19     # rows the top-k / top-p sampling kernel takes 
 
 def sample_rows_filtered(logits: torch.Tensor, inv_temperature: torch.Tensor, uniform: torch.Tensor,
                          top_k: torch.Tensor, top_p: torch.Tensor, out: torch.Tensor,
-                         rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None) -> None:
+                         rows: Optional[torch.Tensor] = None, row_max: Optional[torch.Tensor] = None,
+                         other_uniform: Optional[torch.Tensor] = None, take_other: Optional[torch.Tensor] = None,
+                         drew_none: Optional[torch.Tensor] = None) -> None:
     """Draws one token per row with top-k and top-p: ``top_k[r]`` most likely kept (0: all), then the smallest
     prefix by likelihood whose weight reaches ``top_p[r]`` of the total (1: all), one uniform number a row, which
     walks the candidates in the order of likelihood also where neither filter removes any (``sample_rows`` walks
     them in index order, as the rule is without filters).
     ``out[r]`` is -1 for a row with a NaN and -2 for a row that is all -inf. With ``rows`` (int32 row numbers)
-    only those rows are drawn; the other entries of ``out`` stay as they are. With ``row_max`` (the rows' maxima,
-    which the caller has found to be finite, in rows without a NaN) the kernel does not look for them."""
+    only those rows are drawn; the other entries of ``out`` stay as they are. ``row_max``, ``other_uniform``,
+    ``take_other`` and ``drew_none`` as in ``sample_rows``."""
     _f32(logits, "logits")
     if logits.dim() != 2:
         raise InvalidArgument("logits must be [rows, vocabulary]")
@@ -750,14 +771,12 @@ def sample_rows_filtered(logits: torch.Tensor, inv_temperature: torch.Tensor, un
     _f32(inv_temperature, "inverse temperatures", (R,))
     _f32(top_p, "top_p", (R,))
     _i32(top_k, "top_k", R)
-    _gpu(uniform, "uniform numbers")
-    if uniform.dtype != torch.float64 or uniform.numel() != R:
-        raise InvalidArgument("uniform numbers must be float64, one per row")
+    _uniform_numbers(uniform, other_uniform, take_other, drew_none, R)
     _i32(out, "sample output", R)
     count = _row_selection(rows, row_max, R)
     _call(_lib("sample_filtered").tie_sample_filtered, "sample_filtered", logits.data_ptr(), _ptr(row_max),
-          inv_temperature.data_ptr(), uniform.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), _ptr(rows), count,
-          out.data_ptr(), R, V, _stream())
+          inv_temperature.data_ptr(), uniform.data_ptr(), _ptr(other_uniform), _ptr(take_other), _ptr(drew_none),
+          top_k.data_ptr(), top_p.data_ptr(), _ptr(rows), count, out.data_ptr(), R, V, _stream())
 
 
 # Up to this many workgroups of single decoded rows run in the prefill attention kernel beside a step's prompt

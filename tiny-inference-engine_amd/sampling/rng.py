@@ -21,7 +21,7 @@ _TWO64 = float(2 ** 64)
 
 
 class RandomStream:
-    __slots__ = ("_state", "_next")
+    __slots__ = ("_state", "_next", "_seen")
 
     def __init__(self, seed: int = 0):
         state = [seed & _MASK64]
@@ -30,6 +30,7 @@ class RandomStream:
             state.append((6364136223846793005 * (prev ^ (prev >> 62)) + i) & _MASK64)
         self._state = state
         self._next = _N
+        self._seen = []            # outputs looked at with ``peek_unit`` and not taken yet, the next one first
 
     def _refill(self) -> None:
         s = self._state
@@ -42,6 +43,11 @@ class RandomStream:
         self._next = 0
 
     def next_u64(self) -> int:
+        if self._seen:
+            return self._seen.pop(0)
+        return self._generate()
+
+    def _generate(self) -> int:
         if self._next >= _N:
             self._refill()
         y = self._state[self._next]
@@ -54,8 +60,23 @@ class RandomStream:
 
     def unit(self) -> float:
         """A double in [0, 1): one output scaled by 2^-64, clamped below 1."""
-        u = self.next_u64() / _TWO64
+        return self._as_unit(self.next_u64())
+
+    @staticmethod
+    def _as_unit(output: int) -> float:
+        u = output / _TWO64
         return u if u < 1.0 else math.nextafter(1.0, 0.0)
+
+    def peek_unit(self, ahead: int = 0) -> float:
+        """What the ``ahead + 1``-th call of ``unit`` from now will return; takes nothing from the stream."""
+        while len(self._seen) <= ahead:
+            self._seen.append(self._generate())
+        return self._as_unit(self._seen[ahead])
+
+    def skip(self, count: int = 1) -> None:
+        """Takes ``count`` outputs from the stream, unseen."""
+        for _ in range(count):
+            self.next_u64()
 
     def uniform(self, low: float, high: float) -> float:
         return self.unit() * (high - low) + low

@@ -20,7 +20,7 @@ own stream. The top-k / top-p kernel sums its weights as integers in units of 2^
 
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -74,27 +74,38 @@ def sample(logits: np.ndarray, params: SamplingParams, rng: RandomStream) -> int
     return int(pick if ids is None else ids[pick])
 
 
-class GreedyTicket:
-    """Rows whose argmax has been asked of the GPU and not yet read: see ``DeviceSampler.launch_greedy``."""
+class Ticket:
+    """Rows whose tokens have been asked of the GPU and not yet read: see ``DeviceSampler.launch``."""
 
-    __slots__ = ("rows", "device_tokens", "host", "event")
+    __slots__ = ("rows", "device_tokens", "host", "event", "drew_none", "drawing", "rngs")
 
-    def __init__(self, rows, device_tokens, host, event):
+    def __init__(self, rows, device_tokens, host, event, drew_none=None, drawing=(), rngs=()):
         self.rows = rows
         self.device_tokens = device_tokens     # int32 [rows] on the device: the chosen tokens, in row order
         self.host = host                       # pinned int32 [2 * rows]: tokens, then the maxima's bits
         self.event = event
+        self.drew_none = drew_none             # int32 [rows] on the device: 1 where a drawing row took no number
+        self.drawing = drawing                 # the rows that draw, and their streams: a number is taken from a
+        self.rngs = rngs                       # stream when the row is known to have used one
 
 
 class DeviceSampler:
-    """Samples the rows of one step's logits, on the GPU where the parameters allow it.
+    """Samples the rows of one step's logits on the GPU.
 
-    The results come back through pinned host buffers that live as long as the sampler: a step of greedy
-    rows is one kernel, one copy of ``2 R`` words and one wait. ``launch_greedy`` / ``collect`` split that
-    into asking and reading, so that a caller may queue the next step (whose tokens it takes from
-    ``ticket.device_tokens``) before it reads this one's; two sets of buffers alternate for that."""
+    The results come back through pinned host buffers that live as long as the sampler: a step is the argmax
+    kernel over all rows (the greedy rows' answer, the maxima for the others, and what finds a NaN or a row of
+    -inf), a drawing kernel for the rows with a temperature and one for those with top-k or top-p, which put
+    their tokens where the argmax stood, one copy of ``2 R`` words and one wait. ``launch`` / ``collect`` split
+    that into asking and reading, so that a caller may queue the next step (whose tokens it takes from
+    ``ticket.device_tokens``) before it reads this one's; two sets of buffers alternate for that.
+
+    A row's uniform number is the next of its request's stream, but a row with a +inf logit takes none, and
+    whether that happened in a step not yet read is known on the GPU only. A step queued behind such a step
+    (``previous``) therefore carries two numbers a row, the stream's next and the one after, and the kernel takes
+    the one that fits what the step before did; the streams move on when a step is read."""
 
     GREEDY, PLAIN, FILTERED = 0, 1, 2      # argmax kernel / temperature kernel / top-k and top-p kernel
+    RESULTS, PARAMETERS = 3, 8             # words a row: tokens, maxima, marks / what the drawing kernels take
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -103,38 +114,92 @@ class DeviceSampler:
         self._turn = 0
 
     def _buffers(self, rows: int):
-        """Device words and pinned host words: 3 R of results (argmax, maxima, draws), then 6 R of parameters."""
         if rows > self._rows:
             self._rows = max(64, 2 * rows)
-            self._sets = [(torch.empty(9 * self._rows, dtype=torch.int32, device=self.device),
-                           torch.empty(9 * self._rows, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
+            words = (self.RESULTS + self.PARAMETERS) * self._rows
+            self._sets = [(torch.empty(words, dtype=torch.int32, device=self.device),
+                           torch.empty(words, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
                           for _ in range(2)]
         self._turn ^= 1
         return self._sets[self._turn]
 
-    def _fetch(self, dev: torch.Tensor, host: torch.Tensor, count: int) -> np.ndarray:
-        host[:count].copy_(dev[:count], non_blocking=True)
-        if self.device.type == "cuda":
-            torch.cuda.current_stream(self.device).synchronize()
-        return host.numpy()[:count]
-
-    # ------------------------------------------------------------- greedy rows, asked for and read apart
-    def launch_greedy(self, logits: torch.Tensor) -> GreedyTicket:
+    # ------------------------------------------------------------------------- asked for and read apart
+    def launch_greedy(self, logits: torch.Tensor) -> Ticket:
         """Queues the argmax of every row and the copy of the results to the host; returns at once."""
         from .. import kernels
 
         R = logits.shape[0]
         dev, host = self._buffers(R)
         kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
+        return self._ticket(dev, host, R)
+
+    def _ticket(self, dev, host, R, drew_none=None, drawing=(), rngs=()) -> Ticket:
         host[:2 * R].copy_(dev[:2 * R], non_blocking=True)
         event = None
         if self.device.type == "cuda":
             event = torch.cuda.Event()
             event.record()
-        return GreedyTicket(R, dev[:R], host, event)
+        return Ticket(R, dev[:R], host, event, drew_none, drawing, rngs)
 
-    def collect(self, ticket: GreedyTicket) -> List[int]:
-        """Waits for a ticket's results; the tokens of its rows (ties went to the lowest id)."""
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], rngs: Sequence[RandomStream],
+               previous: Optional[Ticket] = None) -> Ticket:
+        """Queues the choice of a token for every row; returns at once. ``previous``: the ticket of the step
+        before, of the same requests in the same rows, if it has not been collected yet."""
+        from .. import kernels
+
+        R, V = logits.shape
+        if R != len(params) or R != len(rngs):
+            raise InvalidArgument("one set of sampling parameters and one random stream per row")
+        if previous is not None and previous.rows != R:
+            raise InvalidArgument(f"the step before had {previous.rows} rows, this one has {R}")
+        # Without a filter the reference walks the candidates in index order, with one in the order of likelihood
+        # (src/sampling/sampler.cpp:41-54): the same uniform number picks different tokens, so each has its kernel.
+        kinds = np.fromiter((self.GREEDY if p.greedy else (self.FILTERED if 0 < p.top_k < V or p.top_p < 1.0 else self.PLAIN)
+                             for p in params), dtype=np.int8, count=R)
+        dev, host = self._buffers(R)
+        maxima = dev[R:2 * R].view(torch.float32)
+        kernels.argmax_rows(logits, dev[:R], maxima)
+        filtered, plain = np.flatnonzero(kinds == self.FILTERED), np.flatnonzero(kinds == self.PLAIN)
+        if not filtered.size and not plain.size:
+            return self._ticket(dev, host, R)
+        # The parameters go up in one copy, a word a row each: 1 / temperature, top_p, top_k, the numbers of the
+        # drawing rows (those with a filter first), and two words a row for each of the two uniform numbers.
+        P = R + (R & 1)                                    # the float64 numbers start on 8 bytes
+        at = self.RESULTS * self._rows
+        words = host[at:at + self.PARAMETERS * P].numpy()
+        inv_t, top_p = words[:R].view(np.float32), words[P:P + R].view(np.float32)
+        top_k, rows = words[2 * P:2 * P + R], words[3 * P:3 * P + R]
+        uniform, other = words[4 * P:6 * P].view(np.float64)[:R], words[6 * P:8 * P].view(np.float64)[:R]
+        inv_t[:], top_p[:], top_k[:], uniform[:], other[:] = 1.0, 1.0, 0, 0.0, 0.0
+        drawing = np.concatenate([filtered, plain])
+        if previous is not None and not np.array_equal(previous.drawing, drawing):
+            raise InvalidArgument("the step before did not draw for the same rows")
+        ahead = 0 if previous is None else 1               # numbers of the stream that the step before may have used
+        for i in drawing:
+            inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
+            uniform[i] = rngs[i].peek_unit(ahead)
+            other[i] = rngs[i].peek_unit(0)
+        for i in filtered:
+            top_p[i], top_k[i] = params[i].top_p, min(params[i].top_k, V)
+        rows[:drawing.size] = drawing
+        up = dev[at:at + self.PARAMETERS * P]
+        up.copy_(host[at:at + self.PARAMETERS * P], non_blocking=True)
+        d_inv_t = up[:R].view(torch.float32)
+        d_uniform, d_other = up[4 * P:6 * P].view(torch.float64)[:R], up[6 * P:8 * P].view(torch.float64)[:R]
+        drew_none = dev[2 * R:3 * R]
+        take_other = None if previous is None else previous.drew_none
+        if take_other is None:
+            d_other = None
+        if filtered.size:
+            kernels.sample_rows_filtered(logits, d_inv_t, d_uniform, up[2 * P:2 * P + R], up[P:P + R].view(torch.float32),
+                                         dev[:R], up[3 * P:3 * P + filtered.size], maxima, d_other, take_other, drew_none)
+        if plain.size:
+            kernels.sample_rows(logits, d_inv_t, d_uniform, dev[:R], up[3 * P + filtered.size:3 * P + drawing.size], maxima,
+                                d_other, take_other, drew_none)
+        return self._ticket(dev, host, R, drew_none, drawing, [rngs[i] for i in drawing])
+
+    def collect(self, ticket: Ticket) -> List[int]:
+        """Waits for a ticket's results; the tokens of its rows. Moves the streams of the rows that drew."""
         if ticket.event is not None:
             ticket.event.synchronize()
         R = ticket.rows
@@ -144,66 +209,14 @@ class DeviceSampler:
             raise InvalidArgument(f"a logit of row {int(np.flatnonzero(best < 0)[0])} is NaN")
         if (top == -np.inf).any():
             raise InvalidArgument(f"all logits of row {int(np.flatnonzero(top == -np.inf)[0])} are -inf")
+        for i, rng in zip(ticket.drawing, ticket.rngs):
+            if top[i] != np.inf:               # a +inf logit is certain and takes no random number
+                rng.skip()
         return best.tolist()
 
     # ------------------------------------------------------------------------------------ any rows, at once
     def sample_rows(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                     rngs: Sequence[RandomStream]) -> List[int]:
-        from .. import kernels
-
-        R = logits.shape[0]
-        if R != len(params) or R != len(rngs):
-            raise InvalidArgument("one set of sampling parameters and one random stream per row")
-        V = logits.shape[1]
-        # Without a filter the reference walks the candidates in index order, with one in the order of likelihood
-        # (src/sampling/sampler.cpp:41-54): the same uniform number picks different tokens, so each has its kernel.
-        kinds = np.fromiter((self.GREEDY if p.greedy else (self.FILTERED if 0 < p.top_k < V or p.top_p < 1.0 else self.PLAIN)
-                             for p in params), dtype=np.int8, count=R)
-        if not kinds.any():
+        if all(p.greedy for p in params):
             return self.collect(self.launch_greedy(logits))
-        # The argmax kernel works on all rows: it answers the greedy rows, finds NaN and all -inf rows, and a
-        # +inf logit, which is certain and consumes no random number. Index and maximum lie side by side, so one
-        # copy brings both.
-        dev, host = self._buffers(R)
-        kernels.argmax_rows(logits, dev[:R], dev[R:2 * R].view(torch.float32))
-        fetched = self._fetch(dev, host, 2 * R)
-        best, top = fetched[:R], fetched[R:].view(np.float32)
-        if (best < 0).any():
-            raise InvalidArgument(f"a logit of row {int(np.flatnonzero(best < 0)[0])} is NaN")
-        if (top == -np.inf).any():
-            raise InvalidArgument(f"all logits of row {int(np.flatnonzero(top == -np.inf)[0])} are -inf")
-        out = best.astype(np.int64)
-        plain = np.flatnonzero((kinds == self.PLAIN) & (top != np.inf))
-        filtered = np.flatnonzero((kinds == self.FILTERED) & (top != np.inf))
-        if not plain.size and not filtered.size:
-            return out.tolist()
-        # The parameters of the drawing rows go up in one copy: 1 / temperature, top_p, top_k, the numbers of the
-        # drawing rows, those with a filter first (one word a row each), one uniform number a row (two words).
-        P = R + (R & 1)                                    # the float64 numbers start on 8 bytes
-        at = 3 * self._rows
-        words = host[at:at + 6 * P].numpy()
-        inv_t, top_p = words[:R].view(np.float32), words[P:P + R].view(np.float32)
-        top_k, rows, uniform = words[2 * P:2 * P + R], words[3 * P:3 * P + R], words[4 * P:6 * P].view(np.float64)[:R]
-        inv_t[:], top_p[:], top_k[:], uniform[:] = 1.0, 1.0, 0, 0.0
-        for i in np.concatenate([plain, filtered]):
-            inv_t[i] = np.float32(1.0) / np.float32(params[i].temperature)
-            uniform[i] = rngs[i].unit()
-        for i in filtered:
-            top_p[i], top_k[i] = params[i].top_p, min(params[i].top_k, V)
-        rows[:filtered.size] = filtered
-        rows[filtered.size:filtered.size + plain.size] = plain
-        up = dev[at:at + 6 * P]
-        up.copy_(host[at:at + 6 * P], non_blocking=True)
-        d_inv_t, d_uniform = up[:R].view(torch.float32), up[4 * P:6 * P].view(torch.float64)[:R]
-        drawn = dev[2 * R:3 * R]
-        maxima = dev[R:2 * R].view(torch.float32)
-        if plain.size:
-            kernels.sample_rows(logits, d_inv_t, d_uniform, drawn,
-                                up[3 * P + filtered.size:3 * P + filtered.size + plain.size], maxima)
-        if filtered.size:
-            kernels.sample_rows_filtered(logits, d_inv_t, d_uniform, up[2 * P:2 * P + R], up[P:P + R].view(torch.float32),
-                                         drawn, up[3 * P:3 * P + filtered.size], maxima)
-        got = self._fetch(dev[2 * R:], host[2 * R:], R)
-        out[plain] = got[plain]
-        out[filtered] = got[filtered]
-        return out.tolist()
+        return self.collect(self.launch(logits, params, rngs))
