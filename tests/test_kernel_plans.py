@@ -86,6 +86,19 @@ def test_the_tiled_product_plans_by_rounds_of_workgroups():
             assert ranges in (1, 2, 4, 8) and (ranges == 1 or K // ranges >= 512), (M, N, K, ranges)
             assert kernels.gemm_tile(M, N, K, True) in TILE_ROWS_COLS
             assert kernels.gemm_tile(M, N, K, True, 1) in TILE_ROWS_COLS
+    # 65 to 128 rows: the weights are read once, and one round of workgroups should fill the compute units.
+    # 8B gate/up on 128 x 128 tiles (192 workgroups; 96 of 128 x 256 took 82 us against 61), the 1.7B's on
+    # 64 x 128 (192), the 32B's on 128 x 256 (200); the 32B's QKV in 4 ranges (160 workgroups; 8 are two rounds)
+    assert kernels.gemm_tile(128, *gate_up, True, 1) == 7 and kernels.gemm_tile(80, *gate_up, True, 1) == 7
+    assert kernels.gemm_tile(96, 12288, 2048, True, 1) == 9 and kernels.gemm_tile(128, 51200, 5120, True, 1) == 6
+    assert (kernels.gemm_tile(128, 10240, 5120, True), kernels.gemm_splits(128, 10240, 5120, True)) == (6, 4)
+    assert (kernels.gemm_tile(128, 4096, 2048, True), kernels.gemm_splits(128, 4096, 2048, True)) == (9, 4)
+    assert (kernels.gemm_tile(128, *down, True), kernels.gemm_splits(128, *down, True)) == (7, 8)
+    for N, K in (qkv, o, down, (2048, 2048), (10240, 5120), (5120, 25600), (2048, 6144)):
+        for M in range(65, 129, 9):
+            ranges = kernels.gemm_splits(M, N, K, True)
+            assert ranges in (1, 2, 4, 8) and (ranges == 1 or K // ranges >= 512), (M, N, K, ranges)
+            assert kernels.gemm_tile(M, N, K, True) in (6, 7, 8, 9) and kernels.gemm_tile(M, N, K, True, 1) in (6, 7, 8, 9)
     # shapes the straight-to-LDS tiles do not take keep the older tiles and their rule
     assert kernels.gemm_splits(300, 200, 1000) == 2 and kernels.gemm_tile(300, 200, 1000) == 1
     assert kernels.gemm_splits(128, 4096, 4096) == 8 and kernels.gemm_splits(128, 4096, 256) == 1

@@ -608,8 +608,8 @@ static bool gemm_dma_takes(const void* x, const void* w, const void* out, int N,
 // Which tile, and how many ranges of K (planes of partial sums that the caller adds), a product takes when
 // left to choose.
 //
-// Up to 128 rows over packed weights: rules measured on the projections of the 1.7B, 8B and 32B shapes.
-// Above that, for shapes the straight-to-LDS tiles take: the cheapest of (tile, ranges) by an estimate of
+// Up to 64 rows over packed weights: rules measured on the projections of the 1.7B, 8B and 32B shapes; 65 to 128
+// rows: few_rows_us. Above that, for shapes the straight-to-LDS tiles take: the cheapest of (tile, ranges) by an estimate of
 // the time, whose terms were fitted to sweeps over the same shapes at 256 to 2048 rows:
 //   * a compute unit holds one workgroup (two of the 128 x 128 tile), so the workgroups run in rounds of
 //     256; a round that is nearly empty lasts as long as a full one, which is what a rule by thresholds
@@ -656,14 +656,49 @@ static float estimated_us(const DmaTile& t, int M, int N, int K, int ranges) {
   return us + ranges * plane_mb * (1.0f / 6.0f + 1.0f / 5.0f);   // written here, read by the consumer: MB / (TB/s) = us
 }
 
+// 65 to 128 rows: a workgroup's pace is set by the bytes it loads a slice of 32 along K, its rows of x and its
+// columns of w (about 40 GB/s a compute unit), and all of them together by the weights' bytes (5.5 TB/s);
+// workgroups run in rounds of 256. Fitted to sweeps over the projections of the 1.7B, 8B and 32B shapes at 80,
+// 96 and 128 rows: 8B gate/up at 128 rows 61 us on 128 x 128 tiles (192 workgroups) against 82 on 128 x 256 (96).
+struct FewRowsTile { int id, bm, bn; };
+static const FewRowsTile kFewRowsTiles[] = {{6, 128, 256}, {7, 128, 128}, {8, 64, 256}, {9, 64, 128}};
+
+static float few_rows_us(const FewRowsTile& t, int M, int N, int K, int ranges) {
+  const long wgs = static_cast<long>((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * ranges;
+  const int k_slices = K / GD_BK;
+  const int slices = (k_slices + ranges - 1) / ranges;
+  const float per_slice = static_cast<float>(t.bm + t.bn) * (GD_BK * 2) / 40000.f;
+  float us = static_cast<float>((wgs + 255) / 256) * (4.f + slices * per_slice);
+  us = fmaxf(us, static_cast<float>(N) * K * 2e-6f / 5.5f);
+  if (ranges > 1) us += ranges * static_cast<float>(M) * N * 4e-6f * (1.0f / 6.0f + 1.0f / 5.0f);
+  return us;
+}
+
 // splits: 0 = free to choose (the caller adds planes), else the number of ranges the caller has fixed (1: none).
 static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, int splits, bool packed) {
   const bool may_split = splits == 0;
-  if (straight_to_lds && packed && M <= 128) {
-    // Few rows over packed weights: tiles of 64 or 128 rows (measured on the projections of the 1.7B, 8B and
-    // 32B shapes at 48 to 128 rows). Wide weights take 256 columns a tile, narrow ones 128 and more ranges of K.
-    const bool wide = M <= 64 ? N >= 8192 : N >= 5120;
-    const int tile = M <= 64 ? (wide ? 8 : 9) : (wide ? 6 : 7);
+  if (straight_to_lds && packed && M > 64 && M <= 128) {
+    // 65 to 128 rows over packed weights: the weights are read once by few workgroups, so what counts is that
+    // one round of workgroups fills the compute units. The cheapest of (tile, ranges) by few_rows_us.
+    GemmPlan best = {7, may_split ? 1 : splits};
+    float best_us = 0.f;
+    for (int r = may_split ? 1 : splits; r <= (may_split ? 8 : splits); r *= 2) {
+      if (may_split && r > 1 && K / r < 512) break;
+      for (const FewRowsTile& t : kFewRowsTiles) {
+        const float us = few_rows_us(t, M, N, K, r);
+        if (best_us == 0.f || us < best_us * 0.98f) {       // ties go to fewer planes, then to the larger tile
+          best = {t.id, r};
+          best_us = us;
+        }
+      }
+    }
+    return best;
+  }
+  if (straight_to_lds && packed && M <= 64) {
+    // Up to 64 rows over packed weights: tiles of 64 rows (measured on the projections of the 1.7B, 8B and
+    // 32B shapes at 48 to 64 rows). Wide weights take 256 columns a tile, narrow ones 128 and more ranges of K.
+    const bool wide = N >= 8192;
+    const int tile = wide ? 8 : 9;
     if (!may_split) return {tile, splits};
     const long tiles = (N + (wide ? 255 : 127)) / (wide ? 256 : 128);
     for (int r = 1; r <= 8; r *= 2)
