@@ -329,10 +329,12 @@ def test_skinny_gemm_bf16(M, N, K):
 
 @pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
 @pytest.mark.parametrize("N,K,gated", [(10240, 5120, False), (5120, 8192, False), (5120, 25600, False), (1600, 5120, True),
-                                       (2048, 6144, False), (4096, 2048, False)])
+                                       (2048, 6144, False), (4096, 2048, False), (1024, 4032, False)])
 def test_skinny_gemm_bf16_at_the_widths_of_other_model_sizes(M, N, K, gated):
     """The projections of the 32B shape (rows of 5120, K up to 25600) and of the 1.7B shape, packed, cut along K
-    as the plan says (2, 4 or 8 planes), with every pair of tile count and batch of loads the launcher may pick."""
+    as the plan says (2, 4 or 8 planes), with every pair of tile count and batch of loads the launcher may pick.
+    For the kernel that shares x through LDS they hold ranges of 4, 16, 20 and 40 chunks of k-blocks (fewer than
+    its ring is deep, and many rounds of it) and, at K = 4032, a range whose last chunk is half empty."""
     from tie_amd import kernels
 
     x = rnd(M, K, seed=41, dtype=torch.bfloat16).cuda()

@@ -25,6 +25,8 @@
 // (6.1 against 5.1 TB/s on a 201 MB weight); read once, the stream is loaded non-temporally.
 #include "common.h"
 
+#include <type_traits>
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
@@ -192,31 +194,76 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
 // weight block of 1 KB needs MT blocks of x, and a compute unit serves a load instruction of a wave in about 65
 // cycles whether it comes from HBM or from L2, so at 64 rows (7 loads for 3 KB of weights) the weights stream
 // at 3.6 TB/s. Here the WAVES waves of a workgroup walk the SAME range of K, each over its own RT weight
-// tiles, and share x: a chunk of XU k-blocks of all rows goes from global memory straight into LDS (buffer
+// tiles, and share x: a chunk of U k-blocks of all rows goes from global memory straight into LDS (buffer
 // loads with the lds flag; one instruction brings one 16-row block of 32 k, lane l's 16 bytes - row l % 16,
-// k-chunk l / 16 - to byte 16 l, which is the order the matrix core takes its A operand), one chunk ahead
-// of the arithmetic, and all waves read their fragments from there. Weights still go from memory straight
-// into registers, non-temporally, one chunk ahead. x then costs MT / (WAVES x RT) of the weights' load
-// instructions; the price is a barrier a chunk, so only long, wide products gain (rows_kernel_tiles below).
+// k-chunk l / 16 - to byte 16 l, which is the order the matrix core takes its A operand) and all waves read
+// their fragments from there. Weights still go from memory straight into registers, non-temporally. x then
+// costs MT / (WAVES x RT) of the weights' load instructions.
+//
+// Both streams run DEPTH chunks ahead of the arithmetic, through a ring of DEPTH + 1 LDS buffers and register
+// sets, and a step waits only until the NEXT chunk has landed (loads complete in the order they were asked
+// for, so that is when at most the loads of the DEPTH - 1 chunks after it are outstanding): the queue of
+// loads never runs empty. (Waiting for everything at each chunk's barrier, as a first version did, left a wave
+// idle for a memory latency a chunk: gate/up of the 8B shape at 64 rows 54 us, now 42.) What bounds it now is
+// x itself: every workgroup reads all of it, 512 KB beside its 785 KB of weights on that shape, and a compute
+// unit takes about 38 GB/s.
 //
 // The sums are the very ones of the kernel above: a plane's range of K is walked in the same four parts
 // of per_wave k-blocks, each summed by the matrix core in k order, and the parts are added in their order
 // (there: by the reduction through LDS; here: by folding the accumulator into a running total at each
 // part's end). A row's result therefore does not depend on which of the two kernels its batch size picks.
 typedef __attribute__((address_space(3))) void sk_lds_void_t;
-#define SK_XU 8
 // Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
 // selects x, y, z, w; no swizzle, no stride.
 #define SK_RSRC_FLAGS 0x27000
 
-template <int MT, int RT, int WAVES, typename TO>
+// The matrix instructions of one chunk: x from LDS, the weights from registers. A function of its own with
+// restrict pointers, so that the compiler knows these LDS reads from the loads into LDS that are in flight
+// (otherwise it waits for all of them before the first read).
+template <int MT, int RT, int U, bool FULL>
+__device__ __forceinline__ void rows_chunk(const bf16_t* __restrict__ xc, const bf16x8_t (&wr)[RT][U],
+                                           floatx4 (&acc)[MT][RT], int kb0, int kb_hi, int lane) {
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (FULL || kb0 + u < kb_hi) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const sk_u32x4_t av = *reinterpret_cast<const sk_u32x4_t*>(xc + (u * MT + mt) * 512 + lane * 8);
+        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&av);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, wr[t][u], acc[mt][t], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters at their maxima).
+template <int N>
+__device__ __forceinline__ void rows_wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Calls f(integral_constant<int, I>) for I = 0 .. N - 1.
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void rows_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    rows_static_for<N, I + 1>(f);
+  }
+}
+
+// U: k-blocks of a chunk; DEPTH: chunks in flight behind the one at work.
+template <int MT, int RT, int WAVES, int U, int DEPTH, typename TO>
 __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16_t* __restrict__ x,
                                                                       const bf16_t* __restrict__ w,
                                                                       TO* __restrict__ out, int M, int N, int K,
                                                                       int accumulate, int gated, int per_wave) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int U = SK_XU;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][U][MT][512];
+  constexpr int NS = DEPTH + 1;
+  constexpr int NX = (U * MT + WAVES - 1) / WAVES;      // blocks of x a wave loads a chunk
+  constexpr int PER_CHUNK = NX + RT * U;                // loads a wave issues a chunk
+  __shared__ __attribute__((aligned(16))) bf16_t xs[NS][U * MT * 512];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TIE_WAVE);
   const int tiles = N / 16;
@@ -235,24 +282,27 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16
       const_cast<bf16_t*>(x), 0, static_cast<int>(static_cast<size_t>(M) * K * 2), SK_RSRC_FLAGS);
   const unsigned lane_off = (static_cast<unsigned>(lane & 15) * K + (lane >> 4) * 8) * 2;   // bytes, within a 16-row block
   const unsigned tile_rows = 16u * K * 2;
-  // Blocks (u, mt) of a chunk are dealt to the waves in turn.
-  auto fetch_rows = [&](int kb0, int buf) {
+
+  // Chunk c: k-blocks kb_lo + c U and the U - 1 after it. Its loads, into set S of the ring: every wave issues
+  // the same number of them whatever the chunk (the waits count instructions): the blocks (u, mt) of x are dealt
+  // to the waves in turn, a wave with one block fewer loads one of the others' again, and k-blocks beyond the
+  // range are the range's last again (their products are not formed).
+  bf16x8_t wr[NS][RT][U];
+  auto issue = [&](auto set, int chunk) {
+    constexpr int S = decltype(set)::value;
+    const int kb0 = kb_lo + chunk * U;
 #pragma unroll
-    for (int i = 0; i < (U * MT + WAVES - 1) / WAVES; ++i) {
-      const int b = i * WAVES + wave;
+    for (int i = 0; i < NX; ++i) {
+      const int b = (i * WAVES + wave) % (U * MT);
       const int u = b / MT, mt = b % MT;
-      if (b < U * MT && kb0 + u < kb_hi)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (sk_lds_void_t*)(&xs[buf][u][mt][0]), 16,
-                                                 lane_off + mt * tile_rows, (kb0 + u) * 64, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (sk_lds_void_t*)(&xs[S][(u * MT + mt) * 512]), 16,
+                                               lane_off + mt * tile_rows, min(kb0 + u, kb_hi - 1) * 64, 0, 0);
     }
-  };
-  bf16x8_t b[RT][U], nb[RT][U];
-  auto fetch_weights = [&](bf16x8_t (&bb)[RT][U], int kb0) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int t = 0; t < RT; ++t)
-        bb[t][u] = (kb0 + u < kb_hi) ? load_weight_frag<true>(wp[t] + static_cast<size_t>(kb0 + u) * 512) : zero_frag();
+        wr[S][t][u] = load_weight_frag<true>(wp[t] + static_cast<size_t>(min(kb0 + u, kb_hi - 1)) * 512);
   };
 
   floatx4 acc[MT][RT], total[MT][RT];
@@ -260,59 +310,65 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < RT; ++t) acc[mt][t] = total[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  bool first_part = true;
-  auto fold = [&]() {          // a part of K has ended: total = total + part, the first part as it is
+  // A part of K has ended: total += part. Parts are whole chunks (the host sees to it), so this stands between
+  // two chunks.
+  int part_end = kb_lo + per_wave;
+  auto fold_at = [&](int kb0) {
+    if (kb0 != part_end) return;
+    part_end += per_wave;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
-        if (first_part) total[mt][t] = acc[mt][t];
-        else
 #pragma unroll
-          for (int v = 0; v < 4; ++v) total[mt][t][v] += acc[mt][t][v];
+        for (int v = 0; v < 4; ++v) total[mt][t][v] += acc[mt][t][v];
         acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
       }
-    first_part = false;
   };
 
   if (kb_lo < kb_hi) {
-    fetch_rows(kb_lo, 0);
-    fetch_weights(b, kb_lo);
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    int buf = 0;
-    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += U) {
-      const bool more = kb0 + U < kb_hi;
-      if (more) {
-        fetch_rows(kb0 + U, buf ^ 1);          // everyone's reads of that buffer ended before the last barrier
-        fetch_weights(nb, kb0 + U);
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kb = kb0 + u;
-        if (kb < kb_hi) {
-          if (kb > kb_lo && (kb - kb_lo) % per_wave == 0) fold();
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const sk_u32x4_t av = *reinterpret_cast<const sk_u32x4_t*>(&xs[buf][u][mt][lane * 8]);
-            const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&av);
-#pragma unroll
-            for (int t = 0; t < RT; ++t) acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t][u], acc[mt][t], 0, 0, 0);
-          }
-        }
-      }
-      if (more) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int t = 0; t < RT; ++t) b[t][u] = nb[t][u];
-      }
-      // The next chunk of x (and of the weights: they were asked for after it) has landed; after the barrier
-      // it may be read, and this chunk's buffer written again.
+    const int chunks = (kb_hi - kb_lo + U - 1) / U;
+    // DEPTH chunks are in flight behind the one whose products are formed. A step: ask for chunk c + DEPTH
+    // (into the set that chunk c - 1 left), form chunk c's products, then wait until chunk c + 1 has landed,
+    // which is when at most the loads of the DEPTH - 1 chunks after it are outstanding, and meet the other
+    // waves: their blocks of x have landed too, and all have read chunk c's.
+    auto step = [&](auto set, auto next_set, int c) {
+      issue(next_set, c + DEPTH);
+      fold_at(kb_lo + c * U);
+      rows_chunk<MT, RT, U, true>(&xs[decltype(set)::value][0], wr[decltype(set)::value], acc, kb_lo + c * U, kb_hi, lane);
+      rows_wait_loads<(DEPTH - 1) * PER_CHUNK>();
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    // The range's last chunks, with nothing more to ask for.
+    auto last_step = [&](auto set, int c) {
+      fold_at(kb_lo + c * U);
+      rows_chunk<MT, RT, U, false>(&xs[decltype(set)::value][0], wr[decltype(set)::value], acc, kb_lo + c * U, kb_hi, lane);
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      buf ^= 1;
-    }
+    };
+    static_assert((DEPTH - 1) * PER_CHUNK < 64, "the wait counts loads with six bits");
+    rows_static_for<DEPTH>([&](auto i) { issue(i, decltype(i)::value); });
+    rows_wait_loads<(DEPTH - 1) * PER_CHUNK>();
+    asm volatile("s_barrier" ::: "memory");
+    // The ring's sets are named at compile time, so the steps come in groups of NS.
+    int c = 0;
+    for (; c + NS - 1 + DEPTH < chunks; c += NS)
+      rows_static_for<NS>([&](auto i) {
+        constexpr int I = decltype(i)::value;
+        step(i, std::integral_constant<int, (I + DEPTH) % NS>{}, c + I);
+      });
+    // Up to NS - 1 + DEPTH chunks are left; those that still have a chunk DEPTH ahead ask for it.
+    rows_static_for<NS - 1 + DEPTH>([&](auto i) {
+      constexpr int I = decltype(i)::value;
+      if (c + I + DEPTH < chunks) step(std::integral_constant<int, I % NS>{}, std::integral_constant<int, (I + DEPTH) % NS>{}, c + I);
+      else if (c + I < chunks) last_step(std::integral_constant<int, I % NS>{}, c + I);
+    });
   }
-  fold();
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) total[mt][t][v] += acc[mt][t][v];
 
   // D layout: lane holds rows (lane / 16) * 4 + v of a 16-row tile of x, column lane % 16 of the weight tile.
   const int c = lane & 15, q4 = (lane >> 4) * 4;
@@ -375,15 +431,34 @@ static int choose_rt(int M, int N, int splits) {
 }
 
 // Weight tiles a workgroup of the kernel that shares x through LDS takes (8: four waves x two tiles, 6: three
-// waves x two), or 0 where the kernel that reads x from memory is as fast or faster. Measured on the
-// projections of the 1.7B, 8B and 32B shapes: very wide weights (the lm_head, a gate/up of 51200 rows) gain 10
-// to 20 % from 17 rows on (5 % with K = 2048, in the smaller workgroups, and only up to 32 rows); a gate/up of 24576 x 4096 gains 11 % at 64 rows and nothing below 48; narrow
-// weights cut along K (O, down, QKV) and short K (2048) lose up to 40 %, their workgroups being too short
-// to pay for the extra barrier a chunk.
-static int rows_kernel_tiles(int M, int N, int K, int gated) {
-  if (N >= 32768) return K >= 4096 ? 8 : (M <= 32 ? 6 : 0);
-  if (gated && M > 48 && N >= 16384 && K >= 4096) return 6;
-  return 0;
+// waves x two, 3: three waves x one), or 0 where another kernel is as fast or faster: the one that reads x from
+// memory, or above 32 rows the tiled product with 64-row tiles. Measured on the projections of the 1.7B, 8B and
+// 32B shapes at 20 to 64 rows:
+//   * very wide weights (the lm_head, a gate/up of 51200 rows): 10 to 25 % over the memory kernel up to 32
+//     rows; above, the tiled product is faster still;
+//   * a gate/up of 24576 x 4096: 7 % at 20 rows, 11 % at 32, 18 % at 48, 25 % at 64; of 12288 x 2048: 8 to 13 %
+//     up to 48 rows in the small workgroups;
+//   * weights cut along K (QKV, O, down): where the workgroups of six tiles fill the compute units in one
+//     round (200 to 256 of them: the 8B shape's QKV, the 32B's QKV and O) 7 to 24 %, also over the tiled
+//     product at 48 and 64 rows; with fewer workgroups (172 for a 4096-row weight) or short ranges the others win.
+static int rows_kernel_tiles(int M, int N, int K, int gated, int splits) {
+  if (M <= 16 || M > 64) return 0;
+  const int kblocks = (K + 31) / 32;
+  const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
+  if (K % 32 != 0 || per_wave % 4 != 0) return 0;      // the parts of K in which the sums are formed are whole chunks
+  if (N >= 32768) return M <= 32 ? (K >= 4096 ? 8 : 6) : 0;
+  if (gated) {
+    if (N >= 16384 && K >= 4096) return M <= 24 ? 3 : 6;
+    if (N >= 8192 && K >= 2048 && M <= 48) return 3;
+    return 0;
+  }
+  const long wgs = static_cast<long>(((N + 15) / 16 + 5) / 6) * splits;
+  return wgs >= 200 && wgs <= 256 && K / splits >= 1024 ? 6 : 0;
+}
+
+// The same for callers that choose between this product and the tiled one (packed weights).
+extern "C" int tie_skinny_rows_kernel_tiles(int M, int N, int K, int gated, int splits) {
+  return rows_kernel_tiles(M, N, K, gated, splits);
 }
 
 // Ranges of K that a product over w[N, K] is cut into when its caller takes partial sums: weights with
@@ -420,23 +495,24 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   // number of tiles a workgroup takes: up to 3 three waves x one tile, up to 6 three waves x two, else four x two.
   const int tiles = (N + 15) / 16;
   const bool rows_fit = static_cast<size_t>(M) * K * 2 < (1ull << 31);
-  const int by_rule = rows_kernel_tiles(M, N, K, gated);
-  if (packed && mt > 1 && rows_kernel && rows_fit && (by_rule != 0 || rows_forced)) {
+  const int by_rule = rows_kernel_tiles(M, N, K, gated, splits);
+  const bool whole_chunks = per_wave % 4 == 0;     // the parts of K in which the sums are formed end between chunks
+  if (packed && mt > 1 && rows_kernel && rows_fit && whole_chunks && (by_rule != 0 || rows_forced)) {
     const int asked = rows_forced && forced_rt != 0 ? forced_rt : (by_rule != 0 ? by_rule : 6);
     const int per_wg = asked <= 3 ? 3 : (asked <= 6 ? 6 : 8);
     const dim3 rgrid((tiles + per_wg - 1) / per_wg, splits);
-#define LAUNCH_ROWS(MT, RT, WAVES, TO)                                                                          \
-  skinny_rows_kernel<MT, RT, WAVES, TO><<<rgrid, WAVES * TIE_WAVE, 0, stream>>>(                                  \
+#define LAUNCH_ROWS(MT, RT, WAVES, U, DEPTH, TO)                                                                \
+  skinny_rows_kernel<MT, RT, WAVES, U, DEPTH, TO><<<rgrid, WAVES * TIE_WAVE, 0, stream>>>(                      \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
       gated, per_wave)
-#define LAUNCH_ROWS_TO(MT, RT, WAVES)                                 \
-  if (out_dtype == TIE_F32) LAUNCH_ROWS(MT, RT, WAVES, float);       \
-  else if (out_dtype == TIE_BF16) LAUNCH_ROWS(MT, RT, WAVES, bf16_t); \
+#define LAUNCH_ROWS_TO(MT, RT, WAVES, U, DEPTH)                                 \
+  if (out_dtype == TIE_F32) LAUNCH_ROWS(MT, RT, WAVES, U, DEPTH, float);       \
+  else if (out_dtype == TIE_BF16) LAUNCH_ROWS(MT, RT, WAVES, U, DEPTH, bf16_t); \
   else return TIE_BAD_ARGUMENT
 #define LAUNCH_ROWS_MT(MT)                                  \
-  if (per_wg == 8) { LAUNCH_ROWS_TO(MT, 2, 4); }            \
-  else if (per_wg == 6) { LAUNCH_ROWS_TO(MT, 2, 3); }       \
-  else { LAUNCH_ROWS_TO(MT, 1, 3); }
+  if (per_wg == 8) { LAUNCH_ROWS_TO(MT, 2, 4, 4, 3); }      \
+  else if (per_wg == 6) { LAUNCH_ROWS_TO(MT, 2, 3, 4, 3); } \
+  else { LAUNCH_ROWS_TO(MT, 1, 3, 4, 3); }
     if (mt == 2) { LAUNCH_ROWS_MT(2) } else { LAUNCH_ROWS_MT(4) }
 #undef LAUNCH_ROWS_MT
 #undef LAUNCH_ROWS_TO

@@ -74,6 +74,7 @@ _SIGNATURES = {
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
+        "tie_skinny_rows_kernel_tiles": [_c_int, _c_int, _c_int, _c_int, _c_int],
         "tie_skinny_gemm_bf16_with": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_void],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -491,17 +492,21 @@ _few_rows_memo: Dict[tuple, bool] = {}
 def decode_product_rows(M: int, w, gated: bool = False) -> bool:
     """Whether ``M`` rows against ``w`` go to the decode product (``skinny_gemm_bf16``) rather than the tiled one.
 
-    Up to 32 rows always, above 64 never; between, by the weight's shape and layout (the tiled product with
-    64-row tiles is the faster one over packed weights, except for gated products that are not very wide).
+    Up to 32 rows always, above 64 never; between, by the weight's shape and layout: the decode product where its
+    kernel that shares x through LDS is the measured best, else the tiled product with 64-row tiles over packed
+    weights, except for gated products that are not very wide.
     """
     if M <= 32 or M > 64:
         return M <= 32
     N, K = w.shape
-    key = (M > 32, N, K, isinstance(w, PackedWeight), bool(gated))
+    packed = isinstance(w, PackedWeight)
+    key = (M, N, K, packed, bool(gated))
     tiled = _few_rows_memo.get(key)
     if tiled is None:
-        tiled = _few_rows_memo[key] = bool(_lib("gemm_bf16").tie_gemm_bf16_wins_few_rows(
-            M, N, K, int(isinstance(w, PackedWeight)), int(gated)))
+        shares_x = packed and _lib("skinny_gemm_bf16").tie_skinny_rows_kernel_tiles(
+            M, N, K, int(gated), 1 if gated else skinny_splits(N, K)) != 0
+        tiled = _few_rows_memo[key] = not shares_x and bool(_lib("gemm_bf16").tie_gemm_bf16_wins_few_rows(
+            M, N, K, int(packed), int(gated)))
     return not tiled
 
 
