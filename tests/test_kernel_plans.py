@@ -26,6 +26,7 @@ def test_key_shares_never_exceed_what_the_merge_takes():
     assert kernels.decode_splits(1, 1, 65536, 16) == kernels.MAX_KEY_SPLITS
     # about 512 waves in shares of at least 128 keys where a wave keeps several tiles in flight
     assert kernels.decode_splits(8, 8, 4096) == 8 and kernels.decode_splits(64, 8, 4096) == 1
+    assert kernels.decode_splits(31, 8, 4096) == 3 and kernels.decode_splits(32, 8, 4096) == 1 and kernels.decode_splits(48, 8, 4096) == 2
     assert kernels.decode_splits(1, 8, 4096) == 32 and kernels.decode_splits(1, 8, 200) == 1
     for items in (1, 2, 5, 40, 300):
         for kv_heads in (1, 2, 8):

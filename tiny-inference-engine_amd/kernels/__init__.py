@@ -807,11 +807,14 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int, block_size
 
     Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take. With pages of 16
     positions or more the kernel keeps several tiles of keys in flight a wave, and about 512 waves (half
-    the GPU's wave slots) with shares of at least 128 keys measured best from batch 1 to 128; with smaller
-    pages a wave has one tile in flight and the GPU wants four times the waves.
+    the GPU's wave slots) with shares of at least 128 keys measured best from batch 1 to 128 (with exactly 256
+    (sequence, KV head) pairs one wave each walks its whole sequence and nothing is merged: 93 against 96 µs a
+    layer at batch 32 and 4096 keys; 384 pairs in one share each are a round and a half and lose 5 %); with
+    smaller pages a wave has one tile in flight and the GPU wants four times the waves.
     """
     if block_size >= 16:
-        by_occupancy = -(-512 // max(1, num_seqs * num_kv_heads))
+        pairs = max(1, num_seqs * num_kv_heads)
+        by_occupancy = 1 if pairs == 256 else -(-512 // pairs)    # a wave a compute unit: whole sequences, no merge
         by_length = max(1, max_context // 128)          # at least four 32-key tiles a share
         return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
     by_occupancy = -(-2048 // max(1, num_seqs * num_kv_heads))     # about 2048 waves ...
