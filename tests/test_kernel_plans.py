@@ -28,6 +28,10 @@ def test_key_shares_never_exceed_what_the_merge_takes():
     assert kernels.decode_splits(8, 8, 4096) == 8 and kernels.decode_splits(64, 8, 4096) == 1
     assert kernels.decode_splits(31, 8, 4096) == 3 and kernels.decode_splits(32, 8, 4096) == 1 and kernels.decode_splits(48, 8, 4096) == 2
     assert kernels.decode_splits(1, 8, 4096) == 32 and kernels.decode_splits(1, 8, 200) == 1
+    # where 512 waves would not spread evenly over 256 compute units, the count up to twice as large that does
+    assert kernels.decode_splits(24, 8, 4096) == 4 and kernels.decode_splits(40, 8, 4096) == 3      # 768 and 960 waves
+    assert kernels.decode_splits(12, 8, 4096) == 8 and kernels.decode_splits(20, 8, 4096) == 6      # 768 and 960
+    assert kernels.decode_splits(24, 8, 300) == 2 and kernels.decode_splits(56, 8, 4096) == 2       # short shares; 1344 are too many
     for items in (1, 2, 5, 40, 300):
         for kv_heads in (1, 2, 8):
             for group in (1, 3, 4, 8, 16):

@@ -806,17 +806,34 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int, block_size
     """How many ways the keys of each sequence are split so that a decode step fills the GPU.
 
     Never more than ``MAX_KEY_SPLITS``, which is what the kernel and its merge take. With pages of 16
-    positions or more the kernel keeps several tiles of keys in flight a wave, and about 512 waves (half
-    the GPU's wave slots) with shares of at least 128 keys measured best from batch 1 to 128 (with exactly 256
-    (sequence, KV head) pairs one wave each walks its whole sequence and nothing is merged: 93 against 96 µs a
-    layer at batch 32 and 4096 keys; 384 pairs in one share each are a round and a half and lose 5 %); with
-    smaller pages a wave has one tile in flight and the GPU wants four times the waves.
+    positions or more the kernel keeps several tiles of keys in flight a wave, a wave is a workgroup, and the
+    GPU holds 1024 of them at a time, four a compute unit. About 512 waves with shares of at least 128 keys
+    measured best from batch 1 to 128 where that many waves spread evenly; where they do not (24 sequences of 8
+    KV heads in 3 shares are 576 waves: two compute units in three carry two, the others three) up to twice the
+    shares are tried for the count that leaves the fewest compute units waiting, each further share weighed at
+    1 % for what it writes and the merge reads (batch 24 at 4096 keys: 4 shares, 73.5 against 82.8 µs a layer;
+    batch 40: 3 shares, 115 against 125; batch 12: 8 shares, 42 against 48). With exactly 256 (sequence, KV head)
+    pairs one wave each walks its whole sequence and nothing is merged (batch 32: 93 against 96 µs). With smaller
+    pages a wave has one tile in flight and the GPU wants four times the waves.
     """
     if block_size >= 16:
         pairs = max(1, num_seqs * num_kv_heads)
-        by_occupancy = 1 if pairs == 256 else -(-512 // pairs)    # a wave a compute unit: whole sequences, no merge
+        if pairs == 256:
+            return 1
         by_length = max(1, max_context // 128)          # at least four 32-key tiles a share
-        return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
+        most = min(by_length, MAX_KEY_SPLITS)
+        first = -(-512 // pairs)
+        if first >= most:
+            return max(1, most)
+        best, best_cost = first, None
+        for n in range(first, min(2 * first, most) + 1):
+            waves = pairs * n
+            if n > first and waves > 1024:
+                break
+            cost = -(-waves // 256) * 256 / waves * (1 + 0.01 * n)
+            if best_cost is None or cost < best_cost:
+                best, best_cost = n, cost
+        return best
     by_occupancy = -(-2048 // max(1, num_seqs * num_kv_heads))     # about 2048 waves ...
     if by_occupancy > 16:
         by_occupancy = -(-by_occupancy // 2)        # ... but half as many where that still leaves many shares to merge
