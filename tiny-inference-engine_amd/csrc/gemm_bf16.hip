@@ -437,40 +437,42 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
   };
 
-  // Slice j's x rows are issued after the barrier of slice j - 3 and its w rows before the barrier of
-  // slice j - 2; the first slices here. The host gives every range of K at least three slices.
+  // A stage is free once every wave has passed the barrier of the slice that read it, which stands in the
+  // middle of that slice (its last fragments are in registers by then). Slice j's x rows are asked for right
+  // after the barrier of slice j - 4, into the stage that slice has just left, and its w rows before the barrier
+  // of slice j - 3: the loads of two to three slices are in flight at any time (64 to 96 KB a workgroup of 256 x 256), which is what
+  // the latency of L2 asks for at a slice every 0.4 us. (One slice less ahead - 32 to 64 KB - the matrix cores
+  // waited a third of the time.) The first slices here; the host gives every range of K at least three.
   issue_x(0);
   issue_w(0);
   issue_x(1);
   issue_w(1);
   issue_x(2);
-  // Slice 0 has landed when at most slice 1's loads and slice 2's x rows (2 PA + PB) are still in flight;
-  // in the loop, at most one slice's (PA + PB).
-#define GD_WAIT_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ")\n\ts_barrier" ::: "memory")
-#define GD_WAIT_ALL_BARRIER(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
-  constexpr int FIRST_WAIT = 2 * PA + PB, STEADY_WAIT = PA + PB;
-  if constexpr (FIRST_WAIT == 12) GD_WAIT_BARRIER(12);
-  else if constexpr (FIRST_WAIT == 10) GD_WAIT_BARRIER(10);
-  else if constexpr (FIRST_WAIT == 8) GD_WAIT_BARRIER(8);
-  else if constexpr (FIRST_WAIT == 6) GD_WAIT_BARRIER(6);
-  else if constexpr (FIRST_WAIT == 4) GD_WAIT_BARRIER(4);
-  else static_assert(FIRST_WAIT == 12, "a tile shape without its wait count");
-  auto steady_wait = [&]() {
-    if constexpr (STEADY_WAIT == 8) GD_WAIT_ALL_BARRIER(8);
-    else if constexpr (STEADY_WAIT == 6) GD_WAIT_ALL_BARRIER(6);
-    else if constexpr (STEADY_WAIT == 5) GD_WAIT_ALL_BARRIER(5);
-    else if constexpr (STEADY_WAIT == 4) GD_WAIT_ALL_BARRIER(4);
-    else if constexpr (STEADY_WAIT == 3) GD_WAIT_ALL_BARRIER(3);
-    else GD_WAIT_ALL_BARRIER(0);
+  issue_w(2);
+  // s_waitcnt vmcnt(n) [lgkmcnt(0)], then the barrier (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
+  // lgkmcnt 11:8; a counter at its maximum is not waited for).
+  auto wait_barrier = [&](auto loads, auto lds_too) {
+    constexpr int n = decltype(loads)::value;
+    static_assert(n >= 0 && n < 64, "vmcnt has six bits");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt((n & 15) | ((n >> 4) << 14) | (7 << 4) | ((decltype(lds_too)::value ? 0 : 15) << 8));
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   };
+  using One = std::integral_constant<int, PA + PB>;
+  using Two = std::integral_constant<int, 2 * (PA + PB)>;
+  using None = std::integral_constant<int, 0>;
+  // Slice 0 has landed when at most the loads of slices 1 and 2 are outstanding.
+  wait_barrier(Two{}, std::false_type{});
   load_frags(stage(0), 0, 0);
+  if (3 < k_tiles) issue_x(3);
 
-  // One slice; its first fragments are in set 0 already. STEADY: slices up to kt + 3 exist, so the loads
-  // sit in straight-line code and exactly those of slice kt + 2 may still be in flight at the barrier.
+  // One slice; its first fragments are in set 0 already. STEADY: slices up to kt + 4 exist, so the loads
+  // sit in straight-line code and exactly those of slices kt + 2 and kt + 3 may still be in flight at the barrier.
   auto slice = [&](int kt, auto steady_tag) {
     constexpr bool STEADY = decltype(steady_tag)::value;
     load_frags(stage(kt), 1, 1);
-    if (STEADY || kt + 2 < k_tiles) issue_w(kt + 2);
+    if (STEADY || kt + 3 < k_tiles) issue_w(kt + 3);
     mfma_step(0);
     if (STEADY && BM == 256) {
 #pragma unroll
@@ -484,17 +486,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
     // My share of slice kt + 1 has landed and my reads of this stage are in registers; after the
     // barrier that holds for every wave.
-    if (STEADY || kt + 2 < k_tiles) {
-      steady_wait();
-    } else {
-      GD_WAIT_ALL_BARRIER(0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    if (STEADY || kt + 3 < k_tiles) wait_barrier(Two{}, std::true_type{});
+    else if (kt + 2 < k_tiles) wait_barrier(One{}, std::true_type{});
+    else wait_barrier(None{}, std::true_type{});
     if (STEADY || kt + 1 < k_tiles) load_frags(stage(kt + 1), 0, 0);
-    if (STEADY || kt + 3 < k_tiles) issue_x(kt + 3);
+    if (STEADY || kt + 4 < k_tiles) issue_x(kt + 4);
     mfma_step(1);
     if (STEADY && BM == 256) {
 #pragma unroll
@@ -520,8 +518,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   }
   for (; kt < k_tiles; ++kt) slice(kt, std::false_type{});
 
-#undef GD_WAIT_BARRIER
-#undef GD_WAIT_ALL_BARRIER
   const bool gated_n = EPI == 3;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
