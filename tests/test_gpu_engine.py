@@ -333,6 +333,29 @@ def test_cancel_release_and_callbacks(model_folders):
     assert engine.cache.num_free() == engine.cache.num_blocks
 
 
+def test_a_request_whose_sampling_the_kernels_cannot_take_is_refused_when_it_is_added(model_folders, monkeypatch):
+    """The drawing kernels take vocabularies up to a size of their own; a request that would need more is
+    refused with that size named, before anything runs, and a greedy request goes through."""
+    import tie_amd
+    from tie_amd import kernels
+    from tie_amd.errors import InvalidArgument
+
+    folder, cfg = model_folders["A"]
+    engine = make_engine(folder, 4)
+    monkeypatch.setattr(kernels, "MAX_FILTERED_VOCAB", cfg["vocab_size"] - 1)
+    with pytest.raises(InvalidArgument, match=f"top-k / top-p takes vocabularies of up to {cfg['vocab_size'] - 1}"):
+        engine.add_request([1, 2, 3], tie_amd.SamplingParams(temperature=0.7, top_k=5))
+    engine.add_request([1, 2, 3], tie_amd.SamplingParams(temperature=0.7, max_tokens=2))      # no filter: the other kernel
+    while engine.has_work():
+        engine.step()
+    monkeypatch.setattr(kernels, "MAX_SAMPLED_VOCAB", cfg["vocab_size"] - 1)
+    with pytest.raises(InvalidArgument, match="a temperature takes vocabularies"):
+        engine.add_request([1, 2, 3], tie_amd.SamplingParams(temperature=0.7))
+    engine.add_request([1, 2, 3], tie_amd.SamplingParams(max_tokens=2))
+    while engine.has_work():
+        engine.step()
+
+
 def test_device_sampling_matches_the_host_sampler():
     import numpy as np
     from tie_amd.sampling import DeviceSampler, RandomStream, SamplingParams, sample

@@ -105,6 +105,12 @@ class Engine:
         if not prompt:
             raise InvalidArgument("a request needs at least one prompt token")
         vocab = self.model.spec.vocab_size
+        if not params.greedy:
+            filtered = 0 < params.top_k < vocab or params.top_p < 1.0
+            most = kernels.MAX_FILTERED_VOCAB if filtered else kernels.MAX_SAMPLED_VOCAB
+            if vocab > most:
+                raise InvalidArgument(f"the sampling kernel for {'top-k / top-p' if filtered else 'a temperature'} takes "
+                                      f"vocabularies of up to {most} tokens, this model has {vocab}")
         if min(prompt) < 0 or max(prompt) >= vocab:
             bad = next(t for t in prompt if not 0 <= t < vocab)
             raise InvalidArgument(f"prompt token {bad} is not in the vocabulary of {vocab}")
