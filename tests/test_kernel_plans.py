@@ -32,6 +32,17 @@ def test_key_shares_never_exceed_what_the_merge_takes():
     assert kernels.decode_splits(24, 8, 4096) == 4 and kernels.decode_splits(40, 8, 4096) == 3      # 768 and 960 waves
     assert kernels.decode_splits(12, 8, 4096) == 8 and kernels.decode_splits(20, 8, 4096) == 6      # 768 and 960
     assert kernels.decode_splits(24, 8, 300) == 2 and kernels.decode_splits(56, 8, 4096) == 2       # short shares; 1344 are too many
+    # whatever the batch: between the count for 512 waves and twice that, more shares than that count only where
+    # the GPU holds all their waves at once, and shares of at least 128 keys
+    for seqs in range(1, 130):
+        for kv_heads in (1, 2, 4, 8):
+            for context in (200, 1024, 4096, 40000):
+                n = kernels.decode_splits(seqs, kv_heads, context)
+                pairs = seqs * kv_heads
+                first = min(-(-512 // pairs), max(1, context // 128), kernels.MAX_KEY_SPLITS)
+                assert (n == 1 and pairs == 256) or first <= n <= 2 * first, (seqs, kv_heads, context, n)
+                assert n == 1 or context // n >= 64, (seqs, kv_heads, context, n)
+                assert n <= first or pairs * n <= 1024, (seqs, kv_heads, context, n)
     for items in (1, 2, 5, 40, 300):
         for kv_heads in (1, 2, 8):
             for group in (1, 3, 4, 8, 16):
