@@ -12,7 +12,14 @@ context length; ``value`` is decoded tokens a second. The same line carries
   bf16 MFMA peak its flops reach;
 * ``roofline``: the bytes a decode step has to read (every weight it uses once, and the cache of
   the live requests) divided by its time, against the HBM peak;
-* ``points``: decoded tokens a second at batch 1 and at batch 64.
+* ``points``: decoded tokens a second at batch 1 and at batch 64, and for each of them (keys
+  ``decode_b1_...``) the step time, the bytes read and the same two fractions.
+
+Every decode point times the same ``--steps`` steps. ``ms_per_step`` and ``value`` come from the wall clock
+around exactly those steps; ``ms_per_step_median`` is the median of the steps' own times, taken from GPU
+events recorded after each. Beside the fractions of the published peaks (HBM 8 TB/s, 2.5 PFLOP/s) stand
+``measured_peak`` and ``frac_of_measured``: what a kernel that only reads cold memory, and one that only issues
+matrix instructions, reach on this very GPU in this process (``tie_amd.bench.peaks``).
 
 The sizes are those of a Qwen3-8B config.json; weights are random (N(0, 0.02), norm weights
 1 + U(-0.1, 0.1)) and token ids are uniform, since neither checkpoints nor datasets exist here.
@@ -123,7 +130,9 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
     The prompts are prefilled through the engine first (untimed). Sequences that finish their prompt
     early decode while the others still prefill, so every prompt is shortened by the number of steps
     the prefill phase takes: no sequence outgrows ``context`` before the timed steps are over.
-    Returns (seconds, mean context length over the timed steps and sequences, graph replays).
+    Returns (seconds, mean context length over the timed steps and sequences, graph replays, the median of
+    the steps' own times in seconds: a GPU event is recorded behind every step, and in the steady state, where
+    the GPU never waits for the host, the time between two of them is one step's).
     """
     import random
 
@@ -154,11 +163,16 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
         engine.step()
     torch.cuda.synchronize()
     first = sum(engine.sequence(i).num_computed + 1 for i in ids) / batch
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     start = time.perf_counter()
-    for _ in range(steps):
+    marks[0].record()
+    for k in range(steps):
         engine.step()
+        marks[k + 1].record()
     torch.cuda.synchronize()
     seconds = time.perf_counter() - start
+    own = sorted(marks[k].elapsed_time(marks[k + 1]) * 1e-3 for k in range(steps))
+    median = own[steps // 2] if steps % 2 else (own[steps // 2 - 1] + own[steps // 2]) / 2
     last = sum(engine.sequence(i).num_computed for i in ids) / batch
     assert all(engine.sequence(i).state == SeqState.DECODING for i in ids), "a sequence finished during the timed steps"
     assert max(engine.sequence(i).num_computed for i in ids) <= context
@@ -166,7 +180,7 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
     replays = engine.runner.graph_replays
     del engine
     torch.cuda.empty_cache()
-    return seconds, (first + last) / 2, replays
+    return seconds, (first + last) / 2, replays, median
 
 
 def measure_prefill(model, cfg, tokens, repeats=3):
@@ -264,19 +278,31 @@ def main():
     sampling = None
     if args.temperature > 0:
         sampling = {"temperature": args.temperature, "top_k": args.top_k, "top_p": args.top_p}
-    seconds, mean_context, replays = measure_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, chunk,
-                                                    sampling)
-    ms_per_step = seconds / args.steps * 1e3
-    value = args.batch * args.steps / seconds
-    step_bytes = weight_bytes_per_step(cfg, args.batch) + args.batch * mean_context * kv_bytes_per_token(cfg)
-    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
-    log(f"decode batch {args.batch}: {ms_per_step:.3f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s ({replays} replays)")
+    from tie_amd.bench.peaks import measured_peaks
 
+    peaks = measured_peaks()
+    log(f"this GPU: a streaming read reaches {peaks['hbm_read_gbs']:.0f} GB/s, matrix instructions on registers "
+        f"{peaks['mfma_bf16_tflops']:.0f} TFLOP/s")
+
+    def decode_point(batch):
+        """One decode measurement: ``--steps`` timed steps at ``batch``; the figures of its roofline."""
+        seconds, mean_context, replays, median = measure_decode(model, cfg, batch, args.context, args.steps,
+                                                                args.warmup, chunk, sampling)
+        ms = seconds / args.steps * 1e3
+        step_bytes = weight_bytes_per_step(cfg, batch) + batch * mean_context * kv_bytes_per_token(cfg)
+        achieved = step_bytes / (ms * 1e-3) / 1e9
+        log(f"decode batch {batch}: {ms:.3f} ms/step (median of the steps {median * 1e3:.3f}), "
+            f"{batch * args.steps / seconds:.1f} tok/s, {achieved:.0f} GB/s ({replays} replays)")
+        return {"tok_s": batch * args.steps / seconds, "ms": ms, "median_ms": median * 1e3, "gb": step_bytes / 1e9,
+                "gbs": achieved, "frac": achieved / PEAK_HBM_GBS, "frac_of_measured": achieved / peaks["hbm_read_gbs"]}
+
+    main_point = decode_point(args.batch)
     result = {
         "metric": f"decode tok/s @ batch {args.batch}, {shape_name} bf16 (plus prefill tok/s @ 2048 and batch 1/64 points)",
-        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "value": round(main_point["tok_s"], 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(main_point["ms"], 4),
+        "ms_per_step_median": round(main_point["median_ms"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
             "model": f"{shape_name} shape, random weights", "layers": layers_of_shape, "layers_run": cfg["num_hidden_layers"],
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
@@ -285,21 +311,31 @@ def main():
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
             "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
         },
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(main_point["gbs"], 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(main_point["frac"], 4), "bytes_gb": round(main_point["gb"], 3),
+                     "measured_peak": round(peaks["hbm_read_gbs"], 1),
+                     "frac_of_measured": round(main_point["frac_of_measured"], 4)},
     }
     if not args.skip_points:
         t = measure_prefill(model, cfg, PREFILL_TOKENS)
         flops = prefill_flops(cfg, PREFILL_TOKENS)
         result["prefill"] = {"value": round(PREFILL_TOKENS / t, 1), "tokens": PREFILL_TOKENS, "ms": round(t * 1e3, 3),
-                             "frac": round(flops / t / PEAK_FLOPS["bf16"], 4)}
+                             "frac": round(flops / t / PEAK_FLOPS["bf16"], 4),
+                             "measured_peak_tflops": round(peaks["mfma_bf16_tflops"], 1),
+                             "frac_of_measured": round(flops / t / 1e12 / peaks["mfma_bf16_tflops"], 4)}
         log(f"prefill {PREFILL_TOKENS}: {t * 1e3:.2f} ms, {PREFILL_TOKENS / t:.0f} tok/s, "
             f"{flops / t / 1e12:.1f} TFLOP/s")
         points = {}
         for b in (1, 64):
-            s, _, _ = measure_decode(model, cfg, b, args.context, max(8, args.steps // 2), args.warmup, chunk, sampling)
-            points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 2)
-            log(f"decode batch {b}: {points[f'decode_b{b}']:.1f} tok/s")
+            point = main_point if b == args.batch else decode_point(b)
+            key = f"decode_b{b}"
+            points[key] = round(point["tok_s"], 2)            # tokens a second; the rest of the point beside it
+            points[key + "_ms"] = round(point["ms"], 4)
+            points[key + "_median_ms"] = round(point["median_ms"], 4)
+            points[key + "_bytes_gb"] = round(point["gb"], 3)
+            points[key + "_gbs"] = round(point["gbs"], 1)
+            points[key + "_frac"] = round(point["frac"], 4)
+            points[key + "_frac_of_measured"] = round(point["frac_of_measured"], 4)
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0

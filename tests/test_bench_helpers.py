@@ -94,4 +94,8 @@ def test_the_report_sums_up_a_run():
     assert "requests 3" in text and "2 preemptions" in text and "1.50 sequences/step" in text and "ttft" in text
     assert set(json.loads(json.dumps(report_json(r)))) == {
         "requests", "prompt_tokens", "output_tokens", "wall_s", "requests_per_s", "output_tok_per_s", "total_tok_per_s",
-        "ttft_ms", "itl_ms", "e2e_ms", "mean_seqs_per_step", "steps", "preemptions"}      # report.cpp:73-86
+        "ttft_ms", "itl_ms", "e2e_ms", "mean_seqs_per_step", "steps", "preemptions",      # report.cpp:73-86
+        "tokens_read_late"}                                # ours: the token times carry one step of delay
+    assert "queued ahead" not in text
+    late = summarize(BenchRun([RequestTiming(0.0, 10, [1.0, 1.5])], 2.0, 2, 2, 0, tokens_read_late=True))
+    assert late.tokens_read_late and "queued ahead" in format_report(late)

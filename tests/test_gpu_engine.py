@@ -461,6 +461,8 @@ def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_fold
     plain_out, plain_reasons, _ = run(False)
     ahead_out, ahead_reasons, engine = run(True)
     assert engine.steps_launched_ahead > 10
+    if kv_blocks == 14:
+        assert engine.stats().preemptions > 0, "14 pages were meant to force evictions"
     for i in (0, 1, 3, 4, 5):                                  # (the cancelled one stops wherever it was)
         assert ahead_out[i] == plain_out[i] and ahead_reasons[i] == plain_reasons[i] == "length"
     # a stop token in the middle of some outputs
@@ -472,3 +474,32 @@ def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_fold
         assert s_ahead[i] == s_plain[i] and r_ahead[i] == r_plain[i]
         if r_plain[i] == "stop":
             assert s_plain[i][-1] == stop and stop not in s_plain[i][:-1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_eviction_while_tokens_are_unread_loses_no_request(model_folders, model_folders_bf16, dtype):
+    """Four requests decode in step, nobody waits, their tokens are read a step late, and all four need their second
+    page in the same step from a pool with one page to spare: requests are evicted with a token still unread, two
+    wait afterwards. Everyone finishes with the tokens of the engine that reads every step at once."""
+    import tie_amd
+
+    folder, cfg = (model_folders_bf16 if dtype == "bfloat16" else model_folders)["A"]
+    vocab = cfg["vocab_size"]
+    prompts = [prompt_of(3, vocab, salt) for salt in range(4)]
+
+    def run(ahead):
+        engine = make_engine(folder, 4, dtype=dtype, kv_blocks=5, max_seqs=4, max_tokens_per_step=16,
+                             launch_ahead=ahead, policy="fcfs")
+        ids = [engine.add_request(p, tie_amd.SamplingParams(max_tokens=9)) for p in prompts]
+        steps = 0
+        while engine.has_work():
+            engine.step()
+            steps += 1
+            assert steps < 500, "a request was lost: the engine never comes to an end"
+        assert engine.cache.num_free() == 5
+        return [engine.sequence(i).generated for i in ids], engine
+
+    plain_out, _ = run(False)
+    ahead_out, engine = run(True)
+    assert engine.ahead_replans > 0 and engine.stats().preemptions >= 2 and engine.steps_launched_ahead > 0
+    assert ahead_out == plain_out and all(len(out) == 9 for out in ahead_out)

@@ -966,6 +966,31 @@ def test_temperature_sampling_kernel_draws_what_the_host_rule_draws(vocab):
     assert three.tolist() == [-1, -2, 2]
 
 
+@pytest.mark.parametrize("vocab", [300, 5000, 151936])
+def test_temperature_sampling_never_picks_a_token_of_weight_zero(vocab):
+    """Uniform numbers at the very end of [0, 1): the walk ends at the last token that weighs anything, also where
+    rounding lets the kernel's sums disagree by an ulp; never at a -inf logit behind it, wherever the row's last
+    finite logit lies (in the last piece of 256, in an earlier one, in the first)."""
+    import numpy as np
+    from tie_amd import kernels
+
+    g = torch.Generator().manual_seed(vocab)
+    ends = sorted({1, 2, 255, 256, 257, vocab // 3, vocab - 257, vocab - 1, vocab} & set(range(1, vocab + 1)))
+    logits = torch.randn(len(ends), vocab, generator=g) * 2
+    for r, end in enumerate(ends):
+        logits[r, end:] = float("-inf")
+        logits[r, end - 1] = logits[r, :end].max()        # weighs at least 1 / vocab of the total at any temperature
+    dev = logits.cuda()
+    R = len(ends)
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    for inv_t in (1.0, 0.37, 2.9):
+        for u in (np.nextafter(1.0, 0.0), 1.0 - 2.0 ** -52, 1.0 - 2.0 ** -50, 1.0 - 1e-13):
+            kernels.sample_rows(dev, torch.full((R,), inv_t, device="cuda"),
+                                torch.full((R,), u, dtype=torch.float64, device="cuda"), out)
+            for r, end in enumerate(ends):
+                assert int(out[r]) == end - 1, f"row ending at {end}, uniform 1 - {1.0 - u:.3g}, 1/T {inv_t}"
+
+
 @pytest.mark.parametrize("vocab", [1000, 151936])
 def test_sampling_kernel_with_top_k_and_top_p_draws_what_the_host_rule_draws(vocab):
     """The kernel that selects instead of sorting, against ``sample`` (sort, sums in double precision), draw by
@@ -1066,3 +1091,33 @@ def test_gated_product_is_silu_gate_times_up(M, I, K):
         big = torch.empty_like(out)
         kernels.gemm_bf16(x, w, big, gated=True)                    # both kernels hold the same epilogue
         close(big, out.float(), 8e-3, "gated product, tiled kernel")
+
+
+def test_random_weights_are_the_same_bits_on_the_gpu_and_on_the_host():
+    """``random_tensor(..., device="cuda")`` against the host's draw, bit for bit: normal values (the central
+    rational function and the near tails with their root and logarithm series; the far tail beyond 6.7 standard
+    deviations comes up about once in 10^11 draws and is not met by sampling), norm weights, sizes that are no
+    multiple of the kernel's block, float32 and the two 16-bit roundings, and a whole model folder."""
+    from conftest import TINY_B
+    from tie_amd.models.builder import expected_tensors_for_config
+    from tie_amd.weights import random_init as ri
+    from tie_amd.weights.binder import TensorSpec
+
+    for shape, init, role in (((1537, 1031), ("normal", 0.02), "matrix"), ((3, 5, 7), ("normal", 1.0), "matrix"),
+                              ((4097,), ("one_plus_uniform", 0.1), "vector"), ((1,), ("normal", 0.5), "matrix")):
+        for dtype in (torch.float32, torch.bfloat16, torch.float16):
+            spec = TensorSpec("model.layers.3.x.weight", shape, role, init)
+            host = ri.random_tensor(spec, 17, dtype, "cpu")
+            dev = ri.random_tensor(spec, 17, dtype, "cuda")
+            assert dev.is_cuda and dev.dtype == dtype and tuple(dev.shape) == shape
+            same = torch.equal(dev.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                               host.view(torch.int16 if dtype != torch.float32 else torch.int32))
+            assert same, f"{shape} {init} {dtype}: {int((dev.cpu() != host).sum())} elements differ"
+    tails = ri.random_tensor(TensorSpec("t", (1 << 22,), "matrix", ("normal", 1.0)), 1, torch.float32, "cuda")
+    assert float(tails.abs().max()) > 4.5                      # the tail branch ran (and matched above at 1.6 M values)
+    specs = [s for s in expected_tensors_for_config(TINY_B) if not s.optional]
+    on_host = dict(ri.random_tensors(specs, 5, torch.bfloat16, "cpu", vector_dtype=torch.float32))
+    on_gpu = dict(ri.random_tensors(specs, 5, torch.bfloat16, "cuda", vector_dtype=torch.float32))
+    assert list(on_host) == list(on_gpu)
+    for name, t in on_host.items():
+        assert torch.equal(on_gpu[name].cpu().float(), t.float()), name

@@ -245,13 +245,13 @@ def register_toy_parts():
     from tie_amd.cache.spec import FixedState
     from tie_amd.parts import FeedForward, Mixer, Position, TensorSpec, register_part
 
-    @register_part("mixer", "toy_decay")
-    class ToyDecayMixer(Mixer):
+    @register_part("mixer", "toy_decay_undeclared")
+    class ToyDecayMixerThatSaysNothing(Mixer):
         """s_t = decay * s_{t-1} + W_in h_t ; out_t = W_out s_t, with s kept per request in a state slot.
 
-        It walks the step's sequences on the host, so a recording of it would hold one step's slots for good."""
-
-        capturable = False
+        It walks the step's sequences on the host, so a recording of it would hold one step's slots for good -
+        and it is written as by someone who never heard of recording: it says nothing about ``capturable``.
+        The default must keep it out of HIP graphs."""
 
         def __init__(self, params):
             super().__init__(params)
@@ -277,6 +277,14 @@ def register_toy_parts():
                     state.mul_(self.decay).add_(u[t])
                     residual[t] += state @ self.w_out.float().T
                 row += n
+
+    assert not any("capturable" in vars(c) for c in ToyDecayMixerThatSaysNothing.__mro__ if c.__module__ == __name__)
+
+    @register_part("mixer", "toy_decay")
+    class ToyDecayMixer(ToyDecayMixerThatSaysNothing):
+        """The same, by an author who knows that it cannot be recorded and says so."""
+
+        capturable = False
 
     @register_part("mixer", "toy_decay_on_device")
     class ToyDecayMixerOnDevice(ToyDecayMixer):
@@ -341,6 +349,8 @@ def register_toy_parts():
     class ToyShiftPosition(Position):
         """Not a rotation: adds position * slope to the first dimension of every query and key head."""
 
+        capturable = True         # torch operations on the step's device arrays only
+
         def __init__(self, params):
             super().__init__(params)
             self.slope = params["slope"]
@@ -356,6 +366,7 @@ def unregister_toy_parts():
 
     unregister_part("mixer", "toy_decay")
     unregister_part("mixer", "toy_decay_on_device")
+    unregister_part("mixer", "toy_decay_undeclared")
     unregister_part("feed_forward", "toy_routed")
     unregister_part("position", "toy_shift")
 
@@ -369,7 +380,7 @@ def toy_spec(cfg):
     layers = []
     for l, kind in enumerate(cfg["mixers"]):
         p = f"layers.{l}."
-        if kind in ("decay", "decay_on_device"):
+        if kind in ("decay", "decay_on_device", "decay_undeclared"):
             mixer = PartSpec("toy_" + kind, {"hidden": D, "width": cfg["state_width"], "decay": cfg["decay"],
                                            "names": {"in": p + "mix.in", "out": p + "mix.out"}})
         else:
@@ -401,7 +412,7 @@ def toy_plain(weights, cfg, tokens):
     for l, kind in enumerate(cfg["mixers"]):
         p = f"layers.{l}."
         h = plain.rms_norm(x, weights[p + "n1"], cfg["eps"])
-        if kind in ("decay", "decay_on_device"):
+        if kind in ("decay", "decay_on_device", "decay_undeclared"):
             u = plain.linear(h, weights[p + "mix.in"])
             s = torch.zeros(cfg["state_width"], dtype=F64)
             out = []
@@ -495,11 +506,13 @@ def changing_live_sets(requests, head, subsets):
     return steps
 
 
-@pytest.mark.parametrize("kind", ["recorded", "eager"])
+@pytest.mark.parametrize("kind", ["recorded", "eager", "undeclared"])
 def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, kind):
     """The serving precision, where decode-only steps are recorded and replayed. A model whose parts all read
     the step on the device is recorded, and replays must follow the step's slots as the live set changes; a
-    model with one part that reads the step on the host (or waits for the GPU) must not be recorded at all."""
+    model with one part that reads the step on the host (or waits for the GPU) must not be recorded at all -
+    whether that part says so ("eager") or says nothing ("undeclared": every other part of that model could be
+    recorded, so only the default keeps the host-side walk over the state slots out of a graph)."""
     import tie_amd
     from tie_amd.config.registry import register_architecture, unregister_architecture
     from tie_amd.engine.replay import TraceReplayer
@@ -513,6 +526,8 @@ def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, k
                "eps": 1e-5, "max_positions": 256, "experts": 5, "top_k": 2, "expert_width": 24}
         if kind == "recorded":
             cfg.update(mixers=["decay_on_device", "attention", "decay_on_device"], feed_forwards=["dense"] * 3)
+        elif kind == "undeclared":
+            cfg.update(mixers=["decay_on_device", "attention", "decay_undeclared"], feed_forwards=["dense"] * 3)
         else:
             cfg.update(mixers=["decay", "attention", "decay_on_device"], feed_forwards=["dense", "routed", "dense"])
         folder = write_random_model(tmp_path / "toy", cfg, seed=4, dtype="bfloat16")

@@ -63,18 +63,45 @@ def test_sizes_no_kernel_takes_are_refused_when_the_model_is_built():
     Model(build_qwen3_spec(Qwen3Config.from_json(dict(TINY_A, head_dim=512))))
 
 
-def test_a_float16_cache_is_refused_when_it_is_made():
-    from tie_amd.cache.manager import CacheManager
-    from tie_amd.cache.spec import plan_cache
+def test_the_cache_has_a_precision_of_its_own_where_a_kernel_takes_the_pair():
+    """float32 arithmetic runs over float32, bfloat16 or float16 pages (the reference's KVCacheConfig.dtype,
+    src/kv/paged_kv_cache.h:18-25); the matrix-core kernels read bfloat16 pages only. What no kernel takes is
+    refused when the engine is made, by name, before any weight is read."""
+    from tie_amd import kernels
+    from tie_amd.api import create_engine
+    from tie_amd.engine.replay import TraceReplayer
     from tie_amd.errors import InvalidArgument
+
+    assert kernels.cache_dtype_for("float32") == "float32" and kernels.cache_dtype_for("bfloat16") == "bfloat16"
+    assert kernels.cache_dtype_for("float32", "bf16") == "bfloat16"
+    assert kernels.cache_dtype_for("float32", "float16") == "float16"
+    assert kernels.cache_dtype_for("bfloat16", "bfloat16") == "bfloat16"
+    for mode, asked, words in (("bfloat16", "float32", "bfloat16 arithmetic over a float32 cache"),
+                               ("bfloat16", "float16", "bfloat16 arithmetic over a float16 cache"),
+                               ("float32", "int8", "float32, bfloat16 or float16")):
+        with pytest.raises(InvalidArgument, match=words):
+            kernels.cache_dtype_for(mode, asked)
+    # the folder does not exist: the refusal comes first
+    with pytest.raises(InvalidArgument, match="over a float32 cache"):
+        create_engine("/nonexistent/model", dtype="bfloat16", kv_dtype="float32")
+    with pytest.raises(InvalidArgument, match="over a float16 cache"):
+        TraceReplayer.from_folder("/nonexistent/model", "bfloat16", 64, kv_dtype="float16")
+
+
+def test_cache_pages_are_sized_by_the_cache_dtype():
+    from tie_amd.cache.manager import CacheManager
     from tie_amd.config.qwen3 import Qwen3Config
+    from tie_amd.errors import InvalidArgument
     from tie_amd.models import Model
     from tie_amd.models.qwen3 import build_qwen3_spec
     from conftest import TINY_A
 
-    model = Model(build_qwen3_spec(Qwen3Config.from_json(TINY_A)))
-    with pytest.raises(InvalidArgument, match="float16"):
-        CacheManager(model.cache_plan, block_size=4, num_blocks=8, dtype="float16")
+    plan = Model(build_qwen3_spec(Qwen3Config.from_json(TINY_A))).cache_plan
+    sizes = {d: CacheManager(plan, block_size=4, num_blocks=8, dtype=d).bytes_per_block
+             for d in ("float32", "bfloat16", "float16")}
+    assert sizes["float32"] == 2 * sizes["bfloat16"] == 2 * sizes["float16"] == 2 * 2 * 2 * 4 * 16 * 4
+    with pytest.raises(InvalidArgument, match="int8"):
+        CacheManager(plan, block_size=4, num_blocks=8, dtype="int8")
 
 
 TILE_ROWS_COLS = {4: (256, 256), 5: (256, 128), 6: (128, 256), 7: (128, 128)}

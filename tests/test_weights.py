@@ -171,3 +171,40 @@ def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
     assert float(n.min()) >= 0.9 and float(n.max()) <= 1.1 and float(n.std()) > 0.01  # 1 + U(-0.1, 0.1)
     with pytest.raises(InvalidArgument):
         write_random_model(tmp_path / "d", TINY_B, seed=1, dtype="int8")
+
+
+def test_a_random_element_depends_on_its_key_and_index_alone():
+    """The generator is counter-based: element i of a tensor is a function of (seed, name, i), so a tensor's
+    prefix does not change with its length, with the pieces it is drawn in or with the other tensors around it,
+    and a GPU can draw the same bits element by element (tests/test_gpu_kernels.py checks that it does)."""
+    import numpy as np
+    from scipy import stats
+    from tie_amd.weights import random_init as ri
+    from tie_amd.weights.binder import TensorSpec
+
+    long = ri.random_tensor(TensorSpec("w", (3, 50_000), "matrix", ("normal", 0.02)), 9, torch.float32).flatten()
+    short = ri.random_tensor(TensorSpec("w", (1000,), "matrix", ("normal", 0.02)), 9, torch.float32)
+    assert torch.equal(long[:1000], short)
+    old = ri._CHUNK
+    try:
+        ri._CHUNK = 777                                    # drawn in other pieces: the same values
+        pieces = ri.random_tensor(TensorSpec("w", (150_000,), "matrix", ("normal", 0.02)), 9, torch.float32)
+    finally:
+        ri._CHUNK = old
+    assert torch.equal(pieces, long)
+    other_name = ri.random_tensor(TensorSpec("v", (1000,), "matrix", ("normal", 0.02)), 9, torch.float32)
+    other_seed = ri.random_tensor(TensorSpec("w", (1000,), "matrix", ("normal", 0.02)), 10, torch.float32)
+    assert not torch.equal(short, other_name) and not torch.equal(short, other_seed)
+    # the distribution: N(0, 0.02) by the inverse distribution function, tails included
+    z = long.double().numpy() / 0.02
+    assert stats.kstest(z, "norm").pvalue > 1e-3
+    assert abs(float((np.abs(z) > 3).mean()) - 0.0027) < 0.001 and float(np.abs(z).max()) > 3.8
+    # the inverse distribution function itself against the library's, and the series that stands in for log
+    p = np.concatenate([np.logspace(-16, -1, 500), np.linspace(0.05, 0.95, 1001), 1.0 - np.logspace(-15, -1, 500)])
+    want = stats.norm.ppf(p)
+    assert float(np.max(np.abs(ri._normal_of(p) - want) / np.maximum(1e-3, np.abs(want)))) < 1e-13
+    x = np.concatenate([np.logspace(-300, -2, 2000), np.linspace(1e-3, 0.999, 2000)])
+    assert float(np.max(np.abs(ri._log(x) - np.log(x)) / np.abs(np.log(x)))) < 1e-15
+    u = ri.random_tensor(TensorSpec("n", (20_000,), "vector", ("one_plus_uniform", 0.1)), 9, torch.float32)
+    assert 0.9 <= float(u.min()) < 0.9001 and 1.0999 < float(u.max()) <= 1.1 and abs(float(u.mean()) - 1.0) < 2e-3
+    assert stats.kstest((u.double().numpy() - 0.9) / 0.2, "uniform").pvalue > 1e-3

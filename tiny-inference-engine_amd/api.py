@@ -11,13 +11,14 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+from . import kernels
 from .cache.manager import CacheManager
 from .engine.engine import Engine
 from .engine.scheduler import BatchScheduler, SchedulerConfig
 from .engine.serving import ServingConfig
 from .models.builder import Model, load_model
 from .sampling.params import SamplingParams
-from .weights.binder import FLOAT32, normalize_mode
+from .weights.binder import normalize_mode
 
 DEFAULT_KV_BYTES = 4 << 30  # the reference's default KV budget (src/cli/args.h:24)
 
@@ -26,16 +27,21 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
                   block_size: int = 16, max_seqs: int = 64, max_tokens_per_step: int = 512, prefill_chunk: int = 0,
                   policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1,
                   stop_tokens: Sequence[int] = (), max_seq_len: Optional[int] = None,
-                  device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead: bool = True) -> Engine:
+                  device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead: bool = True,
+                  kv_dtype: Optional[str] = None) -> Engine:
     """``model`` is a folder (config.json + safetensors) or a Model that is already loaded.
 
     ``use_graphs`` False runs every step eagerly; None (the default) records decode-only steps into HIP
     graphs in bfloat16 mode when every part of the model allows it. ``launch_ahead``: in the steady state of
     decoding the next step is queued before the last one's tokens are read (``Engine``'s module text says how);
-    tokens then appear one ``step()`` later."""
+    tokens then appear one ``step()`` later. ``kv_dtype``: the precision of the cached keys and values, by
+    default that of ``dtype``; float32 arithmetic also runs over a bfloat16 or float16 cache (the reference's
+    arrangement, ``src/kv/paged_kv_cache.h:18-25``). A pair no kernel takes is refused here, before anything
+    is loaded."""
+    mode = model.mode if isinstance(model, Model) else normalize_mode(dtype)
+    cache_dtype = kernels.cache_dtype_for(mode, kv_dtype)
     if not isinstance(model, Model):
-        model = load_model(model, normalize_mode(dtype), device)
-    cache_dtype = "float32" if model.mode == FLOAT32 else "bfloat16"
+        model = load_model(model, mode, device)
     if kv_blocks is None and kv_mem is None:
         kv_mem = DEFAULT_KV_BYTES
     context = min(model.spec.max_positions, max_seq_len) if max_seq_len else model.spec.max_positions

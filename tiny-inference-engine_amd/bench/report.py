@@ -32,6 +32,7 @@ class BenchRun:
     steps: int
     seqs_scheduled: int
     preemptions: int
+    tokens_read_late: bool = False        # the engine queued decode steps ahead: a token's time is one step late
 
 
 @dataclasses.dataclass
@@ -49,6 +50,9 @@ class BenchReport:
     mean_seqs_per_step: float = 0.0
     steps: int = 0
     preemptions: int = 0
+    # Not among the reference's fields: whether the engine read a decode step's tokens while the next step ran
+    # (``launch_ahead``). Token times (ttft, itl, e2e) then carry one step of delay that throughput does not.
+    tokens_read_late: bool = False
 
 
 def percentile(values: Sequence[float], p: float) -> float:
@@ -71,7 +75,7 @@ def _p50_p90_p99_ms(seconds: Sequence[float]) -> Dict[str, float]:
 def summarize(run: BenchRun) -> BenchReport:
     first, gaps, whole = [], [], []
     report = BenchReport(requests=len(run.requests), wall_s=run.wall_seconds, steps=run.steps,
-                         preemptions=run.preemptions)
+                         preemptions=run.preemptions, tokens_read_late=run.tokens_read_late)
     for timing in run.requests:
         report.prompt_tokens += timing.prompt_len
         report.output_tokens += len(timing.token_times)
@@ -98,7 +102,9 @@ def format_report(r: BenchReport) -> str:
             f"tokens   {r.prompt_tokens} prompt + {r.output_tokens} output  |  output {r.output_tok_per_s:.1f} tok/s"
             f"  |  total {r.total_tok_per_s:.1f} tok/s\n"
             + row("ttft", r.ttft_ms) + row("itl", r.itl_ms) + row("e2e", r.e2e_ms) +
-            f"steps    {r.steps}  |  {r.mean_seqs_per_step:.2f} sequences/step  |  {r.preemptions} preemptions\n")
+            f"steps    {r.steps}  |  {r.mean_seqs_per_step:.2f} sequences/step  |  {r.preemptions} preemptions\n"
+            + ("note     decode steps were queued ahead: every token above is timed one step after it existed "
+               "(--no-launch-ahead times them as they appear)\n" if r.tokens_read_late else ""))
 
 
 def report_json(r: BenchReport) -> dict:

@@ -59,4 +59,4 @@ def run_workload(engine: Engine, requests: Sequence[BenchRequest], sampling: Opt
     for seq_id in list(of_sequence):
         engine.release(seq_id)
     return BenchRun(timings, wall, after.steps - before.steps, after.seqs_scheduled - before.seqs_scheduled,
-                    after.preemptions - before.preemptions)
+                    after.preemptions - before.preemptions, tokens_read_late=bool(getattr(engine, "launch_ahead", False)))

@@ -37,7 +37,9 @@ from ..errors import CapacityError, InvalidArgument
 from .block_pool import BlockPool
 from .spec import CachePlan, FixedState, PagedKV
 
-_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}       # what the kernels read and write
+# What the kernels read and write; which of them goes with which compute mode is the kernels' to say
+# (``kernels.cache_dtype_for``).
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
 _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
 _INT32_MAX = 2 ** 31 - 1
 FREED = -1  # table entry of a page that a window has passed and that was given back

@@ -34,6 +34,8 @@ generate options:
   --prompt-file FILE       read the prompt token ids from FILE instead
   --device hip             compute device (default hip; there is no CPU path)
   --dtype D                bfloat16 (default) or float32
+  --kv-dtype D             precision of the cached keys and values: that of --dtype by default; float32
+                           arithmetic also runs over bfloat16 or float16 pages
   --temp T                 sampling temperature, 0 = greedy (default 0.7)
   --top-k K                keep the K most likely tokens, 0 = off (default 20)
   --top-p P                nucleus sampling threshold (default 0.8)
@@ -49,7 +51,7 @@ generate options:
   --policy fcfs|srpt-aging admission order (default srpt-aging)
   --aging N                srpt-aging priority gained per step waited, in tokens (default 16)
 
-bench options (and -m, --device, --dtype, --temp (default 0), --top-k, --top-p, --seed, --kv-mem, --kv-blocks,
+bench options (and -m, --device, --dtype, --kv-dtype, --temp (default 0), --top-k, --top-p, --seed, --kv-mem, --kv-blocks,
 --block-size, --max-seqs, --max-tokens-per-step, --prefill-chunk, --policy, --aging as above; --seed also seeds
 the synthetic workload and the arrivals):
   --prompts FILE           JSONL, one {"prompt_ids": [...], "max_tokens": N} per line
@@ -59,6 +61,9 @@ the synthetic workload and the arrivals):
   --max-tokens N           output tokens for JSONL lines without max_tokens (default 128)
   --rate R                 requests per second, Poisson arrivals; inf = all at once (default inf)
   --json                   print the report as one JSON object
+  --no-launch-ahead        read every step's tokens before the next step is queued: token times are then the
+                           moments the tokens exist (by default a decode step is queued before the one before
+                           it is read, which is faster and shows every token one step late)
 """
 
 
@@ -68,6 +73,7 @@ class GenerateOptions:
     prompt: List[int] = dataclasses.field(default_factory=list)
     device: str = "hip"
     dtype: str = "bfloat16"
+    kv_dtype: Optional[str] = None
     sampling: SamplingParams = dataclasses.field(
         default_factory=lambda: SamplingParams(temperature=0.7, top_k=20, top_p=0.8))
     stop_ids: List[int] = dataclasses.field(default_factory=list)
@@ -153,6 +159,10 @@ def _engine_flag(flag: str, flags: _Flags, o) -> bool:
         o.dtype = flags.value()
         if o.dtype not in ("bfloat16", "float32", "bf16", "fp32"):
             raise InvalidArgument(f"--dtype must be bfloat16 or float32, got '{o.dtype}'")
+    elif flag == "--kv-dtype":
+        o.kv_dtype = flags.value()
+        if o.kv_dtype not in ("float32", "fp32", "bfloat16", "bf16", "float16", "fp16"):
+            raise InvalidArgument(f"--kv-dtype must be float32, bfloat16 or float16, got '{o.kv_dtype}'")
     elif flag == "--temp":
         o.sampling.temperature = parse_float(flag, flags.value())
     elif flag == "--top-k":
@@ -232,6 +242,8 @@ class BenchOptions:
     rate: float = math.inf
     device: str = "hip"
     dtype: str = "bfloat16"
+    kv_dtype: Optional[str] = None
+    launch_ahead: bool = True
     sampling: SamplingParams = dataclasses.field(default_factory=lambda: SamplingParams(temperature=0.0))
     kv_bytes: int = 4 << 30
     kv_blocks: Optional[int] = None
@@ -274,6 +286,8 @@ def parse_bench_args(args: Sequence[str]) -> BenchOptions:
                 raise InvalidArgument(f"--rate must be positive or inf, got '{text}'")
         elif flag == "--json":
             o.json = True
+        elif flag == "--no-launch-ahead":
+            o.launch_ahead = False
         else:
             raise InvalidArgument(f"unknown option '{flag}'")
     if not o.model:

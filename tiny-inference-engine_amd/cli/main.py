@@ -26,8 +26,8 @@ def run_generate(argv: Sequence[str]) -> int:
     if not torch.cuda.is_available():
         raise KernelUnavailable("no GPU is visible: this engine runs on HIP only")
     load_start = time.perf_counter()
-    engine = create_engine(opt.model, dtype=opt.dtype, kv_mem=opt.kv_bytes, kv_blocks=opt.kv_blocks,
-                           block_size=opt.block_size, max_seqs=opt.max_seqs,
+    engine = create_engine(opt.model, dtype=opt.dtype, kv_dtype=opt.kv_dtype, kv_mem=opt.kv_bytes,
+                           kv_blocks=opt.kv_blocks, block_size=opt.block_size, max_seqs=opt.max_seqs,
                            max_tokens_per_step=opt.max_tokens_per_step, prefill_chunk=opt.prefill_chunk,
                            policy=opt.policy, aging=opt.aging, stop_tokens=opt.stop_ids)
     load_seconds = time.perf_counter() - load_start
@@ -77,10 +77,10 @@ def run_bench(argv: Sequence[str]) -> int:
 
     if not torch.cuda.is_available():
         raise KernelUnavailable("no GPU is visible: this engine runs on HIP only")
-    engine = create_engine(opt.model, dtype=opt.dtype, kv_mem=opt.kv_bytes, kv_blocks=opt.kv_blocks,
-                           block_size=opt.block_size, max_seqs=opt.max_seqs,
+    engine = create_engine(opt.model, dtype=opt.dtype, kv_dtype=opt.kv_dtype, kv_mem=opt.kv_bytes,
+                           kv_blocks=opt.kv_blocks, block_size=opt.block_size, max_seqs=opt.max_seqs,
                            max_tokens_per_step=opt.max_tokens_per_step, prefill_chunk=opt.prefill_chunk,
-                           policy=opt.policy, aging=opt.aging)
+                           policy=opt.policy, aging=opt.aging, launch_ahead=opt.launch_ahead)
     vocab = engine.model.spec.vocab_size
     if opt.synthetic:
         requests = synthetic_requests(opt.synthetic, opt.prompt_len, opt.output_len, vocab, opt.sampling.seed)

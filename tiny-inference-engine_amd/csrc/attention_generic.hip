@@ -125,6 +125,7 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
   if (q_dtype == TIE_F32 && cache_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (q_dtype == TIE_BF16 && cache_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (q_dtype == TIE_F32 && cache_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(float, bf16_t, float);
+  else if (q_dtype == TIE_F32 && cache_dtype == TIE_F16 && out_dtype == TIE_F32) LAUNCH(float, f16_t, float);
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH
   return tie_launch_status();

@@ -8,6 +8,7 @@
 // Element type codes of the C interface.
 #define TIE_F32 0
 #define TIE_BF16 1
+#define TIE_F16 2   // a cache of keys and values only (beside float32 arithmetic)
 
 // Error codes of the C interface (besides hipError_t values, which are > 0).
 #define TIE_OK 0
@@ -16,6 +17,7 @@
 #define TIE_WAVE 64
 
 typedef uint16_t bf16_t;  // raw bfloat16 bits
+typedef _Float16 f16_t;   // IEEE half precision, converted by the hardware (round to nearest even)
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
@@ -41,8 +43,13 @@ __device__ __forceinline__ float load_as_float<float>(const float* p) { return *
 template <>
 __device__ __forceinline__ float load_as_float<bf16_t>(const bf16_t* p) { return bf16_to_float(*p); }
 
+template <>
+__device__ __forceinline__ float load_as_float<f16_t>(const f16_t* p) { return static_cast<float>(*p); }
+
 template <typename T>
 __device__ __forceinline__ void store_from_float(T* p, float v);
+template <>
+__device__ __forceinline__ void store_from_float<f16_t>(f16_t* p, float v) { *p = static_cast<f16_t>(v); }
 template <>
 __device__ __forceinline__ void store_from_float<float>(float* p, float v) { *p = v; }
 template <>

@@ -185,6 +185,105 @@ extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_
   return tie_launch_status();
 }
 
+// ------------------------------------------------------------ random weights
+// Element i of a tensor is a function of (key, i) alone: the 64-bit mix of key + (i + 1) * 0x9E3779B97F4A7C15
+// (the SplitMix64 step) gives 52 bits of a uniform number u in (0, 1), and a normal value is the inverse normal
+// distribution function of u by Wichura's algorithm AS 241 (PPND16: rational functions, a logarithm and a root
+// in the tails). Every operation below is an IEEE double addition, multiplication, division or square root with
+// nothing contracted into a fused multiply-add, and the logarithm is a fixed series of such operations, so the
+// host (weights/random_init.py, the same steps in numpy) and the GPU draw the same bits.
+__device__ __forceinline__ unsigned long long random_mix(unsigned long long key, unsigned long long i) {
+  unsigned long long z = key + (i + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+__device__ double random_log(double x) {           // x in (0, 1); log(m * 2^e) = 2 atanh((m - 1) / (m + 1)) + e ln 2
+#pragma clang fp contract(off)
+  int e;
+  double m = frexp(x, &e);                         // m in [0.5, 1), exact
+  if (m < 0.70710678118654752440) {
+    m = m * 2.0;
+    e -= 1;
+  }
+  const double s = (m - 1.0) / (m + 1.0), s2 = s * s;
+  double series = 1.0 / 27.0;
+  series = series * s2 + 1.0 / 25.0;
+  series = series * s2 + 1.0 / 23.0;
+  series = series * s2 + 1.0 / 21.0;
+  series = series * s2 + 1.0 / 19.0;
+  series = series * s2 + 1.0 / 17.0;
+  series = series * s2 + 1.0 / 15.0;
+  series = series * s2 + 1.0 / 13.0;
+  series = series * s2 + 1.0 / 11.0;
+  series = series * s2 + 1.0 / 9.0;
+  series = series * s2 + 1.0 / 7.0;
+  series = series * s2 + 1.0 / 5.0;
+  series = series * s2 + 1.0 / 3.0;
+  series = series * s2 + 1.0;
+  return 2.0 * s * series + static_cast<double>(e) * 0.69314718055994530942;
+}
+
+#define RANDOM_POLY(c0, c1, c2, c3, c4, c5, c6, c7, r) \
+  ((((((((c7) * (r) + (c6)) * (r) + (c5)) * (r) + (c4)) * (r) + (c3)) * (r) + (c2)) * (r) + (c1)) * (r) + (c0))
+
+__device__ double random_normal_of(double p) {     // AS 241, PPND16
+#pragma clang fp contract(off)
+  const double q = p - 0.5;
+  if (fabs(q) <= 0.425) {
+    const double r = 0.180625 - q * q;
+    const double num = RANDOM_POLY(3.3871328727963666080, 1.3314166789178437745e2, 1.9715909503065514427e3,
+                                   1.3731693765509461125e4, 4.5921953931549871457e4, 6.7265770927008700853e4,
+                                   3.3430575583588128105e4, 2.5090809287301226727e3, r);
+    const double den = RANDOM_POLY(1.0, 4.2313330701600911252e1, 6.8718700749205790830e2, 5.3941960214247511077e3,
+                                   2.1213794301586595867e4, 3.9307895800092710610e4, 2.8729085735721942674e4,
+                                   5.2264952788528545610e3, r);
+    return q * num / den;
+  }
+  double r = q < 0.0 ? p : 1.0 - p;
+  r = __dsqrt_rn(-random_log(r));
+  double v;
+  if (r <= 5.0) {
+    r = r - 1.6;
+    const double num = RANDOM_POLY(1.42343711074968357734, 4.63033784615654529590, 5.76949722146069140550,
+                                   3.64784832476320460504, 1.27045825245236838258, 2.41780725177450611770e-1,
+                                   2.27238449892691845833e-2, 7.74545014278341407640e-4, r);
+    const double den = RANDOM_POLY(1.0, 2.05319162663775882187, 1.67638483018380384940, 6.89767334985100004550e-1,
+                                   1.48103976427480074590e-1, 1.51986665636164571966e-2, 5.47593808499534494600e-4,
+                                   1.05075007164441684324e-9, r);
+    v = num / den;
+  } else {
+    r = r - 5.0;
+    const double num = RANDOM_POLY(6.65790464350110377720, 5.46378491116411436990, 1.78482653991729133580,
+                                   2.96560571828504891230e-1, 2.65321895265761230930e-2, 1.24266094738807843860e-3,
+                                   2.71155556874348757815e-5, 2.01033439929228813265e-7, r);
+    const double den = RANDOM_POLY(1.0, 5.99832206555887937690e-1, 1.36929880922735805310e-1, 1.48753612908506148525e-2,
+                                   7.86869131145613259100e-4, 1.84631831751005468180e-5, 1.42151175831644588870e-7,
+                                   2.04426310338993978564e-15, r);
+    v = num / den;
+  }
+  return q < 0.0 ? -v : v;
+}
+
+// kind 0: scale * normal; kind 1: 1 + scale * (2 u - 1). Rounded once to float32.
+__global__ void random_fill_kernel(float* __restrict__ out, size_t n, unsigned long long key, int kind, double scale) {
+#pragma clang fp contract(off)
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const double u = (static_cast<double>(random_mix(key, i) >> 12) + 0.5) * 2.2204460492503130808e-16;   // 2^-52
+  const double v = kind == 0 ? scale * random_normal_of(u) : 1.0 + scale * (2.0 * u - 1.0);
+  out[i] = static_cast<float>(v);
+}
+
+extern "C" int tie_random_fill(float* out, long long n, unsigned long long key, int kind, double scale,
+                               hipStream_t stream) {
+  if (n <= 0 || (kind != 0 && kind != 1) || (n + 255) / 256 > 0x7fffffffLL) return TIE_BAD_ARGUMENT;
+  random_fill_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, stream>>>(out, static_cast<size_t>(n), key, kind,
+                                                                                   scale);
+  return tie_launch_status();
+}
+
 // --------------------------------------------------------------------- cast
 template <typename TX, typename TO>
 __global__ void cast_kernel(const TX* __restrict__ x, TO* __restrict__ out, size_t n) {
@@ -522,6 +621,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
     else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH4(float, bf16_t, bf16_t)
     else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH4(bf16_t, bf16_t, bf16_t)
     else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_BF16) LAUNCH4(float, float, bf16_t)
+    else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F16) LAUNCH4(float, float, f16_t)
     else return TIE_BAD_ARGUMENT;
 #undef LAUNCH4
 #undef LAUNCH4_L
@@ -537,6 +637,7 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
   else if (in_dtype == TIE_F32 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(float, bf16_t, bf16_t);
   else if (in_dtype == TIE_BF16 && q_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_BF16) LAUNCH(float, float, bf16_t);
+  else if (in_dtype == TIE_F32 && q_dtype == TIE_F32 && cache_dtype == TIE_F16) LAUNCH(float, float, f16_t);
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH
   return tie_launch_status();
@@ -801,6 +902,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
       if (rem - piece_sums[p] < 0.0) break;
       rem -= piece_sums[p];
     }
+    // Ended without a break on a piece that weighs nothing (rounding: the sums above were added in another
+    // order than the total): the walk in exact arithmetic ended in the last piece that weighs something.
+    while (p > 0 && !(piece_sums[p] > 0.0)) --p;
     owner_piece = p;
     remainder = rem;
   }
@@ -817,18 +921,22 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (lane >= d) upto += other;
   }
   const unsigned long long reached = __ballot(remainder - upto < 0.0);
-  // Rounding may leave a remainder: then the last logit of the piece, as the walk would end at the row's last.
+  // Rounding may leave a remainder (this scan adds in another order than the piece's sum): then the piece's last
+  // logit that weighs anything, where the walk in exact arithmetic ends; never a token of weight zero.
+  const unsigned long long alive = __ballot(mine > 0.0);
   int pick = min(owner_piece * SAMPLE_PIECE + SAMPLE_PIECE, V) - 1;
-  const int who = reached ? __ffsll(reached) - 1 : -1;
-  if (lane == who) {
+  const int who = reached ? __ffsll(reached) - 1 : (alive ? 63 - __clzll(alive) : 0);
+  if (lane == who && reached) {
     double rem = remainder - (upto - mine);
     pick = base + 3;
     if ((rem -= w0) < 0.0) pick = base;
     else if ((rem -= w1) < 0.0) pick = base + 1;
     else if ((rem -= w2) < 0.0) pick = base + 2;
     pick = min(pick, V - 1);
+  } else if (lane == who && alive) {
+    pick = w3 > 0.0 ? base + 3 : w2 > 0.0 ? base + 2 : w1 > 0.0 ? base + 1 : base;
   }
-  if (who < 0 ? lane == 0 : lane == who) out[r] = pick;
+  if (lane == who) out[r] = pick;
 }
 
 // With `rows` only the `num_rows` rows it lists are drawn, and out[] of the others is left as it is. With `row_max`

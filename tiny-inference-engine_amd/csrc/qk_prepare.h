@@ -47,6 +47,12 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, qk_f4_t v) {
   *reinterpret_cast<uint2*>(p) = o;
 }
 
+template <>
+__device__ __forceinline__ void store4<f16_t>(f16_t* p, qk_f4_t v) {
+  typedef __attribute__((ext_vector_type(4))) _Float16 qk_h4_t;
+  *reinterpret_cast<qk_h4_t*>(p) = __builtin_convertvector(v, qk_h4_t);
+}
+
 template <typename TX>
 __device__ __forceinline__ qk_f4_t load4_planes(const TX* p, size_t plane_stride, int planes) {
   if (planes == 2) return load4(p) + load4(p + plane_stride);

@@ -69,7 +69,10 @@ class _Unread:
 class Engine:
     def __init__(self, model: Model, cache: CacheManager, scheduler=None, serving: Optional[ServingConfig] = None,
                  stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None, use_graphs: Optional[bool] = None,
-                 launch_ahead: bool = False):
+                 launch_ahead: bool = False, runner=None, sampler=None):
+        """``runner`` / ``sampler``: stand-ins with the interface of ``ModelRunner`` (``step``,
+        ``max_blocks_per_seq``) and ``DeviceSampler`` (``launch_greedy``, ``launch``, ``collect``,
+        ``sample_rows``), for driving the engine's bookkeeping without a GPU; the default builds the real ones."""
         self.model = model
         self.cache = cache
         self.serving = serving or ServingConfig()
@@ -79,8 +82,8 @@ class Engine:
                                   f"{kernels.MAX_STEP_TOKENS} rows the kernels take in one step")
         self.scheduler = scheduler or BatchScheduler(cache, SchedulerConfig(serving=self.serving))
         self.stop_tokens = frozenset(int(t) for t in stop_tokens)
-        self.runner = ModelRunner(model, cache, max_seq_len, use_graphs=use_graphs)
-        self.sampler = DeviceSampler(model.device)
+        self.runner = runner if runner is not None else ModelRunner(model, cache, max_seq_len, use_graphs=use_graphs)
+        self.sampler = sampler if sampler is not None else DeviceSampler(model.device)
         self.sequences: Dict[int, Sequence] = {}
         self.on_token: Optional[Callable[[int, int], None]] = None     # (sequence id, token), as each token is known
         self._stats = EngineStats()
@@ -89,6 +92,7 @@ class Engine:
         self.launch_ahead = bool(launch_ahead)
         self._unread: Optional[_Unread] = None
         self.steps_launched_ahead = 0
+        self.ahead_replans = 0      # steps planned over unread tokens whose plan was not the steady one after all
 
     # -------------------------------------------------------------- requests
     def _token_limits(self) -> List[Tuple[int, str]]:
@@ -240,6 +244,7 @@ class Engine:
             if unread is not None and not (len(plan.seqs) == len(unread.sampling) and all(
                     share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, unread.sampling))):
                 # Planning changed the picture (a sequence was evicted to make room): read first after all.
+                self.ahead_replans += 1
                 self._read(unread)
                 unread = None
                 for share in [s for s in plan.seqs if s.seq.state == SeqState.FINISHED]:
@@ -333,7 +338,8 @@ class Engine:
             else:
                 seq.tokens[places[i]] = token
                 count = places[i] + 1 - seq.prompt_len       # a later token may stand behind it, still unread
-            seq.state = SeqState.DECODING
+            if seq.state != SeqState.WAITING:    # WAITING: evicted while this token was unread; it stays in the
+                seq.state = SeqState.DECODING    # scheduler's waiting queue and is computed again with the token
             if callback is not None:
                 try:
                     callback(seq.id, token)

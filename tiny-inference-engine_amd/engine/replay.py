@@ -23,23 +23,25 @@ from typing import Dict, List, Optional
 
 import torch
 
+from .. import kernels
 from ..cache.manager import CacheManager, RequestCache
 from ..errors import CapacityError, InvalidArgument
 from ..models.builder import Model, load_model
-from ..weights.binder import FLOAT32, normalize_mode
+from ..weights.binder import normalize_mode
 from .batch import StepEntry
 from .runner import ModelRunner
 
 
 class TraceReplayer:
-    def __init__(self, model: Model, max_tokens: int, block_size: int = 16, use_graphs=None):
+    def __init__(self, model: Model, max_tokens: int, block_size: int = 16, use_graphs=None, kv_dtype=None):
         """``max_tokens``: the most tokens live requests hold at any time, each request's
         count rounded up to a multiple of 64 (of the block size if that is larger); the page pool
-        is made for exactly this many, so pages are used again."""
+        is made for exactly this many, so pages are used again. ``kv_dtype``: the cache's precision if it is
+        to differ from the model's (float32 arithmetic over bfloat16 or float16 pages)."""
         if max_tokens <= 0:
             raise InvalidArgument(f"max_tokens must be positive, got {max_tokens}")
         self.model = model
-        cache_dtype = "float32" if model.mode == FLOAT32 else "bfloat16"
+        cache_dtype = kernels.cache_dtype_for(model.mode, kv_dtype)
         num_blocks = math.ceil(max_tokens / block_size)
         self.cache = CacheManager(model.cache_plan, block_size=block_size, num_blocks=num_blocks,
                                   dtype=cache_dtype, device=model.device, max_state_slots=8)
@@ -50,9 +52,11 @@ class TraceReplayer:
 
     @classmethod
     def from_folder(cls, folder, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
-                    use_graphs=None):
-        model = load_model(folder, normalize_mode(dtype), device)
-        return cls(model, max_tokens, block_size, use_graphs)
+                    use_graphs=None, kv_dtype=None):
+        mode = normalize_mode(dtype)
+        kernels.cache_dtype_for(mode, kv_dtype)        # a pair no kernel takes fails before the weights are read
+        model = load_model(folder, mode, device)
+        return cls(model, max_tokens, block_size, use_graphs, kv_dtype)
 
     def run_step(self, step: dict) -> Optional[torch.Tensor]:
         """Runs one step of a trace; returns float32 logits ``[wanted, vocab]`` (on the device) or None."""

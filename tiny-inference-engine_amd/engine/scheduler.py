@@ -246,7 +246,7 @@ class BatchScheduler:
         if not self.waiting:
             return
         self.waiting.sort(key=self._priority)
-        entered = 0
+        entered = set()
         for seq in self.waiting:
             if budget.spent() or len(self.running) >= self.config.serving.max_seqs:
                 break
@@ -258,9 +258,9 @@ class BatchScheduler:
             seq.state = SeqState.PREFILLING
             self.running.append(seq)
             self._grant(plan, budget, seq, n)
-            entered += 1
-        if entered:
-            self.waiting = [s for s in self.waiting if s.state == SeqState.WAITING]
+            entered.add(id(seq))
+        if entered:         # by identity, not by state: nothing but admission takes a sequence out of this queue
+            self.waiting = [s for s in self.waiting if id(s) not in entered]
 
     def _unblock_oldest(self, plan: StepPlan, budget: _Budget) -> None:
         for seq in self.running:

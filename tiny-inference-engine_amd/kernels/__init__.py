@@ -17,8 +17,32 @@ import torch
 from ..errors import InvalidArgument, KernelUnavailable
 from . import build
 
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
+_CACHE_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+# The cache of keys and values has a precision of its own (the reference's KVCacheConfig.dtype,
+# src/kv/paged_kv_cache.h:18-25: float32 arithmetic over a narrower cache is its default arrangement). Per
+# compute mode, the cache dtypes some kernel here reads and writes; the first is the mode's default.
+CACHE_DTYPES = {"float32": ("float32", "bfloat16", "float16"), "bfloat16": ("bfloat16",)}
+_CACHE_DTYPE_NAMES = {"float32": "float32", "fp32": "float32", "f32": "float32", "bfloat16": "bfloat16",
+                      "bf16": "bfloat16", "float16": "float16", "fp16": "float16", "f16": "float16"}
+
+
+def cache_dtype_for(mode: str, asked: Optional[str] = None) -> str:
+    """The cache dtype a compute mode runs over: its own by default, ``asked`` if the kernels take the pair."""
+    if mode not in CACHE_DTYPES:
+        raise InvalidArgument(f"unknown compute mode '{mode}'")
+    if asked is None:
+        return CACHE_DTYPES[mode][0]
+    name = _CACHE_DTYPE_NAMES.get(asked)
+    if name is None:
+        raise InvalidArgument(f"the cache dtype must be float32, bfloat16 or float16, got '{asked}'")
+    if name not in CACHE_DTYPES[mode]:
+        raise InvalidArgument(f"no kernel runs {mode} arithmetic over a {name} cache: with --dtype {mode} the cache "
+                              f"can be {' or '.join(CACHE_DTYPES[mode])} (the matrix-core attention kernels read "
+                              f"bfloat16 pages; float32 arithmetic reads any of the three)")
+    return name
 
 _c_int, _c_float, _c_void, _c_long = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_long
 
@@ -30,6 +54,7 @@ _SOURCES = {
     "skinny_gemm_bf16": ("tie_skinny_gemm_bf16", "skinny_gemm_bf16.hip"),
     "gemm_bf16": ("tie_gemm_bf16", "gemm_bf16.hip"),
     "sample_filtered": ("tie_sample_filtered", "sample_filtered.hip"),
+    "machine_peaks": ("tie_machine_peaks", "machine_peaks.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -42,6 +67,10 @@ MAX_HEAD_DIM = 512        # the largest head size any attention kernel takes (th
 MAX_STEP_TOKENS = 65535   # rows of one step: a grid dimension of the row-wise kernels
 
 _SIGNATURES = {
+    "machine_peaks": {
+        "tie_stream_read": [_c_void, ctypes.c_longlong, _c_int, _c_void, _c_void, _c_void],
+        "tie_mfma_rate": [_c_int, _c_int, _c_void, _c_void, _c_void],
+    },
     "sample_filtered": {
         "tie_sample_filtered": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                 _c_int, _c_void, _c_int, _c_int, _c_void],
@@ -51,6 +80,7 @@ _SIGNATURES = {
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
+        "tie_random_fill": [_c_void, ctypes.c_longlong, ctypes.c_ulonglong, _c_int, ctypes.c_double, _c_void],
         "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
@@ -236,6 +266,17 @@ def _code(t: torch.Tensor, name: str) -> int:
         raise InvalidArgument(f"{name} must be float32 or bfloat16, got {t.dtype}") from None
 
 
+def _cache_code(cache: torch.Tensor, beside: torch.Tensor, name: str) -> int:
+    """The type code of a cache plane; float16 pages go with float32 activations only."""
+    try:
+        code = _CACHE_CODES[cache.dtype]
+    except KeyError:
+        raise InvalidArgument(f"{name} must be float32, bfloat16 or float16, got {cache.dtype}") from None
+    if code == F16 and beside.dtype != torch.float32:
+        raise InvalidArgument(f"a float16 {name} goes with float32 queries, not {beside.dtype}")
+    return code
+
+
 def _i32(t: torch.Tensor, name: str, numel: Optional[int] = None) -> torch.Tensor:
     _gpu(t, name)
     if t.dtype != torch.int32:
@@ -333,6 +374,42 @@ def cast(x: torch.Tensor, out: torch.Tensor) -> None:
         raise InvalidArgument("cast: sizes differ")
     _call(_lib("elementwise").tie_cast, "cast", x.data_ptr(), _code(x, "cast input"), out.data_ptr(),
                                         _code(out, "cast output"), x.numel(), _stream())
+
+
+def random_fill(out: torch.Tensor, key: int, kind: str, scale: float) -> None:
+    """Fills float32 ``out`` with the random weights of the stream ``key``: element i depends on (key, i) alone
+    and equals, bit for bit, what ``weights.random_init`` draws on the host. ``kind``: "normal" (``scale`` the
+    standard deviation) or "one_plus_uniform" (1 + U(-scale, scale))."""
+    _f32(out, "random output")
+    if not out.is_contiguous():
+        raise InvalidArgument("random_fill needs a contiguous tensor")
+    kinds = {"normal": 0, "one_plus_uniform": 1}
+    if kind not in kinds:
+        raise InvalidArgument(f"random_fill draws 'normal' or 'one_plus_uniform', not '{kind}'")
+    if out.numel():
+        _call(_lib("elementwise").tie_random_fill, "random_fill", out.data_ptr(), out.numel(), int(key) & (2 ** 64 - 1),
+              kinds[kind], float(scale), _stream())
+
+
+def stream_read(data: torch.Tensor, sink: torch.Tensor, workgroups: int = 2048) -> int:
+    """Launches a kernel that reads ``data`` once, in consecutive runs a wave; returns the bytes it reads (whole
+    chunks of 8 KB a wave). For measuring what a streaming read of cold memory reaches: the caller times it."""
+    _gpu(data, "data")
+    _i32(sink, "sink")
+    read = ctypes.c_longlong(0)
+    _call(_lib("machine_peaks").tie_stream_read, "stream_read", data.data_ptr(), data.numel() * data.element_size(),
+          int(workgroups), sink.data_ptr(), ctypes.addressof(read), _stream())
+    return int(read.value)
+
+
+def mfma_rate(sink: torch.Tensor, workgroups: int = 1024, rounds: int = 4096) -> float:
+    """Launches a kernel of bfloat16 matrix instructions on registers alone; returns its floating-point operations.
+    For measuring the rate the matrix cores sustain: the caller times it."""
+    _f32(sink, "sink")
+    flops = ctypes.c_double(0.0)
+    _call(_lib("machine_peaks").tie_mfma_rate, "mfma_rate", int(workgroups), int(rounds), sink.data_ptr(),
+          ctypes.addressof(flops), _stream())
+    return float(flops.value)
 
 
 def gemm_generic(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -609,7 +686,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Opti
         _gpu(k_cache, "k cache")
         _gpu(v_cache, "v cache")
         _check_cache(k_cache, v_cache, KVH, block_size, Dh)
-        cache_code = _code(k_cache, "k cache")
+        cache_code = _cache_code(k_cache, q_out, "k cache")
     _call(_lib("elementwise").tie_qk_norm_rope_kv_write, "qk_norm_rope_kv_write",
         qkv.data_ptr(), _code(qkv, "qkv"), q_out.data_ptr(), _code(q_out, "q output"), _ptr(q_weight),
         _ptr(k_weight), float(eps), _ptr(inv_freq), _ptr(angles), positions.data_ptr(),
@@ -648,7 +725,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     if block_tables.dim() != 2 or block_tables.shape[0] < S:
         raise InvalidArgument(f"block tables {list(block_tables.shape)} do not cover {S} sequences")
     _call(_lib("attention_generic").tie_paged_attention_generic, "paged_attention_generic",
-        q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache, "k cache"),
+        q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _cache_code(k_cache, q, "k cache"),
         out.data_ptr(), _code(out, "attention output"), query_start.data_ptr(), context_lens.data_ptr(),
         block_tables.data_ptr(), seq_of_row.data_ptr(), T, H, KVH, Dh, bs, block_tables.shape[1], float(scale),
         int(window or 0), _stream())

@@ -8,6 +8,7 @@ a step: embedding, the run order, the head on the wanted rows.
 
 from __future__ import annotations
 
+import dataclasses
 import sys
 from typing import Callable, Dict, List, Optional
 
@@ -25,11 +26,16 @@ from ..weights.safetensors_io import StoredTensor
 from .spec import ModelSpec
 
 
-def _walk_parts(obj, tensors, classes, seen) -> None:
-    """The device tensors ``(address, bytes, shape, dtype)`` and the part classes of an object tree, in a fixed order."""
+def _walk_parts(obj, tensors, classes, seen, scalars=None, path="") -> None:
+    """The device tensors ``(address, bytes, shape, dtype)``, the part classes and (``scalars``) the plain values
+    ``(path, value)`` - numbers, strings, None - of an object tree, in a fixed order."""
     if isinstance(obj, torch.Tensor):
         if obj.is_cuda:
             tensors.append((obj.data_ptr(), obj.numel() * obj.element_size(), tuple(obj.shape), obj.dtype))
+        elif scalars is not None:        # a host tensor (a table of frequencies) is a value like any other
+            small = obj.numel() <= 65536
+            scalars.append((path, (tuple(obj.shape), str(obj.dtype),
+                                   tuple(obj.flatten().tolist()) if small else id(obj))))
     elif isinstance(obj, kernels.PackedWeight):
         blocks = obj.blocks
         tensors.append((blocks.data_ptr(), blocks.numel() * blocks.element_size(), tuple(obj.shape), "packed"))
@@ -39,19 +45,42 @@ def _walk_parts(obj, tensors, classes, seen) -> None:
         seen.add(id(obj))
         classes.append(type(obj))
         for name in sorted(vars(obj)):
-            _walk_parts(getattr(obj, name), tensors, classes, seen)
+            _walk_parts(getattr(obj, name), tensors, classes, seen, scalars, f"{path}.{name}")
     elif isinstance(obj, (list, tuple)):
-        for value in obj:
-            _walk_parts(value, tensors, classes, seen)
+        for i, value in enumerate(obj):
+            _walk_parts(value, tensors, classes, seen, scalars, f"{path}[{i}]")
     elif isinstance(obj, dict):
         for name in sorted(obj, key=str):
-            _walk_parts(obj[name], tensors, classes, seen)
+            _walk_parts(obj[name], tensors, classes, seen, scalars, f"{path}[{name!r}]")
+    elif obj is None or isinstance(obj, (bool, int, float, str)):
+        if scalars is not None:
+            scalars.append((path, obj))
+    elif isinstance(obj, (torch.dtype, torch.device)):
+        if scalars is not None:
+            scalars.append((path, str(obj)))
+    elif dataclasses.is_dataclass(obj) and not isinstance(obj, type):
+        if scalars is not None:
+            scalars.append((path, type(obj).__name__))
+        for field in dataclasses.fields(obj):
+            _walk_parts(getattr(obj, field.name), tensors, classes, seen, scalars, f"{path}.{field.name}")
     elif type(obj).__module__.startswith(__name__.split(".")[0] + ".") and hasattr(obj, "__dict__"):
         if id(obj) in seen:          # a helper object of this package that a part holds (a Linear with its weight)
             return
         seen.add(id(obj))
         for name in sorted(vars(obj)):
-            _walk_parts(getattr(obj, name), tensors, classes, seen)
+            _walk_parts(getattr(obj, name), tensors, classes, seen, scalars, f"{path}.{name}")
+    elif scalars is not None:
+        scalars.append((path, ("object", type(obj).__qualname__, id(obj))))     # unknown: alike only if the very same
+
+
+def _constants(scalars, tensor_names) -> tuple:
+    """What of a layer's plain values must agree for two layers to launch the same kernels with the same numbers:
+    everything but the strings that name its tensors (whole names, their parts and prefixes), which differ from
+    layer to layer by design."""
+    def names_a_tensor(value) -> bool:
+        return isinstance(value, str) and value != "" and any(value in name for name in tensor_names)
+
+    return tuple((path, value) for path, value in scalars if not names_a_tensor(value))
 
 
 class _Launch:
@@ -149,19 +178,24 @@ class Model:
     def _find_layers_alike(self) -> None:
         """Finds runs of consecutive entries of the run order whose layers are of one shape.
 
-        Alike: the same part classes, every one of them ``replayable``, device tensors of the same shapes and
-        dtypes in the same places, the same kind of cache binding; each entry a layer of its own.
+        Alike: the same part classes, every one of them ``replayable``, the same parameters and other plain values
+        (an eps, a scale, a window: all but the names of tensors), device tensors of the same shapes and dtypes in
+        the same places, the same kind of cache binding; each entry a layer of its own, and each with a cache plane
+        of its own or all reading one.
         """
         self._alike, self._layer_tensors = {}, {}
         signatures = []
         for index, call in enumerate(self.spec.order):
-            tensors, classes = [], []
-            _walk_parts(self.layers[call.layer].parts(), tensors, classes, set())
+            tensors, classes, scalars = [], [], []
+            layer_parts = self.layers[call.layer].parts()
+            _walk_parts(layer_parts, tensors, classes, set(), scalars)
             self._layer_tensors[index] = [(address, size) for address, size, _, _ in tensors]
             entry = self.cache_plan.calls[index]
             binding = None if entry is None else (entry.group, entry.writes)
             ok = all(getattr(c, "replayable", False) for c in classes)
-            signatures.append((tuple(classes), tuple(t[2:] for t in tensors), binding) if ok else None)
+            names = {spec.name for part in layer_parts for spec in part.all_tensors()}
+            signatures.append((tuple(classes), tuple(t[2:] for t in tensors), binding, _constants(scalars, names))
+                              if ok else None)
         start = 0
         while start < len(signatures):
             end = start + 1
@@ -178,6 +212,11 @@ class Model:
                 if len(addresses) not in (1, end - start):
                     end = start + 1
                     break
+            # The same for the cache: entries that read an earlier entry's plane pass for "the same argument" too.
+            planes = {None if self.cache_plan.calls[i] is None else self.cache_plan.calls[i].plane
+                      for i in range(start, end)}
+            if len(planes) not in (1, end - start):
+                end = start + 1
             if end - start >= self.MIN_ALIKE:
                 self._alike[start] = end
             start = end

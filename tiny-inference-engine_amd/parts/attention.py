@@ -28,6 +28,7 @@ from .linear import Linear
 
 @register_part("mixer", "paged_attention")
 class PagedAttention(Mixer):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
 
     def __init__(self, params):

@@ -83,11 +83,12 @@ class Part:
     the step's arrays (``ctx.batch.tokens``, ``positions``, ``state_slots``, a group's block tables:
     they live at fixed addresses) and the launches themselves depend only on the step's shape. A
     part that reads host-side values of the step (``ctx.batch.host_*``), loops over them, or calls
-    anything that waits for the GPU (``nonzero``, ``.item()``, ``.cpu()``) sets it to False; a model
-    with one such part runs every step eagerly.
+    anything that waits for the GPU (``nonzero``, ``.item()``, ``.cpu()``) must leave it False; a model
+    with one such part runs every step eagerly. False is the default, so a part written elsewhere that
+    says nothing is never baked into a recording; the parts of this package say True.
     """
 
-    capturable = True
+    capturable = False
     # True: in a step, what the part launches is the same for every layer of the same shape except for the
     # addresses of the layer's own tensors and cache (no host-side work per layer beyond kernel launches, no
     # torch operations, nothing that depends on which layer it is). The model then runs such layers from the

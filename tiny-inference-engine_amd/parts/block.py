@@ -16,6 +16,7 @@ from .base import Block, StepContext, register_part
 
 @register_part("block", "pre_norm")
 class PreNormBlock(Block):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
     NORMS = ("pre_mixer", "pre_feed_forward")
 

@@ -17,6 +17,8 @@ from .base import Embedding, StepContext, TensorSpec, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Embedding):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
+
     def __init__(self, params):
         super().__init__(params)
         self.vocab = int(params["vocab"])

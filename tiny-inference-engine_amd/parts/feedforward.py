@@ -21,6 +21,7 @@ from .linear import Linear
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
 
     def __init__(self, params):

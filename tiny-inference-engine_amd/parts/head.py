@@ -20,6 +20,8 @@ from .base import Head, Part, StepContext, TensorSpec, build_part, register_part
 
 @register_part("head", "lm_head")
 class LmHead(Head):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
+
     def __init__(self, params):
         super().__init__(params)
         self.vocab = int(params["vocab"])

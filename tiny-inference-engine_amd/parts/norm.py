@@ -18,6 +18,7 @@ from .base import Norm, StepContext, TensorSpec, register_part
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
     adds_owed = True
 

@@ -19,6 +19,7 @@ from .base import Position, register_part
 
 @register_part("position", "rope_neox")
 class RopeNeox(Position):
+    capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
 
     def __init__(self, params):
@@ -58,6 +59,7 @@ class RopeNeox(Position):
 class NoPosition(Position):
     """No position encoding: queries and keys are left as they are."""
 
+    capturable = True
     replayable = True
 
     def rotary_table(self):
