@@ -890,21 +890,34 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     double total = 0.0;
     for (int w = 0; w < SAMPLE_WAVES; ++w) total += wave_sums[w];
     double rem = (take_other && take_other[r] ? other_uniform[r] : uniform[r]) * total;
-    int w = 0;
-    for (; w < SAMPLE_WAVES - 1; ++w) {
+    // The walk over the waves' sums, then over the pieces of the wave it stops in. Their sums were added in
+    // other orders than the total, so by a rounding the walk may run past the end of either: then it ended, in
+    // exact arithmetic, at the last token that weighs anything (an infinite remainder says so to the lanes).
+    bool ran_past = false;
+    int w = 0, p;
+    for (; w < SAMPLE_WAVES; ++w) {
       if (rem - wave_sums[w] < 0.0) break;
       rem -= wave_sums[w];
     }
-    int p = w * per_wave;
-    const int last = min(p + per_wave, pieces) - 1;
-    if (p > last) p = pieces - 1;         // rounding left a remainder beyond the last piece with logits
-    for (; p < last; ++p) {
-      if (rem - piece_sums[p] < 0.0) break;
-      rem -= piece_sums[p];
+    if (w == SAMPLE_WAVES) {
+      ran_past = true;
+      p = pieces - 1;
+    } else {
+      p = w * per_wave;                    // the wave weighs more than the remainder: it has pieces
+      const int last = min(p + per_wave, pieces) - 1;
+      for (; p <= last; ++p) {
+        if (rem - piece_sums[p] < 0.0) break;
+        rem -= piece_sums[p];
+      }
+      if (p > last) {
+        ran_past = true;
+        p = last;
+      }
     }
-    // Ended without a break on a piece that weighs nothing (rounding: the sums above were added in another
-    // order than the total): the walk in exact arithmetic ended in the last piece that weighs something.
-    while (p > 0 && !(piece_sums[p] > 0.0)) --p;
+    if (ran_past) {
+      while (p > 0 && !(piece_sums[p] > 0.0)) --p;
+      rem = INFINITY;
+    }
     owner_piece = p;
     remainder = rem;
   }
@@ -920,21 +933,28 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     const double other = __shfl_up(upto, d);
     if (lane >= d) upto += other;
   }
-  const unsigned long long reached = __ballot(remainder - upto < 0.0);
-  // Rounding may leave a remainder (this scan adds in another order than the piece's sum): then the piece's last
-  // logit that weighs anything, where the walk in exact arithmetic ends; never a token of weight zero.
-  const unsigned long long alive = __ballot(mine > 0.0);
-  int pick = min(owner_piece * SAMPLE_PIECE + SAMPLE_PIECE, V) - 1;
+  // Only tokens that weigh something can be chosen. The lanes' running sums are added in different orders, so
+  // that of a lane behind the last such token may exceed the one before it by a rounding, and rounding may also
+  // leave a remainder beyond every lane's sum (this scan adds in another order than the piece's sum): then the
+  // piece's last token that weighs anything, where the walk in exact arithmetic ends.
+  const bool weighs = mine > 0.0;
+  const unsigned long long reached = __ballot(weighs && remainder - upto < 0.0);
+  const unsigned long long alive = __ballot(weighs);
   const int who = reached ? __ffsll(reached) - 1 : (alive ? 63 - __clzll(alive) : 0);
-  if (lane == who && reached) {
+  int pick = min(owner_piece * SAMPLE_PIECE + SAMPLE_PIECE, V) - 1;
+  if (lane == who && alive) {
+    const double w[4] = {w0, w1, w2, w3};
     double rem = remainder - (upto - mine);
-    pick = base + 3;
-    if ((rem -= w0) < 0.0) pick = base;
-    else if ((rem -= w1) < 0.0) pick = base + 1;
-    else if ((rem -= w2) < 0.0) pick = base + 2;
-    pick = min(pick, V - 1);
-  } else if (lane == who && alive) {
-    pick = w3 > 0.0 ? base + 3 : w2 > 0.0 ? base + 2 : w1 > 0.0 ? base + 1 : base;
+    int at = 0;
+    bool found = false;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (found || !(w[i] > 0.0)) continue;
+      at = i;                              // the last that weighs something, unless the walk ends earlier
+      rem -= w[i];
+      found = reached != 0 && rem < 0.0;
+    }
+    pick = base + at;
   }
   if (lane == who) out[r] = pick;
 }
