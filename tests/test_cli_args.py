@@ -23,7 +23,8 @@ def test_every_option_is_read():
                              "--seed", "9", "--max-tokens", "12", "--kv-mem", "512M", "--stop-ids", "2,3",
                              "--dtype", "float32", "--block-size", "4", "--kv-blocks", "40", "--max-seqs", "8",
                              "--max-tokens-per-step", "64", "--prefill-chunk", "13", "--policy", "fcfs",
-                             "--aging", "2", "--device", "hip", "--threads", "4"])
+                             "--aging", "2", "--device", "hip", "--threads", "4", "--kv-dtype", "float16"])
+    assert o.kv_dtype == "float16" and parse_generate_args(["-m", "m", "-p", "7"]).kv_dtype is None
     assert o.sampling.temperature == 0.0 and o.sampling.top_k == 5 and o.sampling.top_p == 0.5
     assert o.sampling.seed == 9 and o.sampling.max_tokens == 12 and o.kv_bytes == 512 << 20
     assert o.stop_ids == [2, 3] and o.dtype == "float32" and o.block_size == 4 and o.kv_blocks == 40
@@ -38,6 +39,7 @@ def test_every_option_is_read():
     (["-m", "x", "-p", "1", "--max-tokens", "0"], "max_tokens"), (["-m", "x", "-p", "a,b"], "integer"),
     (["-m", "x", "-p", "1", "--kv-mem", "4T"], "--kv-mem"), (["-m", "x", "-p", "1", "--device", "cpu"], "no CPU path"),
     (["-m", "x", "-p", "1", "--chat"], "tokenizer"), (["-m", "x", "-p", "1", "--policy", "lifo"], "lifo"),
+    (["-m", "x", "-p", "1", "--kv-dtype", "int8"], "--kv-dtype must be"),
 ])
 def test_bad_arguments_are_refused(argv, match):
     with pytest.raises(InvalidArgument, match=match):
@@ -80,6 +82,9 @@ def test_bench_defaults_and_options():
     assert o.prompts == "w.jsonl" and o.prompt_len == (3, 9) and o.output_len == (7, 7) and o.rate == 2.5
     assert o.max_tokens == 5 and o.json and o.sampling.temperature == 0.5 and o.sampling.seed == 4
     assert o.kv_bytes == 2 << 30 and o.prefill_chunk == 512 and o.max_seqs == 16 and o.policy == "fcfs"
+    assert o.launch_ahead and o.kv_dtype is None
+    o = parse_bench_args(["-m", "d", "--synthetic", "2", "--no-launch-ahead", "--kv-dtype", "bf16"])
+    assert not o.launch_ahead and o.kv_dtype == "bf16"
 
 
 @pytest.mark.parametrize("argv,match", [

@@ -15,6 +15,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
+import tolerances
 import trace_helpers as th
 from conftest import TINY_B, load_plain_weights
 
@@ -26,6 +27,8 @@ def close(got, want, rel, what=""):
     got, want = got.detach().cpu().to(F64), want.detach().cpu().to(F64)
     err = float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
     assert err <= rel, f"{what}: relative error {err:.3e} > {rel:.0e}"
+    if rel >= 1e-3:
+        print(f"[observed] {what}: {err:.3e} (allowed {rel:.0e})")
 
 
 class FakeBatch:
@@ -210,7 +213,7 @@ def plain_with_order(weights, cfg, tokens, order, window=None):
     return plain.linear(x, weights["lm_head.weight"])
 
 
-@pytest.mark.parametrize("dtype,tolerance", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype,tolerance", [("float32", tolerances.FLOAT32), ("bfloat16", tolerances.BFLOAT16["run orders"])])
 @pytest.mark.parametrize("order,window", [
     (((0, None), (1, None), (0, None)), None),            # layer 0 runs twice, each call with a cache of its own
     (((0, None), (1, None), (0, 0), (1, 1)), None),       # the later calls read the earlier calls' caches
@@ -542,7 +545,7 @@ def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, k
         got = th.collect(replayer, changing_live_sets(requests, head, subsets))
         for rid, ref in want.items():
             mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
-            close(mine, ref, 3e-2, f"toy model in bfloat16 ({kind}), request {rid}")
+            close(mine, ref, tolerances.BFLOAT16["toy architecture"], f"toy model in bfloat16 ({kind}), request {rid}")
         assert replayer.cache.num_free_state_slots == replayer.cache.max_state_slots
         assert (replayer.runner.graph_replays > 20) == (kind == "recorded")
         # and through the engine, whose scheduler hands the slots out; recording can also be switched off there
@@ -555,7 +558,8 @@ def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, k
             tokens = list(prompt)
             for t in out:
                 row = toy_plain(weights, cfg, tokens)[-1]
-                assert float(row.max() - row[t]) <= 3e-2 * float(row.abs().max()), "a token the plain logits do not favour"
+                assert float(row.max() - row[t]) <= tolerances.BFLOAT16["toy architecture"] * float(row.abs().max()), \
+                    "a token the plain logits do not favour"
                 tokens.append(t)
     finally:
         unregister_architecture("ToyStateLM")

@@ -16,13 +16,15 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
+import tolerances
 import trace_helpers as th
 from conftest import BLOCK_SIZE, ROOT, TINY, load_plain_weights
 
 pytestmark = pytest.mark.gpu
 
-# max |engine - plain| / max |plain| over a request's logits
-TOLERANCE = {"float32": 1e-4, "bfloat16": 3e-2}
+# max |engine - plain| / max |plain| over a request's logits: float32, and bfloat16 by fixture (the label of every
+# check begins with the fixture's letter)
+TOLERANCE = {"float32": tolerances.FLOAT32, "A": tolerances.BFLOAT16["tiny A"], "B": tolerances.BFLOAT16["tiny B"]}
 LENGTHS = {"A": [5, 11, 17, 40, 64, 33], "B": [1, 23, 40, 64, 90, 37]}
 
 
@@ -33,7 +35,8 @@ def reference_logits(folder, cfg, requests):
 
 def check(got, want, dtype, label, tolerance=None):
     worst = 0.0
-    tolerance = TOLERANCE[dtype] if tolerance is None else tolerance
+    if tolerance is None:
+        tolerance = TOLERANCE["float32"] if dtype == "float32" else TOLERANCE[label[0]]
     for rid, ref in want.items():
         rows = got[rid]
         assert sorted(rows) == list(range(ref.shape[0])), f"{label}: request {rid} misses positions"
@@ -44,6 +47,7 @@ def check(got, want, dtype, label, tolerance=None):
         assert bad < 0, (f"{label}: request {rid} first differs at position {bad} "
                          f"(relative error {float(err[bad]):.3e}, allowed {tolerance:.0e})")
         worst = max(worst, float(err.max()))
+    print(f"[observed] {label}: {worst:.3e}")
     return worst
 
 
@@ -116,7 +120,7 @@ def test_float32_arithmetic_over_a_narrower_cache(folders, name, kv_dtype):
         results[label] = th.collect(rep, trace)
         assert rep.cache.num_free() == rep.cache.num_blocks
         worst = max(worst, check(results[label], want, "float32", f"{name}/float32 over {kv_dtype}/{label}",
-                                 tolerance=NARROW_CACHE_TOLERANCE[kv_dtype]))
+                                 tolerance=tolerances.NARROW_CACHE[kv_dtype]))
     print(f"[observed] {name} float32 over {kv_dtype}: worst relative error {worst:.3e}")
     assert worst > 1e-6, "the cache rounded nothing: is it float32 after all?"
     for label in ("prefill+decode", "portions", "mixed"):
@@ -227,10 +231,45 @@ def test_layers_of_one_shape_run_from_one_layers_launch_list(tmp_path, dtype, us
         got[replay] = th.collect(rep, steps)
         assert (rep.model.layers_replayed > 0) == replay
         assert rep.cache.num_free() == rep.cache.num_blocks
-    check(got[True], want, dtype, f"seven layers alike/{dtype}")
+    check(got[True], want, dtype, f"B with seven layers alike/{dtype}")
     for rid in requests:
         for position, row in got[True][rid].items():
             assert torch.equal(row, got[False][rid][position]), f"request {rid}, position {position}"
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_a_corrupted_page_is_caught(folders, name):
+    """The bound the bfloat16 checks use must not be so wide that a wrong page of the cache passes under it. A
+    request is prefilled, ONE page of ONE layer's keys (then, in another run, values) is overwritten with the
+    page after it, and the last token is decoded: its logits must miss the plain implementation's by more than
+    the bound, in every layer; the clean run of the same steps stays well within it. (Swapping two entries of the
+    block table is no such fault: keys and values move together, and attention does not care in which order it
+    meets them.)"""
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg = folders["bfloat16"][name]
+    tokens = th.make_requests(cfg["vocab_size"], LENGTHS[name], seed=5)["r4"]
+    want = plain.forward(load_plain_weights(folder), cfg, tokens, rows=[len(tokens) - 1]).float()[0]
+    bound = TOLERANCE[name]
+
+    def last_row_error(layer=None, plane=0):
+        rep = TraceReplayer.from_folder(folder, "bfloat16", th.round64(len(tokens)), block_size=BLOCK_SIZE[name])
+        rep.run_step({"step": 0, "entries": [{"id": "a", "tokens": tokens[:-1], "want": []}], "end": []})
+        if layer is not None:
+            table = rep.requests["a"].tables[0]
+            pages = rep.cache.kv[0]                    # [layer, keys | values, page, kv head, ...]
+            pages[layer, plane, table[1]] = pages[layer, plane, table[2]].clone()
+        logits = rep.run_step({"step": 1, "entries": [{"id": "a", "tokens": tokens[-1:], "want": [0]}], "end": ["a"]})
+        return float((logits[0].float().cpu() - want).abs().max() / want.abs().max())
+
+    assert last_row_error() < bound / 2
+    seen = {}
+    for layer in range(cfg["num_hidden_layers"]):
+        for plane, what in ((0, "keys"), (1, "values")):
+            seen[(layer, what)] = last_row_error(layer, plane)
+    print(f"[observed] {name}: a corrupted page moves the last row by {seen} (bound {bound})")
+    first_layer = max(seen[(0, "keys")], seen[(0, "values")])
+    assert seen[(0, "keys")] > 1.25 * bound and first_layer > 2 * bound, f"a wrong page passes under the bound: {seen}"
 
 
 def test_pages_are_used_again(folders):
