@@ -53,9 +53,9 @@ class FakeRunner:
         out = []
         for i, e in enumerate(entries):
             tokens = list(e.tokens)
-            if device_tokens is not None:
-                assert len(tokens) == 1
-                tokens = [device_tokens[i]]
+            if e.token_from >= 0:                   # the token an earlier step's sampling left "on the device"
+                assert len(tokens) == 1 and device_tokens is not None
+                tokens = [device_tokens[e.token_from]]
             assert all(0 <= t < VOCAB for t in tokens), "a token the host never read went into a step as it stood"
             past = self.history.setdefault(id(e.cache), [])
             assert len(past) >= e.start, "a step began beyond what the cache holds"
@@ -119,7 +119,7 @@ def run_all(engine, requests, arrivals=None, limit=20000):
 @pytest.mark.parametrize("policy", [FCFS, SRPT_AGING])
 @pytest.mark.parametrize("launch_ahead", [False, True])
 def test_random_workloads_over_small_pools_lose_nobody(policy, launch_ahead):
-    evictions = ahead = 0
+    evictions = ahead = mixed_ahead = steps = 0
     for seed in range(300):
         rng = random.Random(seed)
         n = rng.randint(2, 6)
@@ -136,8 +136,12 @@ def test_random_workloads_over_small_pools_lose_nobody(policy, launch_ahead):
         assert engine.cache.all_free()
         evictions += engine.stats().preemptions
         ahead += engine.steps_launched_ahead
+        mixed_ahead += engine.ahead_replans
+        steps += engine.stats().steps
     assert evictions > 100
-    assert (ahead > 100) == launch_ahead
+    # Queued ahead are not only the steady repetitions of a decode step but most steps: prompts beside decoders,
+    # admissions, steps after an eviction.
+    assert (ahead > 0.6 * steps and mixed_ahead > 0.2 * steps) if launch_ahead else ahead == mixed_ahead == 0
 
 
 def test_an_eviction_while_tokens_are_unread_keeps_the_evicted_request():

@@ -185,6 +185,25 @@ extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_
   return tie_launch_status();
 }
 
+// ------------------------------------------------------------ tokens the host has not seen
+// tokens[i] = previous[sources[i]] where sources[i] >= 0: rows whose token an earlier step's sampling kernel left
+// on the device (the host queues this step before it has read that one); the other rows keep the host's token.
+__global__ void take_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ sources,
+                                   const int* __restrict__ previous, int T, int num_previous) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T) return;
+  const int from = sources[i];
+  if (from >= 0 && from < num_previous) tokens[i] = previous[from];
+}
+
+extern "C" int tie_take_tokens(int* tokens, const int* sources, const int* previous, int T, int num_previous,
+                               hipStream_t stream) {
+  if (T <= 0 || num_previous <= 0 || tokens == nullptr || sources == nullptr || previous == nullptr)
+    return TIE_BAD_ARGUMENT;
+  take_tokens_kernel<<<(T + 255) / 256, 256, 0, stream>>>(tokens, sources, previous, T, num_previous);
+  return tie_launch_status();
+}
+
 // ------------------------------------------------------------ random weights
 // Element i of a tensor is a function of (key, i) alone: the 64-bit mix of key + (i + 1) * 0x9E3779B97F4A7C15
 // (the SplitMix64 step) gives 52 bits of a uniform number u in (0, 1), and a normal value is the inverse normal

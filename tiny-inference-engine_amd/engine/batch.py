@@ -7,7 +7,7 @@ tokens, freely mixed. ``build`` lays out the arrays the kernels read, as the
 reference's engine does (``src/engine/engine.cpp:104-135``):
 
     tokens[T] positions[T] seq_of_row[T] query_start[S+1] context_lens[S]
-    state_slots[S] logit_rows[R]   and per paged cache group:
+    state_slots[S] logit_rows[R] token_sources[T]   and per paged cache group:
     slot_mapping[T] block_tables[S, max_blocks_per_seq]
 
 ``context_lens`` counts the cached tokens AFTER this step; the query at row t of
@@ -33,6 +33,8 @@ class StepEntry:
     start: int                       # tokens of the request already in the cache
     tokens: Sequence[int]            # its next tokens, run in this step
     want: Sequence[int] = ()         # places among ``tokens`` whose logits are wanted
+    token_from: int = -1             # >= 0: the entry's one token is not known to the host; it is this entry of
+                                     # the tokens an earlier step's sampling left on the device (ModelRunner.step)
 
 
 class GroupStep:
@@ -51,7 +53,8 @@ class StepBatch:
         self.num_tokens = 0
         self.num_seqs = 0
         self.num_logit_rows = 0
-        self.tokens = self.positions = self.seq_of_row = None
+        self.tokens = self.positions = self.seq_of_row = self.token_sources = None
+        self.takes_device_tokens = False      # some row's token comes from an earlier step's sampling output
         self.query_start = self.context_lens = self.state_slots = self.logit_rows = None
         self.groups: Dict[int, GroupStep] = {}
         # host copies for planning
@@ -129,6 +132,8 @@ class BatchBuilder:
             seen.add(key)
             if e.start < 0:
                 raise InvalidArgument(f"an entry starts at position {e.start}")
+            if e.token_from >= 0 and n != 1:
+                raise InvalidArgument(f"an entry takes its token from the device and brings {n} tokens, not one")
             for w in e.want:
                 if not 0 <= w < n:
                     raise InvalidArgument(f"wanted place {w} lies outside the entry's {n} tokens")
@@ -160,6 +165,7 @@ class BatchBuilder:
             raise self._bad_token(ids)
         order = np.arange(S + 1, dtype=np.int32)
         view("tokens")[:] = ids
+        view("token_sources")[:] = np.fromiter((e.token_from for e in entries), dtype=np.int32, count=S)
         view("positions")[:] = starts
         view("seq_of_row")[:] = order[:S]
         view("query_start")[:] = order
@@ -186,6 +192,7 @@ class BatchBuilder:
         bs, MB = self.cache.block_size, self.max_blocks_per_seq
         groups = self.cache.plan.paged_groups
         tokens, positions, seq_of_row = view("tokens"), view("positions"), view("seq_of_row")
+        token_sources = view("token_sources")
         query_start, context_lens = view("query_start"), view("context_lens")
         state_slots, logit_rows = view("state_slots"), view("logit_rows")
         slot_views = [view(("slots", g)) for g in groups]
@@ -200,6 +207,7 @@ class BatchBuilder:
                 raise self._bad_token(ids)
             where = np.arange(start, start + n, dtype=np.int32)
             tokens[row:row + n] = ids
+            token_sources[row:row + n] = e.token_from
             positions[row:row + n] = where
             seq_of_row[row:row + n] = s
             context_lens[s] = start + n
@@ -231,7 +239,7 @@ class BatchBuilder:
         layout = {}
         offset = 0
         for name, count in (("tokens", T), ("positions", T), ("seq_of_row", T), ("query_start", S + 1),
-                            ("context_lens", S), ("state_slots", S), ("logit_rows", R)):
+                            ("context_lens", S), ("state_slots", S), ("logit_rows", R), ("token_sources", T)):
             layout[name] = (offset, count)
             offset += _align(count)
         for g in groups:
@@ -266,6 +274,8 @@ class BatchBuilder:
         batch.tokens, batch.positions, batch.seq_of_row = dev("tokens"), dev("positions"), dev("seq_of_row")
         batch.query_start, batch.context_lens = dev("query_start"), dev("context_lens")
         batch.state_slots, batch.logit_rows = dev("state_slots"), dev("logit_rows")
+        batch.token_sources = dev("token_sources")
+        batch.takes_device_tokens = any(e.token_from >= 0 for e in entries)
         for g in groups:
             batch.groups[g] = GroupStep(dev(("slots", g)), dev(("tables", g), (S, MB)))
         batch.max_context = max(batch.host_context_lens)

@@ -13,17 +13,18 @@ reference engine's (``src/engine/engine.cpp:26-235``):
   ``FinishReason.ERROR`` and frees what they hold, since their cache already counts the step;
 * a sequence ends on a stop token (which stays in its output) or after ``max_tokens`` tokens.
 
-Reading ahead (``launch_ahead``, not in the reference). A decode step's host work - planning, the batch
-arrays, the launch - lies between two steps while the GPU idles, because the next step's tokens are the
-ones just sampled. With ``launch_ahead`` a step only queues its sampling kernels and leaves the
-tokens unread; if the next call to ``step()`` finds the steady state (nobody waiting, the very same
-sequences decoding, none at its last token), it queues the next step first - whose tokens the GPU
-takes from the sampling kernels' own output - and reads the earlier step's tokens while that one runs
-(rows that draw carry both uniform numbers their stream may be at, see ``DeviceSampler``). A
-sequence that turns out to have met a stop token has then run one token too many, which is dropped.
-In every other situation the unread tokens are read before anything is planned, and the engine behaves
-as without the option. Tokens (and callbacks) appear one ``step()`` later; ``has_work()`` stays true
-until they have.
+Reading ahead (``launch_ahead``, not in the reference). A step's host work - planning, the batch arrays,
+the launches - lies between two steps while the GPU idles, because the next step's tokens are the ones just
+sampled. With ``launch_ahead`` a step only queues its sampling kernels and leaves the tokens unread; the next
+call to ``step()`` plans and queues the next step first - the rows that continue a sequence whose token is
+unread take it on the GPU from the sampling kernels' own output - and reads the earlier step's tokens while
+that one runs. Nothing in a plan depends on the value of an unread token, only on its existence: which
+sequences decode, which prompts go on, who is admitted. Two things need the token itself and are read before
+planning: a sequence whose unread token is its last (it ends, and planning it again would be wrong), and rows
+that draw from a random stream unless the step is the steady repetition of the one before (they carry both
+uniform numbers their stream may be at, see ``DeviceSampler``, which asks for the same rows in the same order).
+A sequence that turns out to have met a stop token has then run one token too many, which is dropped. Tokens
+(and callbacks) appear one ``step()`` later; ``has_work()`` stays true until they have.
 """
 
 from __future__ import annotations
@@ -170,8 +171,8 @@ class Engine:
         self._inside_step = True
         try:
             unread = self._unread
-            if unread is not None and not self._steady(unread):
-                self._read(unread)                 # anything but the steady state: know the tokens before planning
+            if unread is not None and not self._may_plan_over(unread):
+                self._read(unread)                 # a token is needed for the plan itself: know it first
                 unread = None
             plan = self.scheduler.schedule()
             if plan:
@@ -181,8 +182,21 @@ class Engine:
         finally:
             self._inside_step = False
 
+    def _may_plan_over(self, unread: _Unread) -> bool:
+        """Whether the next step can be planned while the tokens of ``unread`` are still on the GPU."""
+        if not all(seq.params.greedy for seq in unread.sampling):
+            return self._steady(unread)            # rows that draw: only the same rows again, in the same order
+        for seq in unread.sampling:
+            if seq.state == SeqState.FINISHED:     # cancelled meanwhile: its token will be dropped
+                continue
+            if seq.state != SeqState.DECODING or seq.tokens[-1] != UNREAD:
+                return False
+            if len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:    # the unread token is its last
+                return False
+        return True
+
     def _steady(self, unread: _Unread) -> bool:
-        """Whether the next step can be planned without the unread tokens: the same sequences decode again."""
+        """Whether the next step is the one before once more: the very same sequences decode, nobody waits."""
         running = self.scheduler.running
         if self.scheduler.waiting or len(running) != len(unread.sampling):
             return False
@@ -193,10 +207,12 @@ class Engine:
                 return False
         return True
 
-    def _entries_of(self, plan: StepPlan):
+    def _entries_of(self, plan: StepPlan, unread_rows: Optional[Dict[int, int]] = None):
         """The plan as batch entries, checked on the way: a planner's mistake stops here, before any compute.
 
-        Returns (entries, the sequences that sample after this step, prompt tokens, decoded tokens).
+        ``unread_rows``: for the sequences whose last token is still on the GPU, its place among the tokens the
+        step before left there. Returns (entries, the sequences that sample after this step, prompt tokens,
+        decoded tokens).
         """
         serving = self.serving
         if len(plan.seqs) > serving.max_seqs or plan.total_tokens > serving.max_tokens_per_step:
@@ -226,34 +242,45 @@ class Engine:
             else:
                 prompt_tokens += n
             tokens = seq.tokens[first:last]
+            token_from = -1
             if tokens[-1] == UNREAD:             # the GPU knows it, the host does not: the step takes it from there
-                if n != 1:
+                token_from = -1 if unread_rows is None else unread_rows.get(id(seq), -1)
+                if n != 1 or token_from < 0:
                     raise InvalidArgument(f"sequence {seq.id} would run {n} tokens, one of them not read yet")
                 tokens = (0,)
             if last == len(seq.tokens):          # all it has is cached after this step: it samples
-                entries.append(StepEntry(seq.cache, first, tokens, (n - 1,)))
+                entries.append(StepEntry(seq.cache, first, tokens, (n - 1,), token_from))
                 sampling.append(seq)
             else:
-                entries.append(StepEntry(seq.cache, first, tokens, ()))
+                entries.append(StepEntry(seq.cache, first, tokens, (), token_from))
         return entries, sampling, prompt_tokens, decoded_tokens
 
     def _carry_out(self, plan: StepPlan, unread: Optional[_Unread] = None) -> None:
         """Runs a plan. ``unread``: the step before it, whose tokens are still on the GPU (the steady state)."""
         self._unread = None                # held in ``unread`` from here on; put back if this step never runs
         try:
-            if unread is not None and not (len(plan.seqs) == len(unread.sampling) and all(
-                    share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, unread.sampling))):
-                # Planning changed the picture (a sequence was evicted to make room): read first after all.
-                self.ahead_replans += 1
-                self._read(unread)
-                unread = None
-                for share in [s for s in plan.seqs if s.seq.state == SeqState.FINISHED]:
-                    plan.seqs.remove(share)          # it met a stop token; what was reserved for it went back with it
-                    plan.total_tokens -= share.num_tokens
-                if not plan.seqs:
-                    self.scheduler.complete(plan)
-                    return
-            entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan)
+            unread_rows, repeats = None, False
+            if unread is not None:
+                unread_rows = {id(seq): row for row, seq in enumerate(unread.sampling)}
+                repeats = len(plan.seqs) == len(unread.sampling) and all(
+                    share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, unread.sampling))
+                if not repeats:
+                    self.ahead_replans += 1        # (an eviction to make room, a prompt beside the decoders, ...)
+                # The plan can run over the unread tokens if every share that ends in one is that one token of a
+                # sequence of the step before; rows that draw need the step before repeated exactly.
+                fits = all(share.seq.tokens[share.seq.num_computed + share.num_tokens - 1] != UNREAD or
+                           (share.num_tokens == 1 and id(share.seq) in unread_rows) for share in plan.seqs)
+                if not fits or not (repeats or all(seq.params.greedy for seq in unread.sampling)):
+                    self._read(unread)
+                    unread = unread_rows = None
+                    repeats = False
+                    for share in [s for s in plan.seqs if s.seq.state == SeqState.FINISHED]:
+                        plan.seqs.remove(share)      # it met a stop token; what was reserved for it went back with it
+                        plan.total_tokens -= share.num_tokens
+                    if not plan.seqs:
+                        self.scheduler.complete(plan)
+                        return
+            entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan, unread_rows)
             began = time.perf_counter()
             # Queued on the GPU; the sampling kernels queue right behind.
             logits = self.runner.step(entries, None if unread is None else unread.ticket.device_tokens)
@@ -286,8 +313,10 @@ class Engine:
                 if all(s.params.greedy for s in sampling):
                     ticket = self.sampler.launch_greedy(logits)
                 else:
+                    # Rows that drew in the unread step (it is then this step's like: see above) take the number
+                    # their stream will be at once that step is read.
                     ticket = self.sampler.launch(logits, [s.params for s in sampling], [s.rng for s in sampling],
-                                                 None if unread is None else unread.ticket)
+                                                 unread.ticket if unread is not None and repeats else None)
             except BaseException:
                 self._end_all(sampling, FinishReason.ERROR)
                 raise

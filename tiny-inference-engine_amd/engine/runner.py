@@ -70,9 +70,9 @@ class ModelRunner:
 
         The returned tensor is scratch memory of the runner: it is valid until the next step.
 
-        ``device_tokens`` (int32 on the device, one per entry, in the entries' order; only for steps in which
-        every entry brings one token): the tokens to run, which the host does not know yet - an earlier step's
-        sampling kernel left them there. The entries' own token values are then ignored.
+        ``device_tokens`` (int32 on the device): tokens the host does not know yet - an earlier step's sampling
+        kernel left them there. An entry with ``token_from >= 0`` brings one token, whose value is
+        ``device_tokens[token_from]``; the value the entry itself names is ignored.
         """
         total = 0
         for e in entries:
@@ -84,10 +84,13 @@ class ModelRunner:
             raise CapacityError(f"a step of {total} tokens exceeds the {kernels.MAX_STEP_TOKENS} the kernels take; "
                                 f"cut the prompt into portions")
         batch = self.builder.build(entries)
-        if device_tokens is not None:
-            if not batch.all_decode or device_tokens.numel() != batch.num_tokens or device_tokens.dtype != torch.int32:
-                raise InvalidArgument("tokens on the device need a step of single tokens and one int32 per entry")
-            batch.tokens.copy_(device_tokens)      # queued behind the copy of the step's arrays, before any kernel
+        if batch.takes_device_tokens:
+            if device_tokens is None or device_tokens.dtype != torch.int32 or \
+                    max(e.token_from for e in entries) >= device_tokens.numel():
+                raise InvalidArgument("an entry takes its token from the device: the step needs the int32 tokens an "
+                                      "earlier step left there, as many as the entries point into")
+            # queued behind the copy of the step's arrays, before any kernel of the step
+            kernels.take_tokens(batch.tokens, batch.token_sources, device_tokens)
         if not (self.use_graphs and batch.all_decode and self.model.layer_hook is None):
             return self._forward(batch)
 

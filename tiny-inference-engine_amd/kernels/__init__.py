@@ -80,6 +80,7 @@ _SIGNATURES = {
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
+        "tie_take_tokens": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_random_fill": [_c_void, ctypes.c_longlong, ctypes.c_ulonglong, _c_int, ctypes.c_double, _c_void],
         "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
@@ -374,6 +375,17 @@ def cast(x: torch.Tensor, out: torch.Tensor) -> None:
         raise InvalidArgument("cast: sizes differ")
     _call(_lib("elementwise").tie_cast, "cast", x.data_ptr(), _code(x, "cast input"), out.data_ptr(),
                                         _code(out, "cast output"), x.numel(), _stream())
+
+
+def take_tokens(tokens: torch.Tensor, sources: torch.Tensor, previous: torch.Tensor) -> None:
+    """``tokens[i] = previous[sources[i]]`` where ``sources[i] >= 0`` (all int32 on the device): the rows of a step
+    whose token an earlier step's sampling left on the GPU, unread by the host."""
+    T = tokens.numel()
+    _i32(tokens, "tokens")
+    _i32(sources, "token sources", T)
+    _i32(previous, "the earlier step's tokens")
+    _call(_lib("elementwise").tie_take_tokens, "take_tokens", tokens.data_ptr(), sources.data_ptr(), previous.data_ptr(),
+          T, previous.numel(), _stream())
 
 
 def random_fill(out: torch.Tensor, key: int, kind: str, scale: float) -> None:
