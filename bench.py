@@ -100,7 +100,7 @@ def measure_stress(model, cfg, args):
     from tie_amd.bench import assign_arrivals, report_json, run_workload, summarize, synthetic_requests
 
     engine = create_engine(model, kv_mem=args.kv_mem, block_size=BLOCK_SIZE, max_seqs=args.requests,
-                           max_tokens_per_step=512, prefill_chunk=512)
+                           max_tokens_per_step=512, prefill_chunk=512, launch_ahead=args.launch_ahead)
     requests = synthetic_requests(args.requests, (128, 2048), (256, 256), cfg["vocab_size"], seed=0)
     assign_arrivals(requests, float("inf"), seed=0)
     warm = synthetic_requests(4, (600, 700), (8, 8), cfg["vocab_size"], seed=1)       # compiles nothing, but warms up
@@ -223,6 +223,8 @@ def main():
                         help="decode: the headline measurement; stress: many requests through a small cache")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
     parser.add_argument("--kv-mem", type=int, default=2 << 30, help="stress: bytes of cache")
+    parser.add_argument("--launch-ahead", type=int, default=1,
+                        help="stress: steps the engine may leave unread behind the one it queues (0: reads every step at once)")
     parser.add_argument("--skip-points", action="store_true", help="skip batch 1, batch 64 and the prefill")
     parser.add_argument("--temperature", type=float, default=0.0, help="decode: sampling temperature (0 = greedy)")
     parser.add_argument("--top-k", type=int, default=0, help="decode: with a temperature, keep the k most likely (0 = all)")
@@ -262,7 +264,8 @@ def main():
             "config": {"model": f"{shape_name} shape, random weights", "layers": layers_of_shape,
                        "layers_run": cfg["num_hidden_layers"], "requests": args.requests, "prompt_len": "128:2048",
                        "output_len": 256, "prefill_chunk": 512, "max_tokens_per_step": 512, "kv_bytes": args.kv_mem,
-                       "kv_block": BLOCK_SIZE, "policy": "srpt-aging", "sampling": "greedy"},
+                       "kv_block": BLOCK_SIZE, "policy": "srpt-aging", "sampling": "greedy",
+                       "launch_ahead": args.launch_ahead},
             "report": report}), flush=True)
         return 0
 

@@ -16,7 +16,7 @@ from tie_amd.cache.manager import CacheManager
 from tie_amd.cache.spec import PagedKV, plan_cache
 from tie_amd.engine.engine import Engine
 from tie_amd.engine.scheduler import FCFS, SRPT_AGING, BatchScheduler, SchedulerConfig
-from tie_amd.engine.sequence import SeqState
+from tie_amd.engine.sequence import UNREAD, SeqState
 from tie_amd.engine.serving import ServingConfig
 from tie_amd.sampling.params import SamplingParams
 
@@ -117,7 +117,7 @@ def run_all(engine, requests, arrivals=None, limit=20000):
 
 
 @pytest.mark.parametrize("policy", [FCFS, SRPT_AGING])
-@pytest.mark.parametrize("launch_ahead", [False, True])
+@pytest.mark.parametrize("launch_ahead", [False, True, 2, 3])
 def test_random_workloads_over_small_pools_lose_nobody(policy, launch_ahead):
     evictions = ahead = mixed_ahead = steps = 0
     for seed in range(300):
@@ -127,12 +127,15 @@ def test_random_workloads_over_small_pools_lose_nobody(policy, launch_ahead):
         arrivals = [rng.randint(0, 8) for _ in range(n)]
         longest = max(len(p) + c for p, c in requests)
         blocks = (longest + 3) // 4 + rng.randint(0, 5)            # the longest fits alone, little more
+        # every other workload has stop tokens: a sequence that meets one has run ahead, and what it ran is dropped
+        stop = tuple(rng.sample(range(VOCAB), 6)) if seed % 2 else ()
         engine = make_engine(blocks, rng.randint(4, 12), rng.randint(2, 4), policy, launch_ahead,
-                             prefill_chunk=rng.choice([0, 3, 5]))
+                             prefill_chunk=rng.choice([0, 3, 5]), stop=stop)
         done = run_all(engine, requests, arrivals)
         for i, (prompt, count) in enumerate(requests):
             assert done[i].state == SeqState.FINISHED
-            assert done[i].generated == expected(prompt, count), f"seed {seed}, request {i}"
+            assert done[i].generated == expected(prompt, count, stop), f"seed {seed}, request {i}"
+            assert UNREAD not in done[i].tokens
         assert engine.cache.all_free()
         evictions += engine.stats().preemptions
         ahead += engine.steps_launched_ahead
@@ -153,13 +156,13 @@ def test_an_eviction_while_tokens_are_unread_keeps_the_evicted_request():
     requests = [([1, 2, 3], 9), ([4, 5, 6], 9), ([7, 8, 9], 9), ([10, 11, 12], 9)]
     engine = make_engine(5, 16, 4, FCFS, launch_ahead=True)
     most_waiting = 0
-    real_read = engine._read
+    real_read = engine._read_oldest
 
-    def counting_read(unread, keep=None):
-        real_read(unread, keep)
+    def counting_read():
+        real_read()
         nonlocal most_waiting
         most_waiting = max(most_waiting, sum(s.num_preemptions > 0 for s in engine.scheduler.waiting))
-    engine._read = counting_read
+    engine._read_oldest = counting_read
     done = run_all(engine, requests)          # checks after every step that a request is in exactly one place
     assert engine.ahead_replans > 0, "no plan was changed by an eviction while tokens were unread"
     assert most_waiting >= 2 and engine.stats().preemptions >= 2 and engine.steps_launched_ahead > 0

@@ -466,7 +466,7 @@ def test_steps_launched_ahead_generate_the_same_tokens(model_folders, model_fold
             if steps == 12:
                 engine.cancel(ids[2])
             assert steps < 2000
-        assert engine.cache.num_free() == kv_blocks and engine._unread is None
+        assert engine.cache.num_free() == kv_blocks and not engine._unread
         out = [engine.sequence(i).generated for i in ids]
         reasons = [engine.sequence(i).finish_reason.value for i in ids]
         for i, tokens in zip(ids, out):

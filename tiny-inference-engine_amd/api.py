@@ -27,14 +27,14 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
                   block_size: int = 16, max_seqs: int = 64, max_tokens_per_step: int = 512, prefill_chunk: int = 0,
                   policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1,
                   stop_tokens: Sequence[int] = (), max_seq_len: Optional[int] = None,
-                  device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead: bool = True,
+                  device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead=True,
                   kv_dtype: Optional[str] = None) -> Engine:
     """``model`` is a folder (config.json + safetensors) or a Model that is already loaded.
 
     ``use_graphs`` False runs every step eagerly; None (the default) records decode-only steps into HIP
-    graphs in bfloat16 mode when every part of the model allows it. ``launch_ahead``: in the steady state of
-    decoding the next step is queued before the last one's tokens are read (``Engine``'s module text says how);
-    tokens then appear one ``step()`` later. ``kv_dtype``: the precision of the cached keys and values, by
+    graphs in bfloat16 mode when every part of the model allows it. ``launch_ahead``: steps are queued before
+    the tokens of the steps before them are read (``Engine``'s module text says how): True leaves one step
+    unread, a number that many, False none; tokens then appear that many ``step()`` calls later. ``kv_dtype``: the precision of the cached keys and values, by
     default that of ``dtype``; float32 arithmetic also runs over a bfloat16 or float16 cache (the reference's
     arrangement, ``src/kv/paged_kv_cache.h:18-25``). A pair no kernel takes is refused here, before anything
     is loaded."""

@@ -23,15 +23,20 @@ sequences decode, which prompts go on, who is admitted. Two things need the toke
 planning: a sequence whose unread token is its last (it ends, and planning it again would be wrong), and rows
 that draw from a random stream unless the step is the steady repetition of the one before (they carry both
 uniform numbers their stream may be at, see ``DeviceSampler``, which asks for the same rows in the same order).
-A sequence that turns out to have met a stop token has then run one token too many, which is dropped. Tokens
-(and callbacks) appear one ``step()`` later; ``has_work()`` stays true until they have.
+A sequence that turns out to have met a stop token has then run a token too many for each step queued behind
+its last, which are dropped. ``launch_ahead`` is also the number of steps that may stay unread once a step is
+queued (True: 1). More than one lets the host's quick steps run further ahead of its slow ones; measured on 64
+requests through a small cache it gains nothing over one (the GPU is then the limit) and makes the slowest
+gaps between a request's tokens longer, so one is the default. Tokens (and callbacks) appear that many
+``step()`` calls later; ``has_work()`` stays true until they have.
 """
 
 from __future__ import annotations
 
+import collections
 import dataclasses
 import time
-from typing import Callable, Dict, List, Optional, Sequence as Seq, Tuple
+from typing import Callable, Deque, Dict, List, Optional, Sequence as Seq, Tuple, Union
 
 from .. import kernels
 from ..cache.manager import CacheManager
@@ -56,6 +61,10 @@ class EngineStats:
     preemptions: int = 0
 
 
+class _PlanAgain(Exception):
+    """A plan was overtaken by what reading the unread steps showed; nothing of it has run."""
+
+
 class _Unread:
     """A launched step whose sampled tokens the host has not read: who sampled, where each token goes."""
 
@@ -70,7 +79,7 @@ class _Unread:
 class Engine:
     def __init__(self, model: Model, cache: CacheManager, scheduler=None, serving: Optional[ServingConfig] = None,
                  stop_tokens: Seq[int] = (), max_seq_len: Optional[int] = None, use_graphs: Optional[bool] = None,
-                 launch_ahead: bool = False, runner=None, sampler=None):
+                 launch_ahead: Union[bool, int] = False, runner=None, sampler=None):
         """``runner`` / ``sampler``: stand-ins with the interface of ``ModelRunner`` (``step``,
         ``max_blocks_per_seq``) and ``DeviceSampler`` (``launch_greedy``, ``launch``, ``collect``,
         ``sample_rows``), for driving the engine's bookkeeping without a GPU; the default builds the real ones."""
@@ -90,8 +99,11 @@ class Engine:
         self._stats = EngineStats()
         self._ids = 0
         self._inside_step = False
-        self.launch_ahead = bool(launch_ahead)
-        self._unread: Optional[_Unread] = None
+        # How many launched steps may stay unread after a step has been queued (0: every step is read at once).
+        self.launch_ahead = 1 if launch_ahead is True else max(0, int(launch_ahead))
+        if self.launch_ahead and hasattr(self.sampler, "keep_apart"):
+            self.sampler.keep_apart(self.launch_ahead + 2)      # result buffers of the unread steps and the next
+        self._unread: Deque[_Unread] = collections.deque()      # oldest first
         self.steps_launched_ahead = 0
         self.ahead_replans = 0      # steps planned over unread tokens whose plan was not the steady one after all
 
@@ -138,7 +150,7 @@ class Engine:
         return seq
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work() or self._unread is not None
+        return self.scheduler.has_work() or bool(self._unread)
 
     def cancel(self, seq_id: int) -> None:
         seq = self.sequence(seq_id)
@@ -170,29 +182,29 @@ class Engine:
             raise InvalidArgument("step() was called from inside a step (a token callback?)")
         self._inside_step = True
         try:
-            unread = self._unread
-            if unread is not None and not self._may_plan_over(unread):
-                self._read(unread)                 # a token is needed for the plan itself: know it first
-                unread = None
+            while self._unread and not self._may_plan_over():
+                self._read_oldest()                # a token is needed for the plan itself: know it first
             plan = self.scheduler.schedule()
             if plan:
-                self._carry_out(plan, unread)
-            elif unread is not None:
-                self._read(unread)
+                self._carry_out(plan)
+            else:
+                self._read_all()
         finally:
             self._inside_step = False
 
-    def _may_plan_over(self, unread: _Unread) -> bool:
-        """Whether the next step can be planned while the tokens of ``unread`` are still on the GPU."""
-        if not all(seq.params.greedy for seq in unread.sampling):
-            return self._steady(unread)            # rows that draw: only the same rows again, in the same order
-        for seq in unread.sampling:
-            if seq.state == SeqState.FINISHED:     # cancelled meanwhile: its token will be dropped
-                continue
-            if seq.state != SeqState.DECODING or seq.tokens[-1] != UNREAD:
-                return False
-            if len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:    # the unread token is its last
-                return False
+    def _may_plan_over(self) -> bool:
+        """Whether the next step can be planned while the tokens of the unread steps are still on the GPU."""
+        if any(not seq.params.greedy for unread in self._unread for seq in unread.sampling):
+            # rows that draw: only the same rows again, in the same order, and one step of them at a time
+            return len(self._unread) == 1 and self._steady(self._unread[0])
+        for unread in self._unread:
+            for seq in unread.sampling:
+                if seq.state == SeqState.FINISHED:     # cancelled meanwhile: its token will be dropped
+                    continue
+                if seq.state != SeqState.DECODING or seq.tokens[-1] != UNREAD:
+                    return False
+                if len(seq.tokens) - seq.prompt_len >= seq.params.max_tokens:    # an unread token is its last
+                    return False
         return True
 
     def _steady(self, unread: _Unread) -> bool:
@@ -255,24 +267,30 @@ class Engine:
                 entries.append(StepEntry(seq.cache, first, tokens, (), token_from))
         return entries, sampling, prompt_tokens, decoded_tokens
 
-    def _carry_out(self, plan: StepPlan, unread: Optional[_Unread] = None) -> None:
-        """Runs a plan. ``unread``: the step before it, whose tokens are still on the GPU (the steady state)."""
-        self._unread = None                # held in ``unread`` from here on; put back if this step never runs
+    def _carry_out(self, plan: StepPlan) -> None:
+        """Runs a plan, over the unread steps if it can: the rows that continue a sequence whose last token is
+        still on the GPU take it from the latest unread step's sampling output."""
         try:
+            latest = self._unread[-1] if self._unread else None
             unread_rows, repeats = None, False
-            if unread is not None:
-                unread_rows = {id(seq): row for row, seq in enumerate(unread.sampling)}
-                repeats = len(plan.seqs) == len(unread.sampling) and all(
-                    share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, unread.sampling))
+            if latest is not None:
+                unread_rows = {id(seq): row for row, seq in enumerate(latest.sampling)}
+                repeats = len(plan.seqs) == len(latest.sampling) and all(
+                    share.seq is seq and share.num_tokens == 1 for share, seq in zip(plan.seqs, latest.sampling))
                 if not repeats:
                     self.ahead_replans += 1        # (an eviction to make room, a prompt beside the decoders, ...)
                 # The plan can run over the unread tokens if every share that ends in one is that one token of a
-                # sequence of the step before; rows that draw need the step before repeated exactly.
+                # sequence of the latest unread step; rows that draw need that step alone, repeated exactly.
+                def continues_latest(share) -> bool:
+                    row = unread_rows.get(id(share.seq))
+                    return share.num_tokens == 1 and row is not None and \
+                        latest.places[row] == share.seq.num_computed == len(share.seq.tokens) - 1
                 fits = all(share.seq.tokens[share.seq.num_computed + share.num_tokens - 1] != UNREAD or
-                           (share.num_tokens == 1 and id(share.seq) in unread_rows) for share in plan.seqs)
-                if not fits or not (repeats or all(seq.params.greedy for seq in unread.sampling)):
-                    self._read(unread)
-                    unread = unread_rows = None
+                           continues_latest(share) for share in plan.seqs)
+                draws = any(not seq.params.greedy for unread in self._unread for seq in unread.sampling)
+                if not fits or (draws and not (repeats and len(self._unread) == 1)):
+                    self._read_all()
+                    latest = unread_rows = None
                     repeats = False
                     for share in [s for s in plan.seqs if s.seq.state == SeqState.FINISHED]:
                         plan.seqs.remove(share)      # it met a stop token; what was reserved for it went back with it
@@ -281,17 +299,27 @@ class Engine:
                         self.scheduler.complete(plan)
                         return
             entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan, unread_rows)
+            if latest is not None and any(not seq.params.greedy for seq in sampling) and \
+                    not (repeats and len(self._unread) == 1):
+                # Rows that begin to draw in this step: their streams stand where the host's do only once
+                # everything before has been read (nothing of this step is queued yet).
+                self._read_all()
+                if any(share.seq.state == SeqState.FINISHED for share in plan.seqs):
+                    raise _PlanAgain()
+                latest = None
+                entries, sampling, prompt_tokens, decoded_tokens = self._entries_of(plan, None)
             began = time.perf_counter()
             # Queued on the GPU; the sampling kernels queue right behind.
-            logits = self.runner.step(entries, None if unread is None else unread.ticket.device_tokens)
-        except BaseException:
+            logits = self.runner.step(entries, None if latest is None else latest.ticket.device_tokens)
+        except BaseException as error:
             # Nothing of the step counts: the pages reserved for it go back and the plan's sequences are free
             # to be planned again.
             for share in plan.seqs:
                 if share.seq.state != SeqState.FINISHED:
                     self.cache.truncate(share.seq.cache, share.seq.num_computed)
             self.scheduler.abandon(plan)
-            self._unread = unread
+            if isinstance(error, _PlanAgain):
+                return                             # the next step() plans afresh, everything read
             raise
         stats = self._stats
         stats.steps += 1
@@ -305,7 +333,7 @@ class Engine:
             if windows:
                 self.cache.trim(seq.cache, seq.num_computed)     # pages a window has passed go back now
         self.scheduler.complete(plan)
-        if unread is not None:
+        if latest is not None:
             self.steps_launched_ahead += 1
         tokens: List[int] = []
         if sampling and self.launch_ahead:
@@ -316,14 +344,14 @@ class Engine:
                     # Rows that drew in the unread step (it is then this step's like: see above) take the number
                     # their stream will be at once that step is read.
                     ticket = self.sampler.launch(logits, [s.params for s in sampling], [s.rng for s in sampling],
-                                                 unread.ticket if unread is not None and repeats else None)
+                                                 latest.ticket if latest is not None else None)
             except BaseException:
                 self._end_all(sampling, FinishReason.ERROR)
                 raise
             for seq in sampling:
                 seq.tokens.append(UNREAD)
                 seq.state = SeqState.DECODING
-            self._unread = _Unread(sampling, [len(seq.tokens) - 1 for seq in sampling], ticket)
+            self._unread.append(_Unread(sampling, [len(seq.tokens) - 1 for seq in sampling], ticket))
             sampling = []
         elif sampling:
             try:
@@ -332,14 +360,14 @@ class Engine:
                 self._end_all(sampling, FinishReason.ERROR)
                 raise
         stats.step_seconds += time.perf_counter() - began     # reading the tokens waited for the GPU
-        if unread is not None:
-            self._read(unread, keep=self._unread)                 # the step before, while this one runs (keep: this one's)
+        while len(self._unread) > self.launch_ahead:
+            self._read_oldest()                                # earlier steps, while this one runs
         if sampling:
             self._deliver(sampling, tokens)
 
-    def _read(self, unread: _Unread, keep: Optional[_Unread] = None) -> None:
-        """Waits for a launched step's tokens, puts them where UNREAD stands, and delivers them."""
-        self._unread = keep
+    def _read_oldest(self) -> None:
+        """Waits for the oldest unread step's tokens, puts them where UNREAD stands, and delivers them."""
+        unread = self._unread.popleft()
         began = time.perf_counter()
         try:
             tokens = self.sampler.collect(unread.ticket)
@@ -348,6 +376,10 @@ class Engine:
             raise
         self._stats.step_seconds += time.perf_counter() - began
         self._deliver(unread.sampling, tokens, unread.places)
+
+    def _read_all(self) -> None:
+        while self._unread:
+            self._read_oldest()
 
     def _end_all(self, seqs: Seq[Sequence], reason: FinishReason) -> None:
         for seq in seqs:

@@ -97,7 +97,8 @@ class DeviceSampler:
     -inf), a drawing kernel for the rows with a temperature and one for those with top-k or top-p, which put
     their tokens where the argmax stood, one copy of ``2 R`` words and one wait. ``launch`` / ``collect`` split
     that into asking and reading, so that a caller may queue the next step (whose tokens it takes from
-    ``ticket.device_tokens``) before it reads this one's; two sets of buffers alternate for that.
+    ``ticket.device_tokens``) before it reads this one's; sets of buffers take turns for that (two, or as many as
+    ``keep_apart`` says).
 
     A row's uniform number is the next of its request's stream, but a row with a +inf logit takes none, and
     whether that happened in a step not yet read is known on the GPU only. A step queued behind such a step
@@ -112,6 +113,13 @@ class DeviceSampler:
         self._rows = 0
         self._sets = []
         self._turn = 0
+        self._num_sets = 2
+
+    def keep_apart(self, tickets: int) -> None:
+        """How many tickets may be outstanding or in the making at a time: each has a set of buffers of its own."""
+        if tickets > self._num_sets:
+            self._num_sets = tickets
+            self._rows = 0                 # the next launch makes the sets anew (outstanding tickets keep theirs)
 
     def _buffers(self, rows: int):
         if rows > self._rows:
@@ -119,8 +127,8 @@ class DeviceSampler:
             words = (self.RESULTS + self.PARAMETERS) * self._rows
             self._sets = [(torch.empty(words, dtype=torch.int32, device=self.device),
                            torch.empty(words, dtype=torch.int32, pin_memory=self.device.type == "cuda"))
-                          for _ in range(2)]
-        self._turn ^= 1
+                          for _ in range(self._num_sets)]
+        self._turn = (self._turn + 1) % self._num_sets
         return self._sets[self._turn]
 
     # ------------------------------------------------------------------------- asked for and read apart
