@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
     python bench.py --shape 32b                 the same measurements at the Qwen3-32B sizes
+    python bench.py --sweep [--shape 32b]       decode at contexts 4096 / 16384 / 32768 x batch 1 / 8 / 32, a line a point
     python bench.py --workload stress           64 requests through the scheduler at the Qwen3-1.7B sizes
 
 Prints ONE JSON line. A "step" is one decode step of the engine (schedule, build the batch, run
@@ -229,6 +230,10 @@ def main():
     parser.add_argument("--temperature", type=float, default=0.0, help="decode: sampling temperature (0 = greedy)")
     parser.add_argument("--top-k", type=int, default=0, help="decode: with a temperature, keep the k most likely (0 = all)")
     parser.add_argument("--top-p", type=float, default=1.0, help="decode: with a temperature, nucleus mass (1 = all)")
+    parser.add_argument("--sweep", action="store_true",
+                        help="decode only, one JSON line for every (context, batch) of --sweep-contexts x --sweep-batches")
+    parser.add_argument("--sweep-contexts", default="4096,16384,32768")
+    parser.add_argument("--sweep-batches", default="1,8,32")
     parser.add_argument("--prefill-only", action="store_true",
                         help="run only the 2048-token prefill (for profiling); prints its figures alone")
     args = parser.parse_args()
@@ -287,9 +292,9 @@ def main():
     log(f"this GPU: a streaming read reaches {peaks['hbm_read_gbs']:.0f} GB/s, matrix instructions on registers "
         f"{peaks['mfma_bf16_tflops']:.0f} TFLOP/s")
 
-    def decode_point(batch):
+    def decode_point(batch, context=None):
         """One decode measurement: ``--steps`` timed steps at ``batch``; the figures of its roofline."""
-        seconds, mean_context, replays, median = measure_decode(model, cfg, batch, args.context, args.steps,
+        seconds, mean_context, replays, median = measure_decode(model, cfg, batch, context or args.context, args.steps,
                                                                 args.warmup, chunk, sampling)
         ms = seconds / args.steps * 1e3
         step_bytes = weight_bytes_per_step(cfg, batch) + batch * mean_context * kv_bytes_per_token(cfg)
@@ -298,6 +303,24 @@ def main():
             f"{batch * args.steps / seconds:.1f} tok/s, {achieved:.0f} GB/s ({replays} replays)")
         return {"tok_s": batch * args.steps / seconds, "ms": ms, "median_ms": median * 1e3, "gb": step_bytes / 1e9,
                 "gbs": achieved, "frac": achieved / PEAK_HBM_GBS, "frac_of_measured": achieved / peaks["hbm_read_gbs"]}
+
+    if args.sweep:
+        # One line a point: decode at the contexts and batch sizes named, for tables of other sizes than the headline's.
+        for context in [int(c) for c in args.sweep_contexts.split(",")]:
+            for batch in [int(b) for b in args.sweep_batches.split(",")]:
+                point = decode_point(batch, context)
+                print(json.dumps({"metric": f"decode tok/s @ batch {batch}, context {context}, {shape_name} bf16",
+                                  "value": round(point["tok_s"], 2), "unit": "tokens/s", "steps": args.steps,
+                                  "ms_per_step": round(point["ms"], 4), "ms_per_step_median": round(point["median_ms"], 4),
+                                  "config": {"model": f"{shape_name} shape, random weights", "layers": layers_of_shape,
+                                             "layers_run": cfg["num_hidden_layers"], "global_batch": batch,
+                                             "seq_len": context, "kv_block": BLOCK_SIZE},
+                                  "roofline": {"bound": "hbm", "bytes_gb": round(point["gb"], 3),
+                                               "achieved": round(point["gbs"], 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                               "frac": round(point["frac"], 4),
+                                               "measured_peak": round(peaks["hbm_read_gbs"], 1),
+                                               "frac_of_measured": round(point["frac_of_measured"], 4)}}), flush=True)
+        return 0
 
     main_point = decode_point(args.batch)
     result = {

@@ -1121,3 +1121,67 @@ def test_random_weights_are_the_same_bits_on_the_gpu_and_on_the_host():
     assert list(on_host) == list(on_gpu)
     for name, t in on_host.items():
         assert torch.equal(on_gpu[name].cpu().float(), t.float()), name
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (3, 4096, 4096), (8, 96, 12288), (16, 1024, 160)])
+@pytest.mark.parametrize("packed", [True, False])
+def test_decode_product_with_the_norms_work_in_its_epilogue(M, N, K, packed):
+    """The product that ends a sub-layer adds to the stream in place and leaves bf16(stream * weight) and the sums
+    of the stream's squares per 16-column tile; the products that read those rows multiply their sums by
+    1 / sqrt(sum of squares / n + eps) - stored whole, in planes over K, or under the gated activation. Against
+    the formulas in float64, and the stream's new value bit for bit against the same product without the
+    epilogue's extra work. Chained, the two give what RMSNorm between two products gives (src/model/qwen3.cpp:
+    230-235: o_proj, add, rms_norm, gate/up)."""
+    from tie_amd import kernels
+
+    x = rnd(M, K, seed=41, dtype=torch.bfloat16).cuda()
+    w = rnd(N, K, seed=42, scale=0.05, dtype=torch.bfloat16).cuda()
+    weight = kernels.pack_weight(w) if packed and kernels.packable(w) else w
+    if packed and weight is w:
+        pytest.skip("this shape cannot be packed")
+    stream = rnd(M, N, seed=43).cuda()
+    norm_w = (1 + 0.1 * rnd(N, seed=44)).cuda()
+    plainly = stream.clone()
+    kernels.skinny_gemm_bf16(x, weight, plainly, accumulate=True)
+    got = stream.clone()
+    rows = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    squares = torch.full((M, N // 16), float("nan"), device="cuda")
+    kernels.skinny_gemm_bf16(x, weight, got, accumulate=True, next_norm=(norm_w, rows, squares))
+    assert torch.equal(got, plainly), "the stream differs from the product without the norm's work"
+    want = stream.cpu().to(F64) + plain.linear(x.cpu(), w.cpu())
+    close(got, want, 1e-5, "stream")
+    assert torch.equal(rows, (got * norm_w).to(torch.bfloat16)), "rows for the next norm"
+    close(squares, (got.cpu().to(F64) ** 2).view(M, N // 16, 16).sum(-1), 1e-6, "sums of squares")
+
+    # the consumers: x2 = rows (no 1 / rms yet) against a second weight
+    eps = 1e-5
+    inv = 1.0 / torch.sqrt((got.cpu().to(F64) ** 2).mean(-1, keepdim=True) + eps)
+    scale = kernels.RowScale(squares, N, eps)
+    N2 = 192
+    w2 = rnd(N2, N, seed=45, scale=0.05, dtype=torch.bfloat16).cuda()
+    weight2 = kernels.pack_weight(w2) if packed and kernels.packable(w2) else w2
+    unscaled = plain.linear(rows.cpu(), w2.cpu())
+    out = torch.empty(M, N2, device="cuda")
+    kernels.skinny_gemm_bf16(rows, weight2, out, row_scale=scale)
+    close(out, unscaled * inv, 1e-5, "scaled product")
+    if N % 256 == 0:                                   # planes over K need k-blocks enough for every range
+        planes = torch.empty(4, M, N2, device="cuda")
+        kernels.skinny_gemm_bf16(rows, weight2, planes, splits=4, row_scale=scale)
+        close(planes.sum(0), unscaled * inv, 1e-5, "scaled product in four planes")
+    gate, up = w2[:N2 // 2], w2[N2 // 2:]
+    both = kernels.interleave_gate_up(gate.contiguous(), up.contiguous())
+    both = kernels.pack_weight(both) if packed and kernels.packable(both) else both
+    act = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device="cuda")
+    kernels.linear_swiglu(rows, both, act, row_scale=scale)
+    g, u = unscaled[:, :N2 // 2] * inv, unscaled[:, N2 // 2:] * inv
+    close(act, g / (1 + torch.exp(-g)) * u, 1e-2, "gated product of scaled sums")
+    # and against the norm itself: (stream * inv * norm_w) @ w2^T, the reference's order of operations
+    normed = plain.rms_norm(got.cpu().to(F64), norm_w.cpu().to(F64), eps)
+    close(out, plain.linear(normed, w2.cpu()), 1e-2, "the two epilogues against RMSNorm between the products")
+    # rows that go where no epilogue applies the factor get it in place
+    copy = rows.clone()
+    kernels.scale_rows(copy, scale)
+    close(copy, rows.cpu().to(F64) * inv, 1e-2, "rows scaled in place")
+    with pytest.raises(kernels.InvalidArgument):
+        kernels.skinny_gemm_bf16(rnd(17, K, dtype=torch.bfloat16).cuda(), weight, torch.empty(17, N, device="cuda"),
+                                 row_scale=scale)

@@ -116,10 +116,13 @@ def test_sums_a_product_leaves_owed_reach_the_stream_through_the_norm_or_settle(
     ctx = make_ctx(T, "bfloat16")
     residual = x.cuda().clone()
     ffn.forward(ctx, h.cuda(), residual)
-    assert ctx._owed is not None, "a product over 1024 of K at this size is expected to leave its sum owed"
+    # up to 16 rows the whole product is still to be launched (the next norm may ask for it with its own work in
+    # the epilogue); above, its planes of partial sums are owed
+    assert (ctx._pending if T <= 16 else ctx._owed) is not None, \
+        "a product over 1024 of K at this size is expected to leave its sum owed"
     assert torch.equal(residual.cpu(), x)                          # nothing added yet
     normed = norm.forward(ctx, residual)                           # adds what is owed, then normalises
-    assert ctx._owed is None
+    assert ctx._owed is None and ctx._pending is None
     close(residual, want, 2e-3, "stream after the norm took the owed sums")
     close(normed, plain.rms_norm(want, w["n"].to(F64), 1e-5), 1e-2, "norm of the updated stream")
 
@@ -127,7 +130,7 @@ def test_sums_a_product_leaves_owed_reach_the_stream_through_the_norm_or_settle(
     residual2 = x.cuda().clone()
     ffn.forward(ctx, h.cuda(), residual2)
     ctx.settle()                                                   # what a block does before a part that does not know
-    assert ctx._owed is None and torch.equal(residual2, residual)
+    assert ctx._owed is None and ctx._pending is None and torch.equal(residual2, residual)
 
 
 @pytest.mark.parametrize("T", [4, 200])
@@ -150,7 +153,8 @@ def test_two_products_in_a_row_that_leave_their_sums_owed(T):
     ctx = make_ctx(T, "bfloat16")
     residual = stream.cuda().clone()
     first(x1.cuda(), residual, accumulate=True, ctx=ctx)
-    assert ctx._owed is not None, "a product over 1024 of K at this size is expected to leave its sum owed"
+    assert (ctx._pending if T <= 16 else ctx._owed) is not None, \
+        "a product over 1024 of K at this size is expected to leave its sum owed"
     second(x2.cuda(), residual, accumulate=True, ctx=ctx)
     ctx.settle()
     close(residual, want, 2e-3, "stream after two owed products")

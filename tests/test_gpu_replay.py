@@ -207,6 +207,66 @@ def test_decode_steps_with_and_without_the_attention_kernel_that_prepares(folder
         assert float((a - b).abs().max() / b.abs().max()) < 2e-2, f"request {rid}: the two ways differ by more than rounding"
 
 
+# Every width a multiple of 32 and none under 96, so that every projection is stored in the decode product's
+# packed layout: only such products take the norms' work (tiny A and B keep some or all of theirs unpacked).
+PACKED_WIDTHS = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 3, "hidden_size": 160, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 32, "intermediate_size": 224, "vocab_size": 300, "rope_theta": 50000.0,
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 128,
+}
+
+
+def test_steps_of_a_few_rows_leave_the_norms_to_the_products(tmp_path, monkeypatch):
+    """In steps of up to 16 rows the product that ends a sub-layer adds to the stream and prepares the next norm in
+    its epilogue, and the products behind that norm apply its 1 / rms: no norm kernel runs between the layers'
+    parts. Both ways against the plain implementation, through decoding, small portions and mixed steps; the norm
+    kernels that still run are the first layer's first (nothing precedes it) and the head's."""
+    from tie_amd import kernels
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.weights.random_init import write_random_model
+
+    cfg = PACKED_WIDTHS
+    folder = str(tmp_path)
+    write_random_model(folder, cfg, seed=31, dtype="bfloat16")
+    requests = th.make_requests(cfg["vocab_size"], [5, 11, 17, 40, 64, 33], seed=15)
+    want = reference_logits(folder, cfg, requests)
+    layers = cfg["num_hidden_layers"]
+    calls = []
+    for fn in ("rms_norm", "add_partials"):
+        real = getattr(kernels, fn)
+        monkeypatch.setattr(kernels, fn, lambda *a, _real=real, _fn=fn, **k: (calls.append(_fn), _real(*a, **k))[1])
+    steps, peak = th.mixed(requests, max_live=4, seed=9, sizes=(31, 7, 2, 18, 3, 2, 9))
+    got = {}
+    for in_products in (True, False):
+        monkeypatch.setattr(kernels, "NORMS_IN_PRODUCTS", in_products)
+        rep = TraceReplayer.from_folder(folder, "bfloat16", peak, block_size=16, use_graphs=False)
+        norm_kernels = {}
+        real_step = rep.run_step
+
+        def counted(step, _real=real_step, _seen=norm_kernels):
+            del calls[:]
+            out = _real(step)
+            rows = sum(len(e["tokens"]) for e in step["entries"])
+            _seen.setdefault(rows <= kernels.NORM_EPILOGUE_ROWS, []).append(len(calls))
+            return out
+
+        rep.run_step = counted
+        got[in_products] = th.collect(rep, steps)
+        check(got[in_products], want, "bfloat16", f"packed widths/mixed, norms in the products: {in_products}",
+              tolerance=tolerances.BFLOAT16["packed widths"])
+        assert norm_kernels[True] and norm_kernels[False], "the trace needs steps of few rows and of many"
+        if in_products:
+            assert max(norm_kernels[True]) <= 3, f"steps of few rows launched {norm_kernels[True]} norm kernels"
+        else:
+            assert min(norm_kernels[True]) >= 2 * layers
+        assert min(norm_kernels[False]) >= 2 * layers          # steps of many rows: every norm a kernel
+    for rid in requests:
+        a = torch.stack([got[True][rid][p] for p in sorted(got[True][rid])])
+        b = torch.stack([got[False][rid][p] for p in sorted(got[False][rid])])
+        assert float((a - b).abs().max() / b.abs().max()) < 1e-2, f"request {rid}: the two ways differ by more than rounding"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("use_graphs", [False, True])
 def test_layers_of_one_shape_run_from_one_layers_launch_list(tmp_path, dtype, use_graphs):

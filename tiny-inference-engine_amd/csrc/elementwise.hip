@@ -185,6 +185,35 @@ extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_
   return tie_launch_status();
 }
 
+// ------------------------------------------------------------ rows that lack their norm's factor
+// rows[m][:] *= 1 / sqrt((squares[m][0] + ... + squares[m][tiles - 1]) / n + eps): the sums of squares come per
+// 16-column tile from the product that prepared the rows; lane l adds the tiles l, l + 64, ... in ascending
+// order and the lanes meet in a fixed butterfly, as in the products that apply the factor themselves.
+template <typename T>
+__global__ void scale_rows_kernel(T* __restrict__ rows, int width, const float* __restrict__ squares, int tiles,
+                                  float n, float eps) {
+  __shared__ float factor;
+  const int m = blockIdx.x;
+  if (threadIdx.x < TIE_WAVE) {
+    float sq = 0.f;
+    for (int t = threadIdx.x; t < tiles; t += TIE_WAVE) sq += squares[static_cast<size_t>(m) * tiles + t];
+    sq = wave_sum(sq);
+    if (threadIdx.x == 0) factor = 1.0f / sqrtf(sq / n + eps);
+  }
+  __syncthreads();
+  T* row = rows + static_cast<size_t>(m) * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) store_from_float(row + i, load_as_float(row + i) * factor);
+}
+
+extern "C" int tie_scale_rows(void* rows, int dtype, int M, int width, const float* squares, int tiles, float n,
+                              float eps, hipStream_t stream) {
+  if (M <= 0 || width <= 0 || tiles <= 0 || !(n > 0.f) || squares == nullptr) return TIE_BAD_ARGUMENT;
+  if (dtype == TIE_F32) scale_rows_kernel<float><<<M, 256, 0, stream>>>(static_cast<float*>(rows), width, squares, tiles, n, eps);
+  else if (dtype == TIE_BF16) scale_rows_kernel<bf16_t><<<M, 256, 0, stream>>>(static_cast<bf16_t*>(rows), width, squares, tiles, n, eps);
+  else return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}
+
 // ------------------------------------------------------------ tokens the host has not seen
 // tokens[i] = previous[sources[i]] where sources[i] >= 0: rows whose token an earlier step's sampling kernel left
 // on the device (the host queues this step before it has read that one); the other rows keep the host's token.

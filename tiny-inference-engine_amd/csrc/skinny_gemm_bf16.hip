@@ -18,6 +18,14 @@
 //
 // Requires K % 8 == 0 (16-byte loads); other shapes go to the generic kernel.
 //
+// Two things a decode step's RMS norms would otherwise need kernels of their own for ride in the epilogue
+// (SkNorm, up to 16 rows): a product that ends a sub-layer and is not cut along K adds its sums to the residual
+// stream x in place, stores bf16(x * w) for the norm that follows (its weight w, the 1 / rms left out) and, per
+// row and 16-column tile, the sum of the squares of the new x; the products that read those rows multiply their
+// sums by 1 / sqrt(sum of the squares / n + eps), the factor that was left out (every workgroup adds the
+// tiles' squares in the same fixed order), which commutes with the product. Sums of squares, the factor and
+// the stream stay float32.
+//
 // PACKED: w is stored as [N/16][K/32] blocks of 1 KB, block (t, b) holding rows 16 t .. 16 t + 15 over
 // k = 32 b .. 32 b + 31 in the order the matrix core takes them: lane l's 16 bytes (row l % 16, k-chunk
 // l / 16) at byte 16 l. A wave's load is then 1 KB of consecutive memory and its stream through K one
@@ -53,19 +61,89 @@ __device__ __forceinline__ bf16x8_t zero_frag() {
   return *reinterpret_cast<const bf16x8_t*>(&v);
 }
 
+// What the epilogue does for the RMS norms around a product (all null / zero: nothing).
+struct SkNorm {
+  // the rows of x are norm inputs without their 1 / rms: sums are multiplied by
+  // 1 / sqrt((scale_squares[m][0] + ... + scale_squares[m][scale_tiles - 1]) / scale_n + scale_eps)
+  const float* scale_squares;
+  int scale_tiles;
+  float scale_n, scale_eps;
+  // the product ends a sub-layer: out is the residual stream (added to in place); next_x[m][n] = bf16(out * next_w[n])
+  // and squares[m][n / 16] = the sum over the tile's 16 columns of out^2 are left for the norm that follows
+  const float* next_w;
+  bf16_t* next_x;
+  float* squares;
+};
+
+#define SK_NORM_ROWS 16     // rows the epilogue's norm work takes
+#define SK_SCALE_LDS_MAX 32768   // bytes of LDS for the tiles' sums of the rows to be scaled: 16 rows of a width of 8192
+
+typedef __attribute__((address_space(3))) void sk_lds_void_t;
+// Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
+// selects x, y, z, w; no swizzle, no stride.
+#define SK_RSRC_FLAGS 0x27000
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters at their maxima).
+template <int N>
+__device__ __forceinline__ void rows_wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// The sums of squares a norm left per 16-column tile, [rows][tiles rounded up to 64]: dynamic LDS, present only in
+// launches whose sums are to be scaled (SkNorm::scale_squares).
+extern __shared__ float sk_scale_parts[];
+
 // MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 in one batch of loads.
 template <int MT, int RT, int U, typename TO, bool PACKED>
 __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
-                                                                         int accumulate, int gated, int per_wave) {
+                                                                         int accumulate, int gated, int per_wave,
+                                                                         SkNorm norm) {
   const int tile_group = blockIdx.x, split = blockIdx.y, num_splits = gridDim.y;
   __shared__ float red[SK_WAVES][MT][RT][256];
+  __shared__ float row_scale[SK_NORM_ROWS];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
+  const bool scaled = norm.scale_squares != nullptr;
+  const int scale_chunks = (norm.scale_tiles + TIE_WAVE - 1) / TIE_WAVE;   // 64 tiles an instruction
+  if (scaled) {
+    // Wave v takes rows v, v + 4, ...: the tiles' sums go from memory straight into LDS, asked for before the
+    // first weight and not waited for until the weights are through (a wait here would hold back the weights'
+    // loads for a memory latency, in a kernel that lasts a few of them). Tiles beyond the row's end are asked
+    // for beyond the buffer's end and arrive as zeros.
+    const unsigned bytes = static_cast<unsigned>(min(M, SK_NORM_ROWS)) * norm.scale_tiles * 4u;
+    const __amdgpu_buffer_rsrc_t sq_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(norm.scale_squares), 0, static_cast<int>(bytes), SK_RSRC_FLAGS);
+    for (int m = wave; m < M && m < SK_NORM_ROWS; m += SK_WAVES)
+      for (int j = 0; j < scale_chunks; ++j) {
+        const int t = j * TIE_WAVE + lane;
+        const unsigned at = t < norm.scale_tiles ? (static_cast<unsigned>(m) * norm.scale_tiles + t) * 4u : bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(sq_rsrc, (sk_lds_void_t*)(&sk_scale_parts[(m * scale_chunks + j) * TIE_WAVE]),
+                                                 4, at, 0, 0, 0);
+      }
+  }
   const int r = lane & 15;   // row of the 16-row tile (of w for B, of x for A)
   const int g = lane >> 4;   // which 8-element chunk of the 32-wide k block
   const int n0 = tile_group * 16 * RT;
+
+  // The end of a sub-layer: what the epilogue adds to and multiplies by is asked for now, for the same reason.
+  // Thread e of the workgroup ends up with row e / 16, column e % 16 of each of the RT tiles; no other thread
+  // or workgroup touches those elements of the stream.
+  float stream_now[RT], next_weight[RT];
+  if constexpr (MT == 1 && std::is_same<TO, float>::value) {
+    if (norm.next_x != nullptr) {
+      const int m = static_cast<int>(threadIdx.x) >> 4;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const int n = n0 + t * 16 + (threadIdx.x & 15);
+        const bool inside = m < M && n < N;
+        stream_now[t] = inside ? out[static_cast<size_t>(m) * N + n] : 0.f;
+        next_weight[t] = inside ? norm.next_w[n] : 0.f;
+      }
+    }
+  }
 
   // Rows beyond N are clamped for the loads; their columns are dropped at the store. wp[t] points at
   // this lane's 16 bytes of k-block 0; a k-block further on is KB_STRIDE elements further on.
@@ -154,6 +232,18 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     }
   }
 
+  if (scaled) {
+    // Each wave sums the rows it asked for: lane l adds the tiles l, l + 64, ... in ascending order, then the
+    // lanes meet in a fixed butterfly. The same sums in every workgroup of every launch, whatever the batch.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int m = wave; m < M && m < SK_NORM_ROWS; m += SK_WAVES) {
+      float sq = 0.f;
+      for (int j = 0; j < scale_chunks; ++j) sq += sk_scale_parts[(m * scale_chunks + j) * TIE_WAVE + lane];
+      sq = wave_sum(sq);
+      if (lane == 0) row_scale[m] = 1.0f / sqrtf(sq / norm.scale_n + norm.scale_eps);
+    }
+  }
+
   // D layout: lane holds rows (lane / 16) * 4 + v of x, column lane % 16 of w.
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -164,6 +254,37 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   __syncthreads();
 
   const bool partial = num_splits > 1;   // then TO is float and out holds one [M, N] plane per split
+  if (norm.next_x != nullptr) {
+    // The end of a sub-layer (MT = 1, one plane, float32 out = the residual stream): the 16 lanes that hold a
+    // row's 16 columns of a tile stay together for the sum of its squares.
+    if constexpr (std::is_same<TO, float>::value) {
+      static_assert(SK_WAVES * TIE_WAVE == 256, "one thread an element of a 16 x 16 tile");
+      const int ee = threadIdx.x;
+      const int c = ee & 15, m = ee >> 4;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const int n = n0 + t * 16 + c;
+        const bool inside = m < M && n < N;
+        float sum = red[0][0][t][ee];
+#pragma unroll
+        for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][0][t][ee];
+        float now = 0.f;
+        if (inside) {
+          if (scaled) sum *= row_scale[m];
+          now = stream_now[t] + sum;
+          out[static_cast<size_t>(m) * N + n] = now;
+          norm.next_x[static_cast<size_t>(m) * N + n] = float_to_bf16(now * next_weight[t]);
+        }
+        float sq = now * now;
+        sq += __shfl_xor(sq, 1, TIE_WAVE);
+        sq += __shfl_xor(sq, 2, TIE_WAVE);
+        sq += __shfl_xor(sq, 4, TIE_WAVE);
+        sq += __shfl_xor(sq, 8, TIE_WAVE);
+        if (c == 0 && m < M && n < N) norm.squares[static_cast<size_t>(m) * (N / 16) + n / 16] = sq;
+      }
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < 256 * RT * MT; e += SK_WAVES * TIE_WAVE) {
     const int ee = e & 255;            // 16 x 16 outputs of a tile
     const int t = (e >> 8) % RT;
@@ -176,10 +297,12 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     float sum = red[0][mt][t][ee];
 #pragma unroll
     for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][t][ee];
+    if (scaled) sum *= row_scale[m];
     if (gated) {
       float up = red[0][mt][t][ee + 8];
 #pragma unroll
       for (int wv = 1; wv < SK_WAVES; ++wv) up += red[wv][mt][t][ee + 8];
+      if (scaled) up *= row_scale[m];
       store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
       continue;
     }
@@ -212,11 +335,6 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
 // of per_wave k-blocks, each summed by the matrix core in k order, and the parts are added in their order
 // (there: by the reduction through LDS; here: by folding the accumulator into a running total at each
 // part's end). A row's result therefore does not depend on which of the two kernels its batch size picks.
-typedef __attribute__((address_space(3))) void sk_lds_void_t;
-// Fourth word of a raw buffer descriptor on gfx9-family GPUs: 32-bit float data format, destination
-// selects x, y, z, w; no swizzle, no stride.
-#define SK_RSRC_FLAGS 0x27000
-
 // The matrix instructions of one chunk: x from LDS, the weights from registers. A function of its own with
 // restrict pointers, so that the compiler knows these LDS reads from the loads into LDS that are in flight
 // (otherwise it waits for all of them before the first read).
@@ -235,13 +353,6 @@ __device__ __forceinline__ void rows_chunk(const bf16_t* __restrict__ xc, const 
       }
     }
   }
-}
-
-// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14; the other counters at their maxima).
-template <int N>
-__device__ __forceinline__ void rows_wait_loads() {
-  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
 // Calls f(integral_constant<int, I>) for I = 0 .. N - 1.
@@ -476,10 +587,19 @@ extern "C" int tie_skinny_gemm_splits(int N, int K) {
 // and receives silu(gate) * up.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 // packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
-extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out, int out_dtype, int accumulate,
-                                         int gated, int M, int N, int K, int splits, int packed, int rt, int u,
-                                         hipStream_t stream) {
+static int launch_skinny(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
+                         int N, int K, int splits, int packed, int rt, int u, const SkNorm& norm,
+                         hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1 || splits > 64) return TIE_BAD_ARGUMENT;
+  const bool norm_work = norm.scale_squares != nullptr || norm.next_x != nullptr;
+  if (norm_work && M > SK_NORM_ROWS) return TIE_BAD_ARGUMENT;
+  if (norm.scale_squares != nullptr && (norm.scale_tiles <= 0 || !(norm.scale_n > 0.f))) return TIE_BAD_ARGUMENT;
+  // the tiles' sums of the rows to be scaled wait in LDS, 64 tiles (256 bytes) a load instruction
+  const size_t scale_lds = norm.scale_squares == nullptr ? 0 : static_cast<size_t>(M) * ((norm.scale_tiles + 63) / 64) * 256;
+  if (scale_lds > SK_SCALE_LDS_MAX) return TIE_BAD_ARGUMENT;
+  if (norm.next_x != nullptr && (norm.next_w == nullptr || norm.squares == nullptr || splits != 1 || gated ||
+                                 !accumulate || out_dtype != TIE_F32 || N % 16 != 0))
+    return TIE_BAD_ARGUMENT;
   if (packed && (N % 16 != 0 || K % 32 != 0)) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || N % 16 != 0 || splits != 1)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
@@ -497,7 +617,7 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   const bool rows_fit = static_cast<size_t>(M) * K * 2 < (1ull << 31);
   const int by_rule = rows_kernel_tiles(M, N, K, gated, splits);
   const bool whole_chunks = per_wave % 4 == 0;     // the parts of K in which the sums are formed end between chunks
-  if (packed && mt > 1 && rows_kernel && rows_fit && whole_chunks && (by_rule != 0 || rows_forced)) {
+  if (!norm_work && packed && mt > 1 && rows_kernel && rows_fit && whole_chunks && (by_rule != 0 || rows_forced)) {
     const int asked = rows_forced && forced_rt != 0 ? forced_rt : (by_rule != 0 ? by_rule : 6);
     const int per_wg = asked <= 3 ? 3 : (asked <= 6 ? 6 : 8);
     const dim3 rgrid((tiles + per_wg - 1) / per_wg, splits);
@@ -526,9 +646,9 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
   if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
 #define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
-  skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, 0, stream>>>(                             \
+  skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, scale_lds, stream>>>(                     \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TO*>(out), M, N, K, accumulate, \
-      gated, per_wave)
+      gated, per_wave, norm)
 #define LAUNCH(MT, RT, U, TO)                  \
   {                                            \
     if (packed) LAUNCH_P(MT, RT, U, TO, true); \
@@ -558,7 +678,25 @@ extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out
   return tie_launch_status();
 }
 
+extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out, int out_dtype, int accumulate,
+                                         int gated, int M, int N, int K, int splits, int packed, int rt, int u,
+                                         hipStream_t stream) {
+  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, rt, u, SkNorm{}, stream);
+}
+
 extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
                                     int M, int N, int K, int splits, int packed, hipStream_t stream) {
   return tie_skinny_gemm_bf16_with(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, 0, stream);
+}
+
+// The product with the norms' work in its epilogue (up to 16 rows; see SkNorm and the top of this file).
+// scale_squares (or null): [M][scale_tiles] sums of squares of the rows x was made from; the sums are multiplied by
+// 1 / sqrt(their total / scale_n + scale_eps). next_x (or null; then accumulate, one plane, float32 out, N % 16 == 0):
+// out += sums in place, next_x = bf16(out * next_w), squares[M][N / 16] = sums of out^2 per 16-column tile.
+extern "C" int tie_skinny_gemm_bf16_norm(const void* x, const void* w, void* out, int out_dtype, int accumulate,
+                                         int gated, int M, int N, int K, int splits, int packed,
+                                         const float* scale_squares, int scale_tiles, float scale_n, float scale_eps,
+                                         const float* next_w, void* next_x, float* squares, hipStream_t stream) {
+  const SkNorm norm = {scale_squares, scale_tiles, scale_n, scale_eps, next_w, static_cast<bf16_t*>(next_x), squares};
+  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, 0, norm, stream);
 }

@@ -80,6 +80,7 @@ _SIGNATURES = {
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
+        "tie_scale_rows": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_float, _c_float, _c_void],
         "tie_take_tokens": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_random_fill": [_c_void, ctypes.c_longlong, ctypes.c_ulonglong, _c_int, ctypes.c_double, _c_void],
         "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -110,6 +111,8 @@ _SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_void],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void],
+        "tie_skinny_gemm_bf16_norm": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                      _c_int, _c_void, _c_int, _c_float, _c_float, _c_void, _c_void, _c_void, _c_void],
     },
     "gemm_bf16": {
         "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
@@ -388,6 +391,18 @@ def take_tokens(tokens: torch.Tensor, sources: torch.Tensor, previous: torch.Ten
           T, previous.numel(), _stream())
 
 
+def scale_rows(rows: torch.Tensor, row_scale: "RowScale") -> None:
+    """``rows[m] *= 1 / sqrt(row_scale.squares[m].sum() / n + eps)`` in place (bfloat16 or float32): for rows that
+    were left without their norm's factor and go to a product that cannot apply it."""
+    _gpu(rows, "rows")
+    M, n = rows.shape
+    _f32(row_scale.squares, "sums of squares")
+    if row_scale.squares.dim() != 2 or row_scale.squares.shape[0] < M or not row_scale.squares.is_contiguous():
+        raise InvalidArgument(f"sums of squares {list(row_scale.squares.shape)} do not cover {M} rows")
+    _call(_lib("elementwise").tie_scale_rows, "scale_rows", rows.data_ptr(), _code(rows, "rows"), M, n,
+          row_scale.squares.data_ptr(), row_scale.squares.shape[1], float(row_scale.n), float(row_scale.eps), _stream())
+
+
 def random_fill(out: torch.Tensor, key: int, kind: str, scale: float) -> None:
     """Fills float32 ``out`` with the random weights of the stream ``key``: element i depends on (key, i) alone
     and equals, bit for bit, what ``weights.random_init`` draws on the host. ``kind``: "normal" (``scale`` the
@@ -511,13 +526,37 @@ def skinny_splits(N: int, K: int) -> int:
     return int(_lib("skinny_gemm_bf16").tie_skinny_gemm_splits(N, K))
 
 
+NORM_EPILOGUE_ROWS = 16      # rows up to which the decode product's epilogue does the norms' work (SkNorm)
+# Whether steps of up to that many rows leave the RMS norms between their sub-layers to the products' epilogues
+# (parts.Linear.prepares_norms). False: every norm is a kernel of its own (tests compare the two ways).
+NORMS_IN_PRODUCTS = True
+
+
+class RowScale:
+    """Rows that are a norm's input times its weight, the ``1 / rms`` still to come: ``squares[m]`` holds, per
+    16-column tile of the row the norm saw, the sum of its squares; the factor is
+    ``1 / sqrt(squares[m].sum() / n + eps)`` and belongs on whatever product is formed from the rows."""
+
+    __slots__ = ("squares", "n", "eps")
+
+    def __init__(self, squares: torch.Tensor, n: int, eps: float):
+        self.squares, self.n, self.eps = squares, int(n), float(eps)
+
+
 def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-                     gated: bool = False, splits: int = 1) -> None:
+                     gated: bool = False, splits: int = 1, row_scale: Optional[RowScale] = None,
+                     next_norm: Optional[tuple] = None) -> None:
     """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores.
 
     ``gated``: w is a gate/up pair interleaved by ``interleave_gate_up`` and out receives silu(gate) * up.
     ``splits`` > 1: out is ``[splits, M, N]`` float32 and receives one plane of partial sums per range
     of K, for the consumer to add (``add_partials``, or a kernel that takes planes).
+    Up to ``NORM_EPILOGUE_ROWS`` rows the epilogue can do the work of the RMS norms around the product:
+    ``row_scale``: x lacks its norm's ``1 / rms``, and the sums are multiplied by it (before the activation of
+    a gated product); ``next_norm = (weight [N], next_x bfloat16 [M, N], squares float32 [M, N / 16])`` with
+    ``accumulate`` and one plane: out is the residual stream, and beside ``out += x @ w.T`` the epilogue leaves
+    ``next_x = bfloat16(out * weight)`` and the sums of ``out ** 2`` per 16-column tile for the norm that follows
+    (a ``RowScale`` for whoever multiplies ``next_x``).
     """
     if splits > 1:
         if out.dim() != 3 or out.shape[0] != splits or out.dtype != torch.float32 or accumulate or gated:
@@ -530,9 +569,35 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
         raise InvalidArgument(f"skinny_gemm_bf16 takes at most 64 rows, got {M}")
     if gated and accumulate:
         raise InvalidArgument("a gated product does not accumulate")
-    _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16, "skinny_gemm_bf16",
+    if row_scale is None and next_norm is None:
+        _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16, "skinny_gemm_bf16",
+            x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
+            int(splits), int(isinstance(w, PackedWeight)), _stream())
+        return
+    if M > NORM_EPILOGUE_ROWS:
+        raise InvalidArgument(f"the product's epilogue does the norms' work for up to {NORM_EPILOGUE_ROWS} rows, not {M}")
+    squares_in, tiles_in, n_in, eps_in = None, 0, 1.0, 0.0
+    if row_scale is not None:
+        _f32(row_scale.squares, "sums of squares")
+        if row_scale.squares.dim() != 2 or row_scale.squares.shape[0] < M or not row_scale.squares.is_contiguous() \
+                or row_scale.n <= 0:
+            raise InvalidArgument(f"sums of squares {list(row_scale.squares.shape)} do not cover {M} rows")
+        squares_in, tiles_in, n_in, eps_in = row_scale.squares, row_scale.squares.shape[1], float(row_scale.n), row_scale.eps
+    next_w = next_x = squares_out = None
+    if next_norm is not None:
+        next_w, next_x, squares_out = next_norm
+        _f32(next_w, "the next norm's weight", (N,))
+        _f32(squares_out, "sums of squares", (M, N // 16))
+        _gpu(next_x, "the next norm's rows")
+        if splits != 1 or gated or not accumulate or out.dtype != torch.float32 or N % 16 or \
+                next_x.dtype != torch.bfloat16 or tuple(next_x.shape) != (M, N) or not next_x.is_contiguous() or \
+                not squares_out.is_contiguous():
+            raise InvalidArgument("a product that prepares the next norm adds to a float32 stream in one plane, is not "
+                                  f"gated, and leaves bfloat16 rows [{M}, {N}] (N in steps of 16)")
+    _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16_norm, "skinny_gemm_bf16_norm",
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
-        int(splits), int(isinstance(w, PackedWeight)), _stream())
+        int(splits), int(isinstance(w, PackedWeight)), _ptr(squares_in), tiles_in, n_in, eps_in, _ptr(next_w),
+        _ptr(next_x), _ptr(squares_out), _stream())
 
 
 def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
@@ -599,20 +664,36 @@ def decode_product_rows(M: int, w, gated: bool = False) -> bool:
     return not tiled
 
 
-def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tensor) -> None:
-    """out = silu(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only."""
+def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tensor,
+                  row_scale: Optional[RowScale] = None) -> None:
+    """out = silu(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only.
+    ``row_scale`` as in ``skinny_gemm_bf16`` (up to ``NORM_EPILOGUE_ROWS`` rows)."""
     if decode_product_rows(x.shape[0], w_interleaved, gated=True):
-        skinny_gemm_bf16(x, w_interleaved, out, gated=True)
+        skinny_gemm_bf16(x, w_interleaved, out, gated=True, row_scale=row_scale)
+    elif row_scale is not None:
+        raise InvalidArgument(f"{x.shape[0]} rows without their norm's factor: only the decode product applies it")
     else:
         gemm_bf16(x, w_interleaved, out, gated=True)
 
 
-def linear(x: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out (+)= x @ w.T, on the fastest kernel that takes these operands (w a matrix or a ``PackedWeight``)."""
+def applies_row_scale(x: torch.Tensor, w) -> bool:
+    """Whether ``linear`` / ``linear_swiglu`` over these operands run on the product whose epilogue applies a
+    ``RowScale`` (the decode product, up to ``NORM_EPILOGUE_ROWS`` rows)."""
+    # the kernel holds the tiles' sums of squares of all rows in 32 KB of LDS, 64 tiles (256 bytes) a load
+    staged = x.shape[0] * (-(-(x.shape[1] // 16) // 64)) * 256
+    return x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 16 == 0 and \
+        x.shape[0] <= NORM_EPILOGUE_ROWS and staged <= 32768
+
+
+def linear(x: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False, row_scale: Optional[RowScale] = None) -> None:
+    """out (+)= x @ w.T, on the fastest kernel that takes these operands (w a matrix or a ``PackedWeight``).
+    ``row_scale``: see ``skinny_gemm_bf16``; only where ``applies_row_scale`` says so."""
+    if row_scale is not None and not (applies_row_scale(x, w) and not (accumulate and out.dtype != torch.float32)):
+        raise InvalidArgument("these operands do not run on the product that applies a row scale: scale the rows first")
     if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and \
             not (accumulate and out.dtype != torch.float32):
         if decode_product_rows(x.shape[0], w):
-            skinny_gemm_bf16(x, w, out, accumulate)
+            skinny_gemm_bf16(x, w, out, accumulate, row_scale=row_scale)
         else:
             gemm_bf16(x, w, out, accumulate)
     elif isinstance(w, PackedWeight):

@@ -306,8 +306,13 @@ class Model:
         batch = ctx.batch
         x = self.embedding.forward(ctx, batch.tokens)
         index, entries = 0, len(self.spec.order)
+        # Layers run from another's launch list only where a layer's launches are its own: in steps of a few rows a
+        # sub-layer's last product may stay pending in the step context for the next layer's norm to launch, and a
+        # replayed launch list would not carry that over.
+        replay = self.replay_layers and self.layer_hook is None and not (
+            kernels.NORMS_IN_PRODUCTS and batch.num_tokens <= kernels.NORM_EPILOGUE_ROWS)
         while index < entries:
-            alike_to = self._alike.get(index) if self.replay_layers and self.layer_hook is None else None
+            alike_to = self._alike.get(index) if replay else None
             if alike_to is not None:
                 self._run_alike(ctx, x, index, alike_to)
                 index = alike_to

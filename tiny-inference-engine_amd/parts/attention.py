@@ -30,6 +30,7 @@ from .linear import Linear
 class PagedAttention(Mixer):
     capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
+    takes_row_scale = True   # h goes into the QKV projection only, through Linear with the step context
 
     def __init__(self, params):
         super().__init__(params)
@@ -87,7 +88,7 @@ class PagedAttention(Mixer):
             qkv = planes[0]
         else:
             qkv = ctx.scratch("attention.qkv", (T, width), torch.float32)
-            self.qkv(h, qkv)
+            self.qkv(h, qkv, ctx=ctx)
         if table is not None:
             inv_freq, rotary_dim, pairing = table
             if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half"

@@ -18,7 +18,10 @@ a matrix product's input) has the activation dtype of the mode. Mixers and
 feed-forwards ADD their result to the ``residual`` tensor they are given, which
 lets the last matrix product of a part fold the addition into its epilogue, or
 leave it owed to the stream (``StepContext.defer_add``) for the next norm to add
-in the pass in which it reads the stream anyway.
+in the pass in which it reads the stream anyway - or, in steps of a few rows,
+leave the whole product owed (``StepContext.defer_product``): the norm that
+follows then has the product's own epilogue add to the stream and prepare the
+norm's output (``Norm.forward(..., lazy=True)``), and no norm kernel runs.
 """
 
 from __future__ import annotations
@@ -175,6 +178,8 @@ class StepContext:
         self.act_dtype = torch.float32 if mode == FLOAT32 else torch.bfloat16
         self.notes: Dict[Any, Any] = {}   # per-step memo shared by parts (e.g. one plan for all layers)
         self._owed = None                  # (target, planes): target += planes[0] + planes[1] + ... is still to be done
+        self._pending = None               # (target, linear, x): target += x @ linear.weight^T is still to be launched
+        self._row_scales: Dict[int, Any] = {}   # address of rows that lack their norm's 1 / rms -> kernels.RowScale
 
     @property
     def num_tokens(self) -> int:
@@ -189,8 +194,43 @@ class StepContext:
         self.settle()
         self._owed = (target, planes)
 
+    # A product that ends a sub-layer in a step of a few rows is not even launched by its part: the norm that
+    # reads the stream next launches it with an epilogue that adds to the stream and prepares that norm's rows
+    # (take_pending_product), or settle() launches it the ordinary way.
+    def defer_product(self, target: torch.Tensor, linear, x: torch.Tensor) -> None:
+        self.settle()
+        self._pending = (target, linear, x)
+
+    def take_pending_product(self, target: torch.Tensor):
+        """``(linear, x)`` of the product still to be added to ``target`` (the caller launches it now), or None."""
+        if self._pending is None:
+            return None
+        owed_to, linear, x = self._pending
+        if owed_to.data_ptr() == target.data_ptr() and owed_to.shape == target.shape:
+            self._pending = None
+            return linear, x
+        return None
+
+    def launch_pending(self) -> None:
+        """Launches a product left pending the ordinary way (it may leave planes of partial sums owed in turn)."""
+        if self._pending is not None:
+            target, linear, x = self._pending
+            self._pending = None
+            linear.add_to(self, x, target)
+
+    # Rows that a norm left without their 1 / rms (kernels.RowScale): the products formed from them apply it.
+    def set_row_scale(self, rows: torch.Tensor, scale) -> None:
+        if scale is None:
+            self._row_scales.pop(rows.data_ptr(), None)
+        else:
+            self._row_scales[rows.data_ptr()] = scale
+
+    def row_scale_of(self, rows: torch.Tensor):
+        return self._row_scales.get(rows.data_ptr()) if self._row_scales else None
+
     def take_owed(self, target: torch.Tensor) -> Optional[torch.Tensor]:
         """The planes still owed to ``target`` (the caller now adds them itself), or None; other debts are settled."""
+        self.launch_pending()
         if self._owed is None:
             return None
         owed_to, planes = self._owed
@@ -201,6 +241,7 @@ class StepContext:
         return None
 
     def settle(self) -> None:
+        self.launch_pending()
         if self._owed is not None:
             from .. import kernels
             target, planes = self._owed
@@ -247,6 +288,9 @@ class StateBinding:
 
 class Norm(Part):
     adds_owed = False   # True: forward() adds partial sums owed to x (ctx.take_owed) in its own pass
+    # True: forward() takes ``lazy=True`` and may then return rows without their 1 / rms, registered with
+    # ``ctx.set_row_scale``: only for a consumer that applies it (``takes_row_scale``; see ``Block.normed``).
+    leaves_row_scale = False
 
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
                 out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
@@ -297,13 +341,18 @@ class Block(Part):
     """The arrangement of one layer's parts. ``layer`` carries .mixer, .feed_forward and .norms.
 
     An arrangement settles what is owed to the residual stream before it hands the stream to a part
-    that does not add the debt itself (``normed`` does so for norms).
+    that does not add the debt itself (``normed`` does so for norms). ``consumer``: the part the normed rows
+    go to and to nothing else; if it says ``takes_row_scale`` (every product it forms from the rows goes through
+    ``parts.Linear`` with the step context, or asks ``ctx.row_scale_of`` itself), a norm that can may hand it the
+    rows without their 1 / rms.
     """
 
     @staticmethod
-    def normed(ctx: StepContext, norm, x: torch.Tensor) -> torch.Tensor:
+    def normed(ctx: StepContext, norm, x: torch.Tensor, consumer=None) -> torch.Tensor:
         if not norm.adds_owed:
             ctx.settle()
+        if getattr(norm, "leaves_row_scale", False) and getattr(consumer, "takes_row_scale", False):
+            return norm.forward(ctx, x, lazy=True)
         return norm.forward(ctx, x)
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:

@@ -21,9 +21,9 @@ class PreNormBlock(Block):
     NORMS = ("pre_mixer", "pre_feed_forward")
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
-        h = self.normed(ctx, layer.norms["pre_mixer"], x)
+        h = self.normed(ctx, layer.norms["pre_mixer"], x, consumer=layer.mixer)
         layer.mixer.forward(ctx, h, cache, x)
-        h = self.normed(ctx, layer.norms["pre_feed_forward"], x)
+        h = self.normed(ctx, layer.norms["pre_feed_forward"], x, consumer=layer.feed_forward)
         layer.feed_forward.forward(ctx, h, x)
 
     @classmethod

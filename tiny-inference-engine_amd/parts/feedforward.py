@@ -23,6 +23,7 @@ from .linear import Linear
 class SwiGLU(FeedForward):
     capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
+    takes_row_scale = True   # h goes into the gate/up product only
 
     def __init__(self, params):
         super().__init__(params)
@@ -51,9 +52,9 @@ class SwiGLU(FeedForward):
         T = h.shape[0]
         act = ctx.scratch("swiglu.act", (T, self.intermediate))
         if self.fused and h.dtype == torch.bfloat16:
-            kernels.linear_swiglu(h, self.gate_up.weight, act)
+            kernels.linear_swiglu(h, self.gate_up.weight, act, row_scale=Linear.row_scale_for(ctx, h, self.gate_up.weight))
         else:
             gate_up = ctx.scratch("swiglu.gate_up", (T, 2 * self.intermediate))
-            self.gate_up(h, gate_up)
+            self.gate_up(h, gate_up, ctx=ctx)
             kernels.swiglu(gate_up, act)
         self.down(act, residual, accumulate=True, ctx=ctx)

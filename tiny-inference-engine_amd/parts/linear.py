@@ -55,20 +55,55 @@ class Linear:
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ctx=None) -> torch.Tensor:
         """out (+)= x @ W^T. With ``ctx`` an accumulating product may leave its addition owed to ``out``.
 
-        A decode-size product over a weight of few rows is cut along K into planes of partial sums;
-        the step context remembers that their sum is still to be added, and the next norm over
-        ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once.
+        In a step of a few rows the whole product is left pending: the norm that reads ``out`` next launches it
+        with the norm's work in its epilogue (``add_to_and_prepare_norm``), or ``ctx.settle()`` launches it the
+        ordinary way. Otherwise a decode-size product over a weight of few rows is cut along K into planes of
+        partial sums; the step context remembers that their sum is still to be added, and the next norm over
+        ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once. With
+        ``ctx``, rows ``x`` that lack their norm's 1 / rms (``ctx.row_scale_of``) have it applied to the sums.
         """
         if ctx is not None and accumulate and out.dtype == torch.float32:
-            # An earlier product's planes may still be owed and live in the buffer the new planes take:
-            # add them before they are overwritten (after a norm that took the debt this does nothing).
-            ctx.settle()
-            planes = self.partial_planes(ctx, x, "linear.partials")
-            if planes is not None:
-                ctx.defer_add(out, planes)
+            if self.prepares_norms(x):
+                ctx.defer_product(out, self, x)
                 return out
-        kernels.linear(x, self.weight, out, accumulate)
+            return self.add_to(ctx, x, out)
+        kernels.linear(x, self.weight, out, accumulate, row_scale=self.row_scale_for(ctx, x, self.weight))
         return out
+
+    def prepares_norms(self, x: torch.Tensor) -> bool:
+        """Whether the decode product takes this product with the next norm's work in its epilogue."""
+        w = self.weight
+        return kernels.NORMS_IN_PRODUCTS and x.dtype == torch.bfloat16 and isinstance(w, kernels.PackedWeight) and \
+            x.shape[0] <= kernels.NORM_EPILOGUE_ROWS and x.is_cuda
+
+    def add_to(self, ctx, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out += x @ W^T now, or as planes of partial sums owed to ``out``."""
+        # An earlier product's planes may still be owed and live in the buffer the new planes take:
+        # add them before they are overwritten (after a norm that took the debt this does nothing).
+        ctx.settle()
+        planes = self.partial_planes(ctx, x, "linear.partials")
+        if planes is not None:
+            ctx.defer_add(out, planes)
+            return out
+        kernels.linear(x, self.weight, out, True, row_scale=self.row_scale_for(ctx, x, self.weight))
+        return out
+
+    def add_to_and_prepare_norm(self, x: torch.Tensor, out: torch.Tensor, norm_weight: torch.Tensor,
+                                next_rows: torch.Tensor, squares: torch.Tensor) -> None:
+        """out += x @ W^T in one plane, and in the same epilogue ``next_rows = bfloat16(out * norm_weight)`` and the
+        sums of ``out ** 2`` per 16-column tile (``prepares_norms`` says whether this product can)."""
+        kernels.skinny_gemm_bf16(x, self.weight, out, accumulate=True, next_norm=(norm_weight, next_rows, squares))
+
+    @staticmethod
+    def row_scale_for(ctx, x: torch.Tensor, weight):
+        """The factor that rows ``x`` still lack, if the product about to run can apply it; otherwise it is applied
+        to the rows themselves first."""
+        scale = ctx.row_scale_of(x) if ctx is not None else None
+        if scale is not None and not kernels.applies_row_scale(x, weight):
+            kernels.scale_rows(x, scale)
+            ctx.set_row_scale(x, None)
+            return None
+        return scale
 
     def partial_planes(self, ctx, x: torch.Tensor, name: str):
         """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None.
@@ -92,8 +127,9 @@ class Linear:
         if splits <= 1:
             return None
         planes = ctx.scratch(name, (splits, M, w.shape[0]), torch.float32)
+        scale = self.row_scale_for(ctx, x, w)
         if decode_product:
-            kernels.skinny_gemm_bf16(x, w, planes, splits=splits)
+            kernels.skinny_gemm_bf16(x, w, planes, splits=splits, row_scale=scale)
         else:
-            kernels.gemm_bf16(x, w, planes, splits=splits)
+            kernels.gemm_bf16(x, w, planes, splits=splits)      # above the rows a scale travels with: none here
         return planes

@@ -21,6 +21,7 @@ class RMSNorm(Norm):
     capturable = True      # reads the step on the device only: may be recorded into a HIP graph
     replayable = True
     adds_owed = True
+    leaves_row_scale = True
 
     def __init__(self, params):
         super().__init__(params)
@@ -36,9 +37,22 @@ class RMSNorm(Norm):
         self.weight = fetch(self.weight_name, "vector")
 
     def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
-                out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
+                out_name: str = "norm.out", out_dtype: torch.dtype = None, lazy: bool = False) -> torch.Tensor:
+        """``lazy``: the caller's consumer applies a row scale (``Block.normed``). If the product that ends the
+        sub-layer before is still pending, it is launched here with an epilogue that adds it to ``x`` and leaves
+        ``x * weight`` and the rows' sums of squares: the result lacks its ``1 / rms``, which the consumer's
+        products apply (``ctx.row_scale_of``), and no norm kernel runs."""
         count = x.shape[0] if rows is None else rows.numel()
         out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
+        if lazy and rows is None and out.dtype == torch.bfloat16 and self.dim % 16 == 0:
+            pending = ctx.take_pending_product(x)
+            if pending is not None:
+                linear, rows_in = pending
+                squares = ctx.scratch(out_name + ".squares", (count, self.dim // 16), torch.float32)
+                linear.add_to_and_prepare_norm(rows_in, x, self.weight, out, squares)
+                ctx.set_row_scale(out, kernels.RowScale(squares, self.dim, self.eps))
+                return out
+        ctx.set_row_scale(out, None)
         owed = ctx.take_owed(x)
         if owed is not None and rows is None:
             kernels.add_partials(x, owed, self.weight, self.eps, out)   # x += owed sums; out = norm(x), one pass
