@@ -1143,15 +1143,21 @@ def test_decode_product_with_the_norms_work_in_its_epilogue(M, N, K, packed):
     norm_w = (1 + 0.1 * rnd(N, seed=44)).cuda()
     plainly = stream.clone()
     kernels.skinny_gemm_bf16(x, weight, plainly, accumulate=True)
-    got = stream.clone()
-    rows = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
-    squares = torch.full((M, N // 16), float("nan"), device="cuda")
-    kernels.skinny_gemm_bf16(x, weight, got, accumulate=True, next_norm=(norm_w, rows, squares))
-    assert torch.equal(got, plainly), "the stream differs from the product without the norm's work"
     want = stream.cpu().to(F64) + plain.linear(x.cpu(), w.cpu())
-    close(got, want, 1e-5, "stream")
-    assert torch.equal(rows, (got * norm_w).to(torch.bfloat16)), "rows for the next norm"
-    close(squares, (got.cpu().to(F64) ** 2).view(M, N // 16, 16).sum(-1), 1e-6, "sums of squares")
+    # waves a workgroup and k-blocks a batch of loads: four waves (the sums of the product without the epilogue's
+    # work, bit for bit), and the wider workgroups that packed weights get where the output is narrow; last, the rule
+    for waves, loads in ([(4, 0), (8, 8), (8, 4), (16, 4), (16, 2), (0, 0)] if packed else [(4, 0), (0, 0)]):
+        got = stream.clone()
+        rows = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        squares = torch.full((M, N // 16), float("nan"), device="cuda")
+        kernels.skinny_gemm_bf16(x, weight, got, accumulate=True, next_norm=(norm_w, rows, squares), waves=waves, loads=loads)
+        if waves == 4:
+            assert torch.equal(got, plainly), "the stream differs from the product without the norm's work"
+        close(got, want, 1e-5, f"stream, {waves} waves")
+        assert torch.equal(rows, (got * norm_w).to(torch.bfloat16)), f"rows for the next norm, {waves} waves"
+        close(squares, (got.cpu().to(F64) ** 2).view(M, N // 16, 16).sum(-1), 1e-6, f"sums of squares, {waves} waves")
+    with pytest.raises(kernels.InvalidArgument):
+        kernels.skinny_gemm_bf16(x, weight, got.clone(), accumulate=True, next_norm=(norm_w, rows, squares), waves=5)
 
     # the consumers: x2 = rows (no 1 / rms yet) against a second weight
     eps = 1e-5

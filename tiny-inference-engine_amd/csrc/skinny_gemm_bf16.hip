@@ -95,14 +95,14 @@ __device__ __forceinline__ void rows_wait_loads() {
 extern __shared__ float sk_scale_parts[];
 
 // MT: 16-row tiles of x; RT: 16-row tiles of w per workgroup; U: k-blocks of 32 in one batch of loads.
-template <int MT, int RT, int U, typename TO, bool PACKED>
-__global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
+template <int MT, int RT, int U, typename TO, bool PACKED, int WAVES = SK_WAVES>
+__global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ w,
                                                                          TO* __restrict__ out, int M, int N, int K,
                                                                          int accumulate, int gated, int per_wave,
                                                                          SkNorm norm) {
   const int tile_group = blockIdx.x, split = blockIdx.y, num_splits = gridDim.y;
-  __shared__ float red[SK_WAVES][MT][RT][256];
+  __shared__ float red[WAVES][MT][RT][256];
   __shared__ float row_scale[SK_NORM_ROWS];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     const unsigned bytes = static_cast<unsigned>(min(M, SK_NORM_ROWS)) * norm.scale_tiles * 4u;
     const __amdgpu_buffer_rsrc_t sq_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(norm.scale_squares), 0, static_cast<int>(bytes), SK_RSRC_FLAGS);
-    for (int m = wave; m < M && m < SK_NORM_ROWS; m += SK_WAVES)
+    for (int m = wave; m < M && m < SK_NORM_ROWS; m += WAVES)
       for (int j = 0; j < scale_chunks; ++j) {
         const int t = j * TIE_WAVE + lane;
         const unsigned at = t < norm.scale_tiles ? (static_cast<unsigned>(m) * norm.scale_tiles + t) * 4u : bytes;
@@ -129,18 +129,19 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
   const int n0 = tile_group * 16 * RT;
 
   // The end of a sub-layer: what the epilogue adds to and multiplies by is asked for now, for the same reason.
-  // Thread e of the workgroup ends up with row e / 16, column e % 16 of each of the RT tiles; no other thread
-  // or workgroup touches those elements of the stream.
-  float stream_now[RT], next_weight[RT];
+  // Thread e of the workgroup ends up with row e / 16 % 16, column e % 16 of tile e / 256 (and of the tiles a
+  // workgroup's worth of threads further on); no other thread or workgroup touches those elements of the stream.
+  constexpr int ENDS = (256 * RT + WAVES * TIE_WAVE - 1) / (WAVES * TIE_WAVE);   // elements a thread ends up with
+  float stream_now[ENDS], next_weight[ENDS];
   if constexpr (MT == 1 && std::is_same<TO, float>::value) {
     if (norm.next_x != nullptr) {
-      const int m = static_cast<int>(threadIdx.x) >> 4;
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const int n = n0 + t * 16 + (threadIdx.x & 15);
-        const bool inside = m < M && n < N;
-        stream_now[t] = inside ? out[static_cast<size_t>(m) * N + n] : 0.f;
-        next_weight[t] = inside ? norm.next_w[n] : 0.f;
+      for (int i = 0; i < ENDS; ++i) {
+        const int e = threadIdx.x + i * WAVES * TIE_WAVE;
+        const int m = (e & 255) >> 4, n = n0 + (e >> 8) * 16 + (e & 15);
+        const bool inside = e < 256 * RT && m < M && n < N;
+        stream_now[i] = inside ? out[static_cast<size_t>(m) * N + n] : 0.f;
+        next_weight[i] = inside ? norm.next_w[n] : 0.f;
       }
     }
   }
@@ -163,9 +164,9 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     xp[mt] = x + static_cast<size_t>(xvalid[mt] ? m : 0) * K;
   }
 
-  // This wave's k range, in blocks of 32: part (split, wave) of gridDim.y * SK_WAVES equal parts.
+  // This wave's k range, in blocks of 32: part (split, wave) of gridDim.y * WAVES equal parts.
   const int kblocks = (K + 31) / 32;
-  const int kb_begin = min(kblocks, (split * SK_WAVES + wave) * per_wave);
+  const int kb_begin = min(kblocks, (split * WAVES + wave) * per_wave);
   const int kb_end = min(kblocks, kb_begin + per_wave);
 
   floatx4 acc[MT][RT];
@@ -236,7 +237,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     // Each wave sums the rows it asked for: lane l adds the tiles l, l + 64, ... in ascending order, then the
     // lanes meet in a fixed butterfly. The same sums in every workgroup of every launch, whatever the batch.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    for (int m = wave; m < M && m < SK_NORM_ROWS; m += SK_WAVES) {
+    for (int m = wave; m < M && m < SK_NORM_ROWS; m += WAVES) {
       float sq = 0.f;
       for (int j = 0; j < scale_chunks; ++j) sq += sk_scale_parts[(m * scale_chunks + j) * TIE_WAVE + lane];
       sq = wave_sum(sq);
@@ -258,22 +259,23 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     // The end of a sub-layer (MT = 1, one plane, float32 out = the residual stream): the 16 lanes that hold a
     // row's 16 columns of a tile stay together for the sum of its squares.
     if constexpr (std::is_same<TO, float>::value) {
-      static_assert(SK_WAVES * TIE_WAVE == 256, "one thread an element of a 16 x 16 tile");
-      const int ee = threadIdx.x;
-      const int c = ee & 15, m = ee >> 4;
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
+      for (int i = 0; i < ENDS; ++i) {
+        const int e = threadIdx.x + i * WAVES * TIE_WAVE;
+        if (e >= 256 * RT) break;            // whole waves at a time: 256 RT is a multiple of the wave
+        const int ee = e & 255, t = e >> 8;
+        const int c = ee & 15, m = ee >> 4;
         const int n = n0 + t * 16 + c;
         const bool inside = m < M && n < N;
         float sum = red[0][0][t][ee];
 #pragma unroll
-        for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][0][t][ee];
+        for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][0][t][ee];
         float now = 0.f;
         if (inside) {
           if (scaled) sum *= row_scale[m];
-          now = stream_now[t] + sum;
+          now = stream_now[i] + sum;
           out[static_cast<size_t>(m) * N + n] = now;
-          norm.next_x[static_cast<size_t>(m) * N + n] = float_to_bf16(now * next_weight[t]);
+          norm.next_x[static_cast<size_t>(m) * N + n] = float_to_bf16(now * next_weight[i]);
         }
         float sq = now * now;
         sq += __shfl_xor(sq, 1, TIE_WAVE);
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     }
     return;
   }
-  for (int e = threadIdx.x; e < 256 * RT * MT; e += SK_WAVES * TIE_WAVE) {
+  for (int e = threadIdx.x; e < 256 * RT * MT; e += WAVES * TIE_WAVE) {
     const int ee = e & 255;            // 16 x 16 outputs of a tile
     const int t = (e >> 8) % RT;
     const int mt = e / (256 * RT);
@@ -296,12 +298,12 @@ __global__ __launch_bounds__(SK_WAVES* TIE_WAVE) void skinny_gemm_kernel(const b
     if (gated && c >= 8) continue;       // gated: columns 0..7 are gates, 8..15 the ups of the same outputs
     float sum = red[0][mt][t][ee];
 #pragma unroll
-    for (int wv = 1; wv < SK_WAVES; ++wv) sum += red[wv][mt][t][ee];
+    for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][mt][t][ee];
     if (scaled) sum *= row_scale[m];
     if (gated) {
       float up = red[0][mt][t][ee + 8];
 #pragma unroll
-      for (int wv = 1; wv < SK_WAVES; ++wv) up += red[wv][mt][t][ee + 8];
+      for (int wv = 1; wv < WAVES; ++wv) up += red[wv][mt][t][ee + 8];
       if (scaled) up *= row_scale[m];
       store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
       continue;
@@ -587,8 +589,14 @@ extern "C" int tie_skinny_gemm_splits(int N, int K) {
 // and receives silu(gate) * up.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 // packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
+// Waves a workgroup of a product that ends a sub-layer (see launch_skinny): sixteen where the output's tiles
+// leave every compute unit at most one workgroup. Measured in a chain of a layer's four products, 4096 wide:
+// 71.8 -> 67.8 us a layer at 1 row, 76.4 -> 75.0 at 8; with 320 tiles (5120 wide, where four waves take
+// several tiles a workgroup and read x less often) sixteen waves lose, 180 -> 193 us at 8 rows.
+static int producer_waves(int N) { return (N + 15) / 16 <= compute_units() ? 16 : SK_WAVES; }
+
 static int launch_skinny(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
-                         int N, int K, int splits, int packed, int rt, int u, const SkNorm& norm,
+                         int N, int K, int splits, int packed, int rt, int u, int waves, const SkNorm& norm,
                          hipStream_t stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || splits < 1 || splits > 64) return TIE_BAD_ARGUMENT;
   const bool norm_work = norm.scale_squares != nullptr || norm.next_x != nullptr;
@@ -610,7 +618,12 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
   if (u < 0) u = u == -1 ? 0 : -u;
   if (u == 1) u = 0;
   const int kblocks = (K + 31) / 32;
-  const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
+  // A product that ends a sub-layer is not cut along K, so a narrow output leaves it one workgroup a compute
+  // unit: more waves a workgroup then keep as many bytes in flight as the planes of a cut product would.
+  const bool many_waves_fit = norm.next_x != nullptr && packed && rt <= 1 && u >= 0;
+  if (waves == 0) waves = many_waves_fit ? producer_waves(N) : SK_WAVES;
+  if (waves != SK_WAVES && !(many_waves_fit && (waves == 8 || waves == 16))) return TIE_BAD_ARGUMENT;
+  const int per_wave = (kblocks + splits * waves - 1) / (splits * waves);
   // x through LDS (17 to 64 rows over packed weights, x within 32-bit byte offsets). With u = 1, rt is the
   // number of tiles a workgroup takes: up to 3 three waves x one tile, up to 6 three waves x two, else four x two.
   const int tiles = (N + 15) / 16;
@@ -637,6 +650,21 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
 #undef LAUNCH_ROWS_MT
 #undef LAUNCH_ROWS_TO
 #undef LAUNCH_ROWS
+    return tie_launch_status();
+  }
+  if (waves != SK_WAVES) {
+    const dim3 wgrid((N + 15) / 16, 1);
+    if (u == 0) u = waves == 8 ? 8 : 4;
+#define LAUNCH_W(U, W)                                                                                         \
+  skinny_gemm_kernel<1, 1, U, float, true, W><<<wgrid, W * TIE_WAVE, scale_lds, stream>>>(                      \
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<float*>(out), M, N, K, accumulate, \
+      gated, per_wave, norm)
+    if (waves == 8 && u == 8) LAUNCH_W(8, 8);
+    else if (waves == 8 && u == 4) LAUNCH_W(4, 8);
+    else if (waves == 16 && u == 4) LAUNCH_W(4, 16);
+    else if (waves == 16 && u == 2) LAUNCH_W(2, 16);
+    else return TIE_BAD_ARGUMENT;
+#undef LAUNCH_W
     return tie_launch_status();
   }
   if (rows_forced) rt = 0;                  // asked for the other kernel, which does not take this shape: by the rule
@@ -681,7 +709,7 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
 extern "C" int tie_skinny_gemm_bf16_with(const void* x, const void* w, void* out, int out_dtype, int accumulate,
                                          int gated, int M, int N, int K, int splits, int packed, int rt, int u,
                                          hipStream_t stream) {
-  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, rt, u, SkNorm{}, stream);
+  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, rt, u, SK_WAVES, SkNorm{}, stream);
 }
 
 extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated,
@@ -693,10 +721,12 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
 // scale_squares (or null): [M][scale_tiles] sums of squares of the rows x was made from; the sums are multiplied by
 // 1 / sqrt(their total / scale_n + scale_eps). next_x (or null; then accumulate, one plane, float32 out, N % 16 == 0):
 // out += sums in place, next_x = bf16(out * next_w), squares[M][N / 16] = sums of out^2 per 16-column tile.
+// u, waves: 0 = by the rule (measurements name k-blocks a batch of loads and waves a workgroup themselves).
 extern "C" int tie_skinny_gemm_bf16_norm(const void* x, const void* w, void* out, int out_dtype, int accumulate,
                                          int gated, int M, int N, int K, int splits, int packed,
                                          const float* scale_squares, int scale_tiles, float scale_n, float scale_eps,
-                                         const float* next_w, void* next_x, float* squares, hipStream_t stream) {
+                                         const float* next_w, void* next_x, float* squares, int u, int waves,
+                                         hipStream_t stream) {
   const SkNorm norm = {scale_squares, scale_tiles, scale_n, scale_eps, next_w, static_cast<bf16_t*>(next_x), squares};
-  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, 0, norm, stream);
+  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, u, waves, norm, stream);
 }

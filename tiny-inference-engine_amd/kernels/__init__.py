@@ -112,7 +112,8 @@ _SIGNATURES = {
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void],
         "tie_skinny_gemm_bf16_norm": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                      _c_int, _c_void, _c_int, _c_float, _c_float, _c_void, _c_void, _c_void, _c_void],
+                                      _c_int, _c_void, _c_int, _c_float, _c_float, _c_void, _c_void, _c_void, _c_int,
+                                      _c_int, _c_void],
     },
     "gemm_bf16": {
         "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
@@ -545,7 +546,7 @@ class RowScale:
 
 def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
                      gated: bool = False, splits: int = 1, row_scale: Optional[RowScale] = None,
-                     next_norm: Optional[tuple] = None) -> None:
+                     next_norm: Optional[tuple] = None, loads: int = 0, waves: int = 0) -> None:
     """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores.
 
     ``gated``: w is a gate/up pair interleaved by ``interleave_gate_up`` and out receives silu(gate) * up.
@@ -597,7 +598,7 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
     _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16_norm, "skinny_gemm_bf16_norm",
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
         int(splits), int(isinstance(w, PackedWeight)), _ptr(squares_in), tiles_in, n_in, eps_in, _ptr(next_w),
-        _ptr(next_x), _ptr(squares_out), _stream())
+        _ptr(next_x), _ptr(squares_out), int(loads), int(waves), _stream())
 
 
 def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
