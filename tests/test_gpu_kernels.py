@@ -426,7 +426,7 @@ def test_gemm_bf16(M, N, K, tile):
 
 @pytest.mark.parametrize("M,N,K", [(65, 72, 96), (100, 384, 224), (300, 200, 4096), (2048, 256, 512), (257, 132, 1024),
                                    (513, 516, 352), (1, 64, 128)])
-@pytest.mark.parametrize("tile", [4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("tile", [4, 5, 6, 7, 8, 9, 10])
 def test_gemm_bf16_loaded_straight_into_lds(M, N, K, tile):
     """The tiles whose operand slices bypass registers: ragged M and N, short and long K, every epilogue."""
     from tie_amd import kernels
@@ -491,7 +491,7 @@ def test_packed_weight_feeds_both_products_the_same_numbers(N, K):
     for M in (40, 64, 65, 128, 300, 513):
         x = rnd(M, K, seed=60 + M, dtype=torch.bfloat16).cuda()
         want = plain.linear(x.cpu(), w.cpu())
-        for tile in (4, 5, 6, 7, 8, 9):
+        for tile in (4, 5, 6, 7, 8, 9, 10):
             a = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
             b_ = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
             kernels.gemm_bf16(x, w, a, tile=tile)

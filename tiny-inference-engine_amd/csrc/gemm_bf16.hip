@@ -631,10 +631,12 @@ static int legacy_splits(int M, int N, int K) {
 
 struct DmaTile { int id, bm, bn; float start_us, full_us, slice_us; int per_cu; };
 // start_us: a round's start and end; full_us: what a round costs more when it fills every compute unit (measured
-// for the 256 x 256 tile only, whatever the length of K: 256 workgroups of it start about 11 us later than 192);
+// for the 256 x 256 and 256 x 192 tiles, whatever the length of K: 256 workgroups of the first start about 11 us
+// later than 192);
 // slice_us: one slice of 32 along K with the compute unit to itself.
-static const DmaTile kDmaTiles[] = {{4, 256, 256, 8.f, 11.f, 0.67f, 1}, {5, 256, 128, 5.f, 0.f, 0.53f, 1},
-                                    {6, 128, 256, 5.f, 0.f, 0.50f, 1}, {7, 128, 128, 4.f, 0.f, 0.36f, 2}};
+static const DmaTile kDmaTiles[] = {{4, 256, 256, 8.f, 11.f, 0.67f, 1}, {10, 256, 192, 5.f, 6.f, 0.61f, 1},
+                                    {5, 256, 128, 5.f, 0.f, 0.53f, 1}, {6, 128, 256, 5.f, 0.f, 0.50f, 1},
+                                    {7, 128, 128, 4.f, 0.f, 0.36f, 2}};
 
 static float estimated_us(const DmaTile& t, int M, int N, int K, int ranges) {
   const long wgs = static_cast<long>((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * ranges;
@@ -756,7 +758,8 @@ extern "C" int tie_gemm_bf16_tile(int M, int N, int K, int packed, int splits) {
 // tile: 0 = choose, 1 = 128x128 (four waves of 64x64), 2 = 256x256 (eight waves of 128x64),
 //       3 = 256x128 (eight waves of 64x64), 4 = 256x256 and 5 = 256x128 loaded straight into LDS (four
 //       waves of 128x128 or 128x64; K % 32 == 0, N % 4 == 0, 16-byte aligned operands, else refused),
-//       6 = 128x256, 7 = 128x128, 8 = 64x256, 9 = 64x128 likewise, for fewer rows.
+//       6 = 128x256, 7 = 128x128, 8 = 64x256, 9 = 64x128 likewise, for fewer rows; 10 = 256x192 likewise, for
+//       widths that 256 columns a tile leave with a round of workgroups that does not fill the compute units.
 // packed: w is stored in blocks of 16 rows x 32 k, 1 KB each, in the matrix cores' operand order (as the
 //       decode product reads it); N % 16 == 0, and only tiles 4 and 5 read it.
 extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
@@ -768,13 +771,13 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
   const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
   const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
-  if (packed && (N % 16 != 0 || !straight || (tile != 0 && (tile < 4 || tile > 9)))) return TIE_BAD_ARGUMENT;
+  if (packed && (N % 16 != 0 || !straight || (tile != 0 && (tile < 4 || tile > 10)))) return TIE_BAD_ARGUMENT;
   if (tile == 0) {
     tile = gemm_plan(M, N, K, straight, splits, packed != 0).tile;
   } else if (tile < 4 && splits > 1) {
     tile = 1;
   }
-  if (tile >= 4 && tile <= 9) {
+  if (tile >= 4 && tile <= 10) {
     if (!straight) return TIE_BAD_ARGUMENT;
 #define DMA(BM, BN)                                                                            \
   return packed ? launch_gemm_dma<BM, BN, true>(x, w, out, epi, M, N, K, splits, stream)       \
@@ -785,7 +788,8 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
       case 6: DMA(128, 256);
       case 7: DMA(128, 128);
       case 8: DMA(64, 256);
-      default: DMA(64, 128);
+      case 9: DMA(64, 128);
+      default: DMA(256, 192);
     }
 #undef DMA
   }

@@ -615,8 +615,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
               gated: bool = False, splits: int = 1) -> None:
     """out (+)= x @ w.T for bfloat16 operands on the matrix cores, any number of rows; K % 8 == 0.
 
-    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256, 3 = 256x128; 4 = 256x256 and 5 = 256x128 with
-    operand slices loaded straight into LDS, which need K % 32 == 0 and N % 4 == 0; 0 lets the kernel choose);
+    ``tile`` picks the workgroup tile (1 = 128x128, 2 = 256x256, 3 = 256x128; 4 = 256x256, 5 = 256x128, 6 = 128x256,
+    7 = 128x128, 8 = 64x256, 9 = 64x128 and 10 = 256x192 with operand slices loaded straight into LDS, which need
+    K % 32 == 0 and N % 4 == 0; 0 lets the kernel choose);
     ``gated`` and ``splits`` as in ``skinny_gemm_bf16`` (planes of partial sums, ``[splits, M, N]`` float32).
     """
     if splits > 1:
