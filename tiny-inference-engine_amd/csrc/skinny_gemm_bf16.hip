@@ -90,6 +90,17 @@ __device__ __forceinline__ void rows_wait_loads() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// The sum of v over the 16 lanes that share lane / 16, in every one of them: four rotations within the row of 16
+// (data-parallel primitives of the vector unit, a few cycles each, where a shuffle goes through LDS). Additions
+// commute, so the 16 lanes end with the same bits.
+__device__ __forceinline__ float sum_of_16_lanes(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
 // The sums of squares a norm left per 16-column tile, [rows][tiles rounded up to 64]: dynamic LDS, present only in
 // launches whose sums are to be scaled (SkNorm::scale_squares).
 extern __shared__ float sk_scale_parts[];
@@ -103,7 +114,6 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
                                                                          SkNorm norm) {
   const int tile_group = blockIdx.x, split = blockIdx.y, num_splits = gridDim.y;
   __shared__ float red[WAVES][MT][RT][256];
-  __shared__ float row_scale[SK_NORM_ROWS];
   const int lane = threadIdx.x & (TIE_WAVE - 1);
   const int wave = threadIdx.x / TIE_WAVE;
   const bool scaled = norm.scale_squares != nullptr;
@@ -233,17 +243,8 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
     }
   }
 
-  if (scaled) {
-    // Each wave sums the rows it asked for: lane l adds the tiles l, l + 64, ... in ascending order, then the
-    // lanes meet in a fixed butterfly. The same sums in every workgroup of every launch, whatever the batch.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    for (int m = wave; m < M && m < SK_NORM_ROWS; m += WAVES) {
-      float sq = 0.f;
-      for (int j = 0; j < scale_chunks; ++j) sq += sk_scale_parts[(m * scale_chunks + j) * TIE_WAVE + lane];
-      sq = wave_sum(sq);
-      if (lane == 0) row_scale[m] = 1.0f / sqrtf(sq / norm.scale_n + norm.scale_eps);
-    }
-  }
+  // The tiles' sums have to be there before the barrier below, whichever wave asked for them.
+  if (scaled) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // D layout: lane holds rows (lane / 16) * 4 + v of x, column lane % 16 of w.
 #pragma unroll
@@ -255,6 +256,18 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
   __syncthreads();
 
   const bool partial = num_splits > 1;   // then TO is float and out holds one [M, N] plane per split
+  // 1 / rms of the row this thread's elements lie in (thread e: row e / 16 % 16, in every pass of the loops
+  // below). The 16 lanes of a row add its tiles j, j + 16, ... each in ascending order, then meet: the same
+  // sums in every workgroup of every launch, whatever the batch.
+  float row_scale = 1.0f;
+  if (scaled) {
+    const int m = (static_cast<int>(threadIdx.x) & 255) >> 4, j = threadIdx.x & 15;
+    float sq = 0.f;
+    if (m < M)
+      for (int i = j; i < scale_chunks * TIE_WAVE; i += 16) sq += sk_scale_parts[m * scale_chunks * TIE_WAVE + i];
+    sq = sum_of_16_lanes(sq);
+    row_scale = 1.0f / sqrtf(sq / norm.scale_n + norm.scale_eps);
+  }
   if (norm.next_x != nullptr) {
     // The end of a sub-layer (MT = 1, one plane, float32 out = the residual stream): the 16 lanes that hold a
     // row's 16 columns of a tile stay together for the sum of its squares.
@@ -272,16 +285,12 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
         for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][0][t][ee];
         float now = 0.f;
         if (inside) {
-          if (scaled) sum *= row_scale[m];
+          if (scaled) sum *= row_scale;
           now = stream_now[i] + sum;
           out[static_cast<size_t>(m) * N + n] = now;
           norm.next_x[static_cast<size_t>(m) * N + n] = float_to_bf16(now * next_weight[i]);
         }
-        float sq = now * now;
-        sq += __shfl_xor(sq, 1, TIE_WAVE);
-        sq += __shfl_xor(sq, 2, TIE_WAVE);
-        sq += __shfl_xor(sq, 4, TIE_WAVE);
-        sq += __shfl_xor(sq, 8, TIE_WAVE);
+        const float sq = sum_of_16_lanes(now * now);
         if (c == 0 && m < M && n < N) norm.squares[static_cast<size_t>(m) * (N / 16) + n / 16] = sq;
       }
     }
@@ -299,12 +308,12 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
     float sum = red[0][mt][t][ee];
 #pragma unroll
     for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][mt][t][ee];
-    if (scaled) sum *= row_scale[m];
+    if (scaled) sum *= row_scale;
     if (gated) {
       float up = red[0][mt][t][ee + 8];
 #pragma unroll
       for (int wv = 1; wv < WAVES; ++wv) up += red[wv][mt][t][ee + 8];
-      if (scaled) up *= row_scale[m];
+      if (scaled) up *= row_scale;
       store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
       continue;
     }
