@@ -99,3 +99,34 @@ def test_the_report_sums_up_a_run():
     assert "queued ahead" not in text
     late = summarize(BenchRun([RequestTiming(0.0, 10, [1.0, 1.5])], 2.0, 2, 2, 0, tokens_read_late=True))
     assert late.tokens_read_late and "queued ahead" in format_report(late)
+
+
+def test_kernel_trace_summaries(tmp_path):
+    """Totals, a decode step's average and the busy share, from a hand-made trace: three steps of an embedding
+    kernel (1 us) and a product (10 us) with 4 us between the steps."""
+    import sqlite3
+
+    from tie_amd.bench import kernel_trace
+
+    path = str(tmp_path / "trace.db")
+    db = sqlite3.connect(path)
+    db.execute("create table kernels (name text, start integer, end integer, grid_x integer, grid_y integer, grid_z integer)")
+    t = 1_000_000
+    for _ in range(3):
+        db.execute("insert into kernels values ('void embed_kernel<float>(int*)', ?, ?, 256, 1, 1)", (t, t + 1000))
+        db.execute("insert into kernels values ('void product<1, 2>(float const*)', ?, ?, 512, 2, 1)", (t + 1000, t + 11000))
+        t += 15000
+    db.commit()
+    db.close()
+    launches = kernel_trace.read_launches(path)
+    assert len(launches) == 6 and launches[1][3] == 1024
+    text = kernel_trace.totals(launches)
+    assert "product<1, 2>" in text and "embed_kernel<float>" in text and "(" not in text.split("\n")[1]
+    assert "kernel time 0.0 ms" in text
+    steps = kernel_trace.last_steps(launches, 2, "embed_kernel")
+    assert "2 steps: kernel span 11.0 us/step, kernel busy 11.0 us/step, step period 15.0 us" in steps
+    # the last 30 us: two whole steps' kernels less the first's first microsecond... exactly: from 11 us before the
+    # first of them ends; 4 us of every 15 idle
+    share = kernel_trace.busy_share(launches, 30e-6)
+    assert "= 0.733" in share and "shorter: 2 totalling" in share
+    assert kernel_trace.main([path, "--steps", "2", "--window", "0.00003", "--by-grid"]) == 0

@@ -218,9 +218,9 @@ PACKED_WIDTHS = {
 
 
 def test_steps_of_a_few_rows_leave_the_norms_to_the_products(tmp_path, monkeypatch):
-    """In steps of up to 16 rows the product that ends a sub-layer adds to the stream and prepares the next norm in
-    its epilogue, and the products behind that norm apply its 1 / rms: no norm kernel runs between the layers'
-    parts. Both ways against the plain implementation, through decoding, small portions and mixed steps; the norm
+    """In steps of a few rows (how few is a measured rule by the weight's shape) the product that ends a sub-layer
+    adds to the stream and prepares the next norm in its epilogue, and the products behind that norm apply its
+    1 / rms: no norm kernel runs between the layers' parts. Both ways against the plain implementation, through decoding, small portions and mixed steps; the norm
     kernels that still run are the first layer's first (nothing precedes it) and the head's."""
     from tie_amd import kernels
     from tie_amd.engine.replay import TraceReplayer
@@ -232,6 +232,8 @@ def test_steps_of_a_few_rows_leave_the_norms_to_the_products(tmp_path, monkeypat
     requests = th.make_requests(cfg["vocab_size"], [5, 11, 17, 40, 64, 33], seed=15)
     want = reference_logits(folder, cfg, requests)
     layers = cfg["num_hidden_layers"]
+    few_rows = kernels.norm_epilogue_rows(cfg["hidden_size"], cfg["intermediate_size"])   # of the product that ends a layer
+    assert 2 <= few_rows == kernels.norm_epilogue_rows(cfg["hidden_size"], 4 * 32) <= kernels.NORM_EPILOGUE_ROWS
     calls = []
     for fn in ("rms_norm", "add_partials"):
         real = getattr(kernels, fn)
@@ -248,7 +250,7 @@ def test_steps_of_a_few_rows_leave_the_norms_to_the_products(tmp_path, monkeypat
             del calls[:]
             out = _real(step)
             rows = sum(len(e["tokens"]) for e in step["entries"])
-            _seen.setdefault(rows <= kernels.NORM_EPILOGUE_ROWS, []).append(len(calls))
+            _seen.setdefault(rows <= few_rows, []).append(len(calls))
             return out
 
         rep.run_step = counted

@@ -594,16 +594,37 @@ extern "C" int tie_skinny_gemm_splits(int N, int K) {
   return splits;
 }
 
+// A product that ends a sub-layer (launch_skinny with SkNorm::next_x) is not cut along K, so a narrow output
+// leaves it few workgroups: wider workgroups then keep as many bytes in flight as the planes of a cut product
+// would. Sixteen waves over one tile where the tiles leave every compute unit at most one workgroup; eight
+// waves over two tiles where pairs of tiles do; else the ordinary four waves. Measured in chains of a layer's
+// four products against the same chain with planes and norm kernels (us a layer, planes | this way):
+//   4096 wide (256 tiles; 2048 and 2560 wide alike): 1 row 73.6 | 67.9, 8 rows 79.9 | 74.4, 16 rows 80.9 | 80.2;
+//   5120 wide (320 tiles), K of 8192 and 25600: 1 row 166.7 | 159.4, 4 rows 161.9 | 163.8, 8 rows 174.4 | 178.6;
+//   5120 wide, K of 5120 and 17408: 1 row 123.3 | 113.2, 4 rows 119.6 | 117.7, 8 rows 127.8 | 128.9.
+// (One tile and sixteen waves over 320 tiles: 193 us at 8 rows; every workgroup reads all of x.)
+struct ProducerShape { int rt, u, waves; };
+static ProducerShape producer_shape(int N) {
+  const int tiles = (N + 15) / 16, cus = compute_units();
+  if (tiles <= cus) return {1, 4, 16};
+  if (tiles <= 2 * cus) return {2, 4, 8};
+  return {0, 0, SK_WAVES};
+}
+
+// The most rows for which a product over w[N, K] that ends a sub-layer is worth running with the next norm's
+// work in its epilogue instead of as planes that a norm kernel adds (the figures above); 0: never.
+extern "C" int tie_skinny_norm_epilogue_rows(int N, int K) {
+  if (N % 16 != 0 || K % 32 != 0) return 0;
+  const int tiles = N / 16, cus = compute_units();
+  if (tiles <= cus) return 8;
+  if (tiles <= 2 * cus) return 4;
+  return 0;
+}
+
 // gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
 // and receives silu(gate) * up.
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 // packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
-// Waves a workgroup of a product that ends a sub-layer (see launch_skinny): sixteen where the output's tiles
-// leave every compute unit at most one workgroup. Measured in a chain of a layer's four products, 4096 wide:
-// 71.8 -> 67.8 us a layer at 1 row, 76.4 -> 75.0 at 8; with 320 tiles (5120 wide, where four waves take
-// several tiles a workgroup and read x less often) sixteen waves lose, 180 -> 193 us at 8 rows.
-static int producer_waves(int N) { return (N + 15) / 16 <= compute_units() ? 16 : SK_WAVES; }
-
 static int launch_skinny(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,
                          int N, int K, int splits, int packed, int rt, int u, int waves, const SkNorm& norm,
                          hipStream_t stream) {
@@ -629,8 +650,16 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
   const int kblocks = (K + 31) / 32;
   // A product that ends a sub-layer is not cut along K, so a narrow output leaves it one workgroup a compute
   // unit: more waves a workgroup then keep as many bytes in flight as the planes of a cut product would.
-  const bool many_waves_fit = norm.next_x != nullptr && packed && rt <= 1 && u >= 0;
-  if (waves == 0) waves = many_waves_fit ? producer_waves(N) : SK_WAVES;
+  const bool many_waves_fit = norm.next_x != nullptr && packed && rt <= 2 && u >= 0;
+  if (waves == 0) {
+    waves = SK_WAVES;
+    if (many_waves_fit && rt == 0 && u == 0) {
+      const ProducerShape by_rule = producer_shape(N);
+      rt = by_rule.rt;
+      u = by_rule.u;
+      waves = by_rule.waves;
+    }
+  }
   if (waves != SK_WAVES && !(many_waves_fit && (waves == 8 || waves == 16))) return TIE_BAD_ARGUMENT;
   const int per_wave = (kblocks + splits * waves - 1) / (splits * waves);
   // x through LDS (17 to 64 rows over packed weights, x within 32-bit byte offsets). With u = 1, rt is the
@@ -662,16 +691,21 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
     return tie_launch_status();
   }
   if (waves != SK_WAVES) {
-    const dim3 wgrid((N + 15) / 16, 1);
-    if (u == 0) u = waves == 8 ? 8 : 4;
-#define LAUNCH_W(U, W)                                                                                         \
-  skinny_gemm_kernel<1, 1, U, float, true, W><<<wgrid, W * TIE_WAVE, scale_lds, stream>>>(                      \
+    if (rt == 0) rt = 1;
+    const dim3 wgrid(((N + 15) / 16 + rt - 1) / rt, 1);
+    if (u == 0) u = waves == 8 ? 8 / rt : 4;
+#define LAUNCH_W(RT, U, W)                                                                                      \
+  skinny_gemm_kernel<1, RT, U, float, true, W><<<wgrid, W * TIE_WAVE, scale_lds, stream>>>(                     \
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<float*>(out), M, N, K, accumulate, \
       gated, per_wave, norm)
-    if (waves == 8 && u == 8) LAUNCH_W(8, 8);
-    else if (waves == 8 && u == 4) LAUNCH_W(4, 8);
-    else if (waves == 16 && u == 4) LAUNCH_W(4, 16);
-    else if (waves == 16 && u == 2) LAUNCH_W(2, 16);
+    if (rt == 1 && waves == 8 && u == 8) LAUNCH_W(1, 8, 8);
+    else if (rt == 1 && waves == 8 && u == 4) LAUNCH_W(1, 4, 8);
+    else if (rt == 1 && waves == 16 && u == 4) LAUNCH_W(1, 4, 16);
+    else if (rt == 1 && waves == 16 && u == 2) LAUNCH_W(1, 2, 16);
+    else if (rt == 2 && waves == 8 && u == 4) LAUNCH_W(2, 4, 8);
+    else if (rt == 2 && waves == 8 && u == 2) LAUNCH_W(2, 2, 8);
+    else if (rt == 2 && waves == 16 && u == 4) LAUNCH_W(2, 4, 16);
+    else if (rt == 2 && waves == 16 && u == 2) LAUNCH_W(2, 2, 16);
     else return TIE_BAD_ARGUMENT;
 #undef LAUNCH_W
     return tie_launch_status();
@@ -730,12 +764,13 @@ extern "C" int tie_skinny_gemm_bf16(const void* x, const void* w, void* out, int
 // scale_squares (or null): [M][scale_tiles] sums of squares of the rows x was made from; the sums are multiplied by
 // 1 / sqrt(their total / scale_n + scale_eps). next_x (or null; then accumulate, one plane, float32 out, N % 16 == 0):
 // out += sums in place, next_x = bf16(out * next_w), squares[M][N / 16] = sums of out^2 per 16-column tile.
-// u, waves: 0 = by the rule (measurements name k-blocks a batch of loads and waves a workgroup themselves).
+// rt, u, waves: 0 = by the rule (measurements name tiles a workgroup, k-blocks a batch of loads and waves a
+// workgroup themselves).
 extern "C" int tie_skinny_gemm_bf16_norm(const void* x, const void* w, void* out, int out_dtype, int accumulate,
                                          int gated, int M, int N, int K, int splits, int packed,
                                          const float* scale_squares, int scale_tiles, float scale_n, float scale_eps,
-                                         const float* next_w, void* next_x, float* squares, int u, int waves,
+                                         const float* next_w, void* next_x, float* squares, int rt, int u, int waves,
                                          hipStream_t stream) {
   const SkNorm norm = {scale_squares, scale_tiles, scale_n, scale_eps, next_w, static_cast<bf16_t*>(next_x), squares};
-  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, 0, u, waves, norm, stream);
+  return launch_skinny(x, w, out, out_dtype, accumulate, gated, M, N, K, splits, packed, rt, u, waves, norm, stream);
 }

@@ -10,6 +10,7 @@ InvalidArgument before anything is launched.
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Dict, Optional
 
 import torch
@@ -111,9 +112,10 @@ _SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_void],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_void],
+        "tie_skinny_norm_epilogue_rows": [_c_int, _c_int],
         "tie_skinny_gemm_bf16_norm": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                       _c_int, _c_void, _c_int, _c_float, _c_float, _c_void, _c_void, _c_void, _c_int,
-                                      _c_int, _c_void],
+                                      _c_int, _c_int, _c_void],
     },
     "gemm_bf16": {
         "tie_gemm_bf16_splits": [_c_int, _c_int, _c_int, _c_int],
@@ -546,7 +548,7 @@ class RowScale:
 
 def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
                      gated: bool = False, splits: int = 1, row_scale: Optional[RowScale] = None,
-                     next_norm: Optional[tuple] = None, loads: int = 0, waves: int = 0) -> None:
+                     next_norm: Optional[tuple] = None, tiles: int = 0, loads: int = 0, waves: int = 0) -> None:
     """out (+)= x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w, on the matrix cores.
 
     ``gated``: w is a gate/up pair interleaved by ``interleave_gate_up`` and out receives silu(gate) * up.
@@ -598,7 +600,7 @@ def skinny_gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumu
     _call(_lib("skinny_gemm_bf16").tie_skinny_gemm_bf16_norm, "skinny_gemm_bf16_norm",
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "matmul output"), int(accumulate), int(gated), M, N, K,
         int(splits), int(isinstance(w, PackedWeight)), _ptr(squares_in), tiles_in, n_in, eps_in, _ptr(next_w),
-        _ptr(next_x), _ptr(squares_out), int(loads), int(waves), _stream())
+        _ptr(next_x), _ptr(squares_out), int(tiles), int(loads), int(waves), _stream())
 
 
 def gemm_splits(M: int, N: int, K: int, packed: bool = False) -> int:
@@ -676,6 +678,14 @@ def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tenso
         raise InvalidArgument(f"{x.shape[0]} rows without their norm's factor: only the decode product applies it")
     else:
         gemm_bf16(x, w_interleaved, out, gated=True)
+
+
+@functools.lru_cache(maxsize=None)
+def norm_epilogue_rows(N: int, K: int) -> int:
+    """The most rows for which a product over a packed ``[N, K]`` weight that ends a sub-layer is worth running
+    with the next norm's work in its epilogue (``skinny_gemm_bf16(next_norm=...)``) rather than as planes that a
+    norm kernel adds; 0 where it never is. Never above ``NORM_EPILOGUE_ROWS``."""
+    return min(NORM_EPILOGUE_ROWS, int(_lib("skinny_gemm_bf16").tie_skinny_norm_epilogue_rows(N, K)))
 
 
 def applies_row_scale(x: torch.Tensor, w) -> bool:

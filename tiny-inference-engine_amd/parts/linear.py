@@ -74,7 +74,7 @@ class Linear:
         """Whether the decode product takes this product with the next norm's work in its epilogue."""
         w = self.weight
         return kernels.NORMS_IN_PRODUCTS and x.dtype == torch.bfloat16 and isinstance(w, kernels.PackedWeight) and \
-            x.shape[0] <= kernels.NORM_EPILOGUE_ROWS and x.is_cuda
+            x.is_cuda and x.shape[0] <= kernels.norm_epilogue_rows(w.shape[0], w.shape[1])
 
     def add_to(self, ctx, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """out += x @ W^T now, or as planes of partial sums owed to ``out``."""
