@@ -162,3 +162,38 @@ def test_the_prefill_attention_kernel_refuses_caches_it_cannot_address():
     assert not kernels.prefill_addressable(plane(1 << 20, 8, 16, 128))      # 32 GB
     assert not kernels.prefill_addressable(plane(4, 64, 4096, 256))         # a page of 128 MB
     assert not kernels.prefill_addressable(plane(1 << 24, 1, 4, 16))        # 2^24 pages
+
+
+def test_the_decode_products_plan_for_17_to_64_rows():
+    """Which kernel, how many tiles a workgroup and how many ranges of K come from one score (what x costs beside
+    the weights, the planes, how full the compute units are), not from a table of shapes: its choices on the shapes
+    it was measured on, and what must hold on any shape."""
+    from tie_amd import kernels
+
+    # 8B QKV at 24 rows: x through LDS, three tiles a workgroup, two ranges: 256 workgroups, one a compute unit
+    # (15.1 us with the kernel that adds the planes; six tiles in four ranges, the same 256 workgroups: 17.1)
+    assert kernels.few_rows_plan(24, 6144, 4096) == (True, 3, 2)
+    # a gate/up of 16384 x 3072: 1024 tiles are 342 workgroups of three or 171 of six, a round and a third or two
+    # thirds of one; x from memory in workgroups of four tiles fills one round exactly (20.6 against 22.4 and 24.7 us)
+    assert kernels.few_rows_plan(24, 16384, 3072, True) == (False, 4, 1)
+    # a gate/up of 34816 x 5120: eight tiles a workgroup would be 272 workgroups, a second round for 16 of them
+    assert kernels.few_rows_plan(32, 34816, 5120, True) == (True, 3, 1)
+    # up to 16 rows the shape alone decides
+    assert kernels.few_rows_plan(16, 6144, 4096) == (False, 0, kernels.skinny_splits(6144, 4096))
+    for N, K in ((6144, 4096), (4096, 12288), (5120, 3072), (2560, 9728), (1024, 2048), (8192, 28672), (10240, 5120)):
+        for M in (17, 24, 32, 33, 48, 64):
+            shares_x, tiles, splits = kernels.few_rows_plan(M, N, K)
+            assert splits in (1, 2, 4, 8) and tiles in ((3, 6, 8) if shares_x else (1, 2, 3, 4)), (M, N, K)
+            if shares_x:      # whole chunks of four k-blocks a wave, ranges of at least 1024 of K
+                assert (K // 32) % (16 * splits) == 0 and (splits == 1 or K // splits >= 1024), (M, N, K, splits)
+            assert kernels.few_rows_plan(M, N, K, True)[2] == 1                      # a gated product is never cut
+    # the tiled product with 64-row tiles: the 32B shape's QKV in two ranges of 64 x 128 tiles (160 workgroups), not
+    # eight of 64 x 256 (320: a second round for 64 of them, 1.7 times the time); a tile is the same whether the
+    # plan is asked for the ranges too or handed them back
+    assert (kernels.gemm_tile(64, 10240, 5120, True), kernels.gemm_splits(64, 10240, 5120, True)) == (9, 2)
+    for N, K in ((6144, 4096), (4096, 12288), (10240, 5120), (8192, 8192), (1024, 2048), (5120, 25600)):
+        for M in (40, 64):
+            ranges = kernels.gemm_splits(M, N, K, True)
+            assert ranges in (1, 2, 4, 8) and (ranges == 1 or K // ranges >= 512)
+            assert kernels.gemm_tile(M, N, K, True) == kernels.gemm_tile(M, N, K, True, ranges) in (8, 9)
+    assert kernels.gemm_tile(64, 51200, 5120, True, 1) == 8 and kernels.gemm_tile(64, 151936, 4096, True, 1) == 8

@@ -693,17 +693,32 @@ static GemmPlan gemm_plan(int M, int N, int K, bool straight_to_lds, int splits,
     return best;
   }
   if (straight_to_lds && packed && M <= 64) {
-    // Up to 64 rows over packed weights: tiles of 64 rows (measured on the projections of the 1.7B, 8B and
-    // 32B shapes at 48 to 64 rows). Wide weights take 256 columns a tile, narrow ones 128 and more ranges of K.
-    const bool wide = N >= 8192;
-    const int tile = wide ? 8 : 9;
-    if (!may_split) return {tile, splits};
-    const long tiles = (N + (wide ? 255 : 127)) / (wide ? 256 : 128);
-    for (int r = 1; r <= 8; r *= 2)
-      if (tiles * r >= 192 && K / r >= 512) return {tile, r};
-    int r = 8;
-    while (r > 1 && K / r < 512) r /= 2;
-    return {tile, r};
+    // Up to 64 rows over packed weights: tiles of 64 rows, one workgroup a compute unit, the weights read once. The
+    // cheapest (tile, ranges) by a score of three factors: what the 64 rows of x cost beside a tile's columns
+    // (1 + 1 / columns' 16-blocks), the planes' traffic and shorter runs of K (1 + 0.25 log2(ranges)), and how
+    // full the rounds of 256 workgroups are. The caller's fixed ranges (a gated product: one) are scored alone,
+    // with the same result when it hands back what this plan chose. Ranges of at least 512 of K. Over the
+    // projections of eight shapes at 48 and 64 rows the choice lies 2.9 % above the best forced (tile, ranges) on
+    // average and at most 17 %; the rule by thresholds that stood here gave the 32B shape's QKV (40 tiles of 256
+    // columns) eight ranges, 320 workgroups, a second round for 64 of them: 1.7 times the time of four.
+    GemmPlan best = {9, may_split ? 1 : splits};
+    float best_score = 0.f;
+    // a weight so wide that the wider tile alone fills a round (an lm_head) has nothing to balance: the wider tile
+    for (int tile = (N + 255) / 256 >= 256 ? 8 : 9; tile >= 8; --tile) {
+      const int columns = tile == 8 ? 256 : 128;
+      const long across = (N + columns - 1) / columns;
+      for (int r = may_split ? 1 : splits; r <= (may_split ? 8 : splits); r *= 2) {
+        if (may_split && r > 1 && K / r < 512) break;
+        const long wgs = across * r;
+        const float fill = static_cast<float>(wgs) / static_cast<float>((wgs + 255) / 256 * 256);
+        const float score = (1.0f + 16.0f / columns) * (1.0f + 0.25f * log2f(static_cast<float>(r))) / fill;
+        if (best_score == 0.f || score < best_score) {
+          best = {tile, r};
+          best_score = score;
+        }
+      }
+    }
+    return best;
   }
   if (straight_to_lds && M > 128) {
     GemmPlan best = {4, may_split ? 1 : splits};

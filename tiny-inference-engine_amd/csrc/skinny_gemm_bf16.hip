@@ -552,35 +552,68 @@ static int choose_rt(int M, int N, int splits) {
   return best;
 }
 
-// Weight tiles a workgroup of the kernel that shares x through LDS takes (8: four waves x two tiles, 6: three
-// waves x two, 3: three waves x one), or 0 where another kernel is as fast or faster: the one that reads x from
-// memory, or above 32 rows the tiled product with 64-row tiles. Measured on the projections of the 1.7B, 8B and
-// 32B shapes at 20 to 64 rows:
-//   * very wide weights (the lm_head, a gate/up of 51200 rows): 10 to 25 % over the memory kernel up to 32
-//     rows; above, the tiled product is faster still;
-//   * a gate/up of 24576 x 4096: 7 % at 20 rows, 11 % at 32, 18 % at 48, 25 % at 64; of 12288 x 2048: 8 to 13 %
-//     up to 48 rows in the small workgroups;
-//   * weights cut along K (QKV, O, down): where the workgroups of six tiles fill the compute units in one
-//     round (200 to 256 of them: the 8B shape's QKV, the 32B's QKV and O) 7 to 24 %, also over the tiled
-//     product at 48 and 64 rows; with fewer workgroups (172 for a 4096-row weight) or short ranges the others win.
-static int rows_kernel_tiles(int M, int N, int K, int gated, int splits) {
-  if (M <= 16 || M > 64) return 0;
-  const int kblocks = (K + 31) / 32;
-  const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
-  if (K % 32 != 0 || per_wave % 4 != 0) return 0;      // the parts of K in which the sums are formed are whole chunks
-  if (N >= 32768) return M <= 32 ? (K >= 4096 ? 8 : 6) : 0;
-  if (gated) {
-    if (N >= 16384 && K >= 4096) return M <= 24 ? 3 : 6;
-    if (N >= 8192 && K >= 2048 && M <= 48) return 3;
-    return 0;
+// Which kernel, how many weight tiles a workgroup and how many ranges of K a product of 17 to 64 rows takes
+// (up to 16 rows: the kernel that reads x from memory, choose_rt and tie_skinny_gemm_splits). One score for
+// every candidate, the smallest wins:
+//
+//     (1 + b x (16-row tiles of x) / (weight tiles that share one load of x)) x (1 + 0.15 log2(ranges)) / fill
+//
+// The first factor is what x costs beside the weights: a wave of the kernel that reads x from memory loads a
+// block of x for every `rt` weight blocks (b = 0.4); in the kernel that shares x through LDS a workgroup loads it
+// once for its 3, 6 or 8 tiles (b = 0.2, and the whole score x 0.95: its loads never drain). The second is the
+// planes' traffic and the shorter runs of K. The third is how full the compute units are: workgroups run in
+// rounds of one a compute unit, and a round that is part empty lasts as long as a full one.
+// The constants were chosen on sweeps over the four projections of eight shapes (widths 1024 to 8192) at 24 to 64
+// rows, every candidate timed together with the kernel that consumes its planes: the choice lies 2.3 % above the
+// best candidate on average (the thresholds on three shapes that stood here before: 7.3 %), within 5 % on 105 of
+// 128 points, and on the three shapes held out of the choosing (widths 2560, 3072 and 5120 with K of 17408) 2.7 %.
+extern "C" int tie_skinny_gemm_splits(int N, int K);
+
+struct FewRowsPlan { int shares_x, tiles, splits; };
+
+static FewRowsPlan few_rows_plan(int M, int N, int K, int gated, int splits_fixed) {
+  const int tiles = (N + 15) / 16, kblocks = (K + 31) / 32, cus = compute_units();
+  const int by_shape = gated ? 1 : tie_skinny_gemm_splits(N, K);
+  FewRowsPlan best = {0, 1, splits_fixed > 0 ? splits_fixed : by_shape};
+  double best_score = 0.0;
+  auto fill = [&](long wgs) { return static_cast<double>(wgs) / static_cast<double>((wgs + cus - 1) / cus * cus); };
+  auto offer = [&](double score, int shares_x, int t, int splits) {
+    if (best_score == 0.0 || score < best_score) {
+      best = {shares_x, t, splits};
+      best_score = score;
+    }
+  };
+  for (int splits = 1; splits <= 8; splits *= 2) {
+    if (splits_fixed > 0 ? splits != splits_fixed : (gated && splits > 1)) continue;
+    const int per_wave = (kblocks + splits * SK_WAVES - 1) / (splits * SK_WAVES);
+    const double cut = 1.0 + 0.15 * log2(static_cast<double>(splits));
+    // x from memory: no more ranges than the shape alone asks for, none shorter than four k-blocks a wave
+    if (splits_fixed > 0 || splits == 1 || (splits <= by_shape && per_wave >= 4))
+      for (int rt = 1; rt <= (M > 8 ? 4 : 3); ++rt)
+        offer((1.0 + 0.4 * (M / 16.0) / rt) * cut / fill(static_cast<long>((tiles + rt - 1) / rt) * splits), 0, rt, splits);
+    // x through LDS: whole chunks of four k-blocks a wave, ranges of at least 1024 of K
+    if (M > 16 && K % 32 == 0 && N % 16 == 0 && per_wave % 4 == 0 && (splits == 1 || K / splits >= 1024)) {
+      const int x_tiles = M <= 32 ? 2 : 4;
+      for (int per : {3, 6, 8})
+        offer(0.95 * (1.0 + 0.2 * x_tiles / per) * cut / fill(static_cast<long>((tiles + per - 1) / per) * splits), 1, per,
+              splits);
+    }
   }
-  const long wgs = static_cast<long>(((N + 15) / 16 + 5) / 6) * splits;
-  return wgs >= 200 && wgs <= 256 && K / splits >= 1024 ? 6 : 0;
+  return best;
 }
 
-// The same for callers that choose between this product and the tiled one (packed weights).
-extern "C" int tie_skinny_rows_kernel_tiles(int M, int N, int K, int gated, int splits) {
-  return rows_kernel_tiles(M, N, K, gated, splits);
+// The plan for callers (17 to 64 rows over a packed weight): *shares_x, *tiles as in FewRowsPlan; returns the ranges
+// of K (1 for a gated product).
+extern "C" int tie_skinny_few_rows_plan(int M, int N, int K, int gated, int* shares_x, int* tiles) {
+  if (M <= 16 || M > 64) {
+    if (shares_x != nullptr) *shares_x = 0;
+    if (tiles != nullptr) *tiles = 0;
+    return gated ? 1 : tie_skinny_gemm_splits(N, K);
+  }
+  const FewRowsPlan plan = few_rows_plan(M, N, K, gated, 0);
+  if (shares_x != nullptr) *shares_x = plan.shares_x;
+  if (tiles != nullptr) *tiles = plan.tiles;
+  return plan.splits;
 }
 
 // Ranges of K that a product over w[N, K] is cut into when its caller takes partial sums: weights with
@@ -666,9 +699,14 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
   // number of tiles a workgroup takes: up to 3 three waves x one tile, up to 6 three waves x two, else four x two.
   const int tiles = (N + 15) / 16;
   const bool rows_fit = static_cast<size_t>(M) * K * 2 < (1ull << 31);
-  const int by_rule = rows_kernel_tiles(M, N, K, gated, splits);
   const bool whole_chunks = per_wave % 4 == 0;     // the parts of K in which the sums are formed end between chunks
-  if (!norm_work && packed && mt > 1 && rows_kernel && rows_fit && whole_chunks && (by_rule != 0 || rows_forced)) {
+  const bool rows_take = !norm_work && packed && mt > 1 && rows_fit && whole_chunks && K % 32 == 0;
+  // 17 to 64 rows, nothing forced: the plan says which kernel and how many tiles a workgroup, for these ranges of K
+  FewRowsPlan plan = {0, 0, splits};
+  if (mt > 1 && packed && forced_rt == 0 && u == 0 && rows_kernel && !rows_forced && waves == SK_WAVES)
+    plan = few_rows_plan(M, N, K, gated, splits);
+  const int by_rule = plan.shares_x ? plan.tiles : 0;
+  if (rows_take && rows_kernel && (by_rule != 0 || rows_forced)) {
     const int asked = rows_forced && forced_rt != 0 ? forced_rt : (by_rule != 0 ? by_rule : 6);
     const int per_wg = asked <= 3 ? 3 : (asked <= 6 ? 6 : 8);
     const dim3 rgrid((tiles + per_wg - 1) / per_wg, splits);
@@ -711,10 +749,19 @@ static int launch_skinny(const void* x, const void* w, void* out, int out_dtype,
     return tie_launch_status();
   }
   if (rows_forced) rt = 0;                  // asked for the other kernel, which does not take this shape: by the rule
-  if (rt == 0) rt = choose_rt(M, N, splits);
+  if (rt == 0) rt = (plan.tiles != 0 && !plan.shares_x) ? plan.tiles : choose_rt(M, N, splits);
   if (rt < 1 || rt > 4) return TIE_BAD_ARGUMENT;
   const dim3 grid(((N + 15) / 16 + rt - 1) / rt, splits);
-  if (u == 0) u = rt == 1 ? 8 : (rt == 2 ? 4 : 2);    // blocks per batch of loads; two batches are in flight
+  if (u == 0) {
+    // k-blocks a batch of loads (two batches are in flight): 8, 4 or 2 by the registers the tiles leave, and the
+    // largest of these that divides a wave's share of K: what is left over a batch is loaded block by block,
+    // nothing in flight beside it (a share of 6 k-blocks in batches of 8: 14.3 us where batches of 2 take 10.7).
+    // If none divides it, the largest that leaves at least two batches.
+    const int most = rt == 1 ? 8 : (rt == 2 ? 4 : 2);
+    for (u = most; u > 2 && per_wave % u != 0; u /= 2) {}
+    if (per_wave % u != 0)
+      for (u = most; u > 2 && 2 * u > per_wave; u /= 2) {}
+  }
   if (u != 2 && u != 4 && u != 8) return TIE_BAD_ARGUMENT;
 #define LAUNCH_P(MT, RT, U, TO, P)                                                                           \
   skinny_gemm_kernel<MT, RT, U, TO, P><<<grid, SK_WAVES * TIE_WAVE, scale_lds, stream>>>(                     \

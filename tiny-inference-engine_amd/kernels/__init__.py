@@ -107,7 +107,7 @@ _SIGNATURES = {
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
-        "tie_skinny_rows_kernel_tiles": [_c_int, _c_int, _c_int, _c_int, _c_int],
+        "tie_skinny_few_rows_plan": [_c_int, _c_int, _c_int, _c_int, _c_void, _c_void],
         "tie_skinny_gemm_bf16_with": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_void],
         "tie_skinny_gemm_bf16": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -525,8 +525,20 @@ def _bf16_product_operands(x, w, out, gated, what):
 
 
 def skinny_splits(N: int, K: int) -> int:
-    """Ranges of K a decode-time product over a ``[N, K]`` weight is best cut into when its caller adds partial sums."""
+    """Ranges of K a decode-time product of up to 16 rows over a ``[N, K]`` weight is best cut into when its caller
+    adds partial sums."""
     return int(_lib("skinny_gemm_bf16").tie_skinny_gemm_splits(N, K))
+
+
+@functools.lru_cache(maxsize=None)
+def few_rows_plan(M: int, N: int, K: int, gated: bool = False) -> tuple:
+    """``(shares_x, tiles, splits)`` of the decode product for ``M`` rows over a packed ``[N, K]`` weight: whether the
+    kernel that shares x through LDS runs (17 to 64 rows), the weight tiles a workgroup takes, and the ranges of K
+    the product is best cut into when its caller adds partial sums (up to 16 rows: ``skinny_splits``)."""
+    shares_x, tiles = ctypes.c_int(0), ctypes.c_int(0)
+    splits = int(_lib("skinny_gemm_bf16").tie_skinny_few_rows_plan(M, N, K, int(gated), ctypes.addressof(shares_x),
+                                                                  ctypes.addressof(tiles)))
+    return bool(shares_x.value), tiles.value, splits
 
 
 NORM_EPILOGUE_ROWS = 16      # rows up to which the decode product's epilogue does the norms' work (SkNorm)
@@ -650,9 +662,8 @@ _few_rows_memo: Dict[tuple, bool] = {}
 def decode_product_rows(M: int, w, gated: bool = False) -> bool:
     """Whether ``M`` rows against ``w`` go to the decode product (``skinny_gemm_bf16``) rather than the tiled one.
 
-    Up to 32 rows always, above 64 never; between, by the weight's shape and layout: the decode product where its
-    kernel that shares x through LDS is the measured best, else the tiled product with 64-row tiles over packed
-    weights, except for gated products that are not very wide.
+    Up to 32 rows always, above 64 never; between, the tiled product with 64-row tiles where it takes the weight
+    (packed, whole slices of K), except for gated products that are not very wide (measured).
     """
     if M <= 32 or M > 64:
         return M <= 32
@@ -661,10 +672,7 @@ def decode_product_rows(M: int, w, gated: bool = False) -> bool:
     key = (M, N, K, packed, bool(gated))
     tiled = _few_rows_memo.get(key)
     if tiled is None:
-        shares_x = packed and _lib("skinny_gemm_bf16").tie_skinny_rows_kernel_tiles(
-            M, N, K, int(gated), 1 if gated else skinny_splits(N, K)) != 0
-        tiled = _few_rows_memo[key] = not shares_x and bool(_lib("gemm_bf16").tie_gemm_bf16_wins_few_rows(
-            M, N, K, int(packed), int(gated)))
+        tiled = _few_rows_memo[key] = bool(_lib("gemm_bf16").tie_gemm_bf16_wins_few_rows(M, N, K, int(packed), int(gated)))
     return not tiled
 
 

@@ -108,8 +108,9 @@ class Linear:
     def partial_planes(self, ctx, x: torch.Tensor, name: str):
         """Runs the product as ``[S, M, N]`` float32 planes of partial sums if that is the faster way; else None.
 
-        The decode product (up to 32 rows, or 64 where the tiled one is not the faster) decides by the weight's
-        shape alone; the tiled product is cut along K when its tiles alone would leave most of the GPU idle.
+        The decode product decides by the weight's shape alone up to 16 rows and by its plan for the number of rows
+        above (up to 32 rows, or 64 where the tiled product is not the faster); the tiled product is cut along K
+        when its tiles alone would leave most of the GPU idle.
         """
         M, K = x.shape
         w = self.weight
@@ -117,9 +118,12 @@ class Linear:
             return None
         decode_product = kernels.decode_product_rows(M, w)
         if decode_product:
-            if self._splits is None:
-                self._splits = kernels.skinny_splits(w.shape[0], K)
-            splits = self._splits
+            if M <= 16 or not isinstance(w, kernels.PackedWeight):
+                if self._splits is None:
+                    self._splits = kernels.skinny_splits(w.shape[0], K)
+                splits = self._splits
+            else:
+                splits = kernels.few_rows_plan(M, w.shape[0], K)[2]
         else:
             splits = self._tiled_splits.get(M)
             if splits is None:
