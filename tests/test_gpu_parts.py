@@ -246,6 +246,102 @@ def test_run_orders_shared_caches_and_windows(tmp_path, order, window, dtype, to
     assert replayer.cache.num_free() == replayer.cache.num_blocks
 
 
+@pytest.mark.parametrize("dtype,tolerance", [("float32", tolerances.FLOAT32), ("bfloat16", tolerances.BFLOAT16["run orders"])])
+def test_projections_with_a_bias_are_a_parameter_of_the_attention_part(dtype, tolerance):
+    """An architecture whose q, k, v and o projections have a bias names the vectors in the mixer's parameters:
+    no kernel and no file of the package changes. Through the step function (whole, decoded, in portions, mixed)
+    against the plain formulas with the bias added; and the bias must matter (without it the check fails)."""
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.models import Model
+    from tie_amd.weights.random_init import random_tensors
+    from tie_amd.weights.safetensors_io import StoredTensor
+
+    model, cfg = attention_model(((0, None), (1, None)))
+    layers = []
+    for i, layer in enumerate(model.spec.layers):
+        p = f"model.layers.{i}.self_attn."
+        bias = {"q": p + "q_proj.bias", "k": p + "k_proj.bias", "v": p + "v_proj.bias", "o": p + "o_proj.bias"}
+        layers.append(dataclasses.replace(layer, mixer=dataclasses.replace(layer.mixer, params={**layer.mixer.params, "bias": bias})))
+    model = Model(dataclasses.replace(model.spec, layers=tuple(layers)))
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    tensors = dict(random_tensors(model.expected_tensors(), 9, store, vector_dtype=torch.float32))
+    for name in tensors:
+        if name.endswith(".bias"):
+            tensors[name] = tensors[name] * 20          # init_std 0.02 would leave the bias below the bfloat16 bound
+    assert sum(name.endswith(".bias") for name in tensors) == 8
+    model.load({n: StoredTensor.from_tensor(n, t) for n, t in tensors.items()}, dtype, "cuda:0")
+    weights = {n: t.to(F64) for n, t in tensors.items()}
+
+    def forward(tokens, with_bias=True):
+        c = plain.normalized_config(cfg)
+        T, H, KVH, Dh, eps = len(tokens), c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["rms_norm_eps"]
+        pos = list(range(T))
+        x = plain.embed(weights["model.embed_tokens.weight"], tokens)
+        for layer in range(2):
+            p = f"model.layers.{layer}."
+            b = (lambda n: weights[p + f"self_attn.{n}_proj.bias"]) if with_bias else (lambda n: 0.0)
+            h = plain.rms_norm(x, weights[p + "input_layernorm.weight"], eps)
+            q = plain.rope_neox(plain.rms_norm((plain.linear(h, weights[p + "self_attn.q_proj.weight"]) + b("q")).view(T, H, Dh),
+                                               weights[p + "self_attn.q_norm.weight"], eps), pos, c["rope_theta"])
+            k = plain.rope_neox(plain.rms_norm((plain.linear(h, weights[p + "self_attn.k_proj.weight"]) + b("k")).view(T, KVH, Dh),
+                                               weights[p + "self_attn.k_norm.weight"], eps), pos, c["rope_theta"])
+            v = (plain.linear(h, weights[p + "self_attn.v_proj.weight"]) + b("v")).view(T, KVH, Dh)
+            a = plain.causal_attention(q, k, v, float(np.float32(1.0) / np.sqrt(np.float32(Dh))), None).reshape(T, H * Dh)
+            x = x + plain.linear(a, weights[p + "self_attn.o_proj.weight"]) + b("o")
+            h = plain.rms_norm(x, weights[p + "post_attention_layernorm.weight"], eps)
+            x = x + plain.swiglu(h, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
+                                 weights[p + "mlp.down_proj.weight"])
+        return plain.linear(plain.rms_norm(x, weights["model.norm.weight"], eps), weights["lm_head.weight"])
+
+    requests = th.make_requests(cfg["vocab_size"], [45, 70, 33], seed=8)
+    want = {rid: forward(toks).float() for rid, toks in requests.items()}
+    steps, peak = th.mixed(requests, max_live=3, seed=2)
+    for label, trace, room in (("whole", th.whole(requests), 192), ("prefill + decode", th.prefill_then_decode(requests), 192),
+                               ("mixed", steps, peak)):
+        replayer = TraceReplayer(model, room, block_size=4)
+        got = th.collect(replayer, trace)
+        for rid, ref in want.items():
+            mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
+            close(mine, ref, tolerance, f"biased projections, {label}, request {rid}")
+        assert replayer.cache.num_free() == replayer.cache.num_blocks
+    unbiased = forward(requests["r0"], with_bias=False).float()
+    assert float((unbiased - want["r0"]).abs().max() / want["r0"].abs().max()) > 10 * tolerance, "the bias does not matter"
+
+
+def test_a_projection_with_a_bias_alone():
+    """``Linear(bias=...)``: the product, then the bias, whether it stores, adds to a stream that planes are still
+    owed to, or feeds rows that lack their norm's factor; bfloat16 and float32 rows."""
+    from tie_amd import kernels
+    from tie_amd.parts.linear import Linear
+
+    g = torch.Generator().manual_seed(6)
+    D, K, T = 96, 1024, 5
+    w = {"a": (torch.randn(D, K, generator=g) * 0.05).to(torch.bfloat16), "a.bias": torch.randn(D, generator=g),
+         "b": (torch.randn(D, K, generator=g) * 0.05).to(torch.bfloat16)}
+    fetch = fetcher(w, "bfloat16")
+    biased, plain_one = Linear(["a"], [D], K, bias=["a.bias"]), Linear(["b"], [D], K)
+    biased.load(fetch)
+    plain_one.load(fetch)
+    assert [s.name for s in biased.tensors()] == ["a", "a.bias"] and biased.tensors()[1].shape == (D,)
+    x = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    product = plain.linear(x.to(F64), w["a"].to(F64)) + w["a.bias"].to(F64)
+    for out_dtype, bound in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+        out = torch.full((T, D), float("nan"), dtype=out_dtype, device="cuda")
+        biased(x.cuda(), out)
+        close(out, product, bound, f"biased product stored as {out_dtype}")
+    ctx = make_ctx(T, "bfloat16")
+    stream = torch.randn(T, D, generator=g)
+    residual = stream.cuda().clone()
+    plain_one(x.cuda(), residual, accumulate=True, ctx=ctx)           # left pending or owed
+    biased(x.cuda(), residual, accumulate=True, ctx=ctx)
+    assert ctx._owed is None and ctx._pending is None and biased.partial_planes(ctx, x.cuda(), "p") is None
+    close(residual, stream.to(F64) + plain.linear(x.to(F64), w["b"].to(F64)) + product, 1e-5, "stream after both")
+    with pytest.raises(kernels.InvalidArgument):
+        Linear(["a", "b"], [D, D], K, bias=["a.bias"])
+    with pytest.raises(kernels.InvalidArgument):
+        kernels.add_bias(torch.zeros(T, D, device="cuda"), torch.zeros(D + 1, device="cuda"))
+
+
 # ------------------------------------------------------------------ toy parts, defined and registered here
 def register_toy_parts():
     from tie_amd import kernels

@@ -1,9 +1,10 @@
 """How far the products' own choice of kernel, tile and ranges of K lies from the best forced choice.
 
-For the four projections of a layer shape (QKV, O, gate/up, down) at a list of row counts up to 64, every
-candidate the launchers can be forced to - the decode product reading x from memory (1 to 4 weight tiles a
+For the four projections of a layer shape (QKV, O, gate/up, down) at a list of row counts, every candidate
+the launchers can be forced to - the decode product reading x from memory (1 to 4 weight tiles a
 workgroup, 2 to 8 k-blocks a batch of loads) or sharing it through LDS (3, 6 or 8 tiles a workgroup), the tiled
-product with 64-row tiles (128 or 256 columns), each in 1 to 8 ranges of K - is timed together with what its
+product (64-row tiles up to 64 rows, tiles of 64 and 128 rows up to 128, of 128 and 256 rows above), each in 1 to 8
+ranges of K - is timed together with what its
 consumer has to do for it (planes: the kernel that adds them to the stream and norms; one plane: accumulate in
 place, then the norm kernel), in a recorded chain over several copies of the weight so that no cache holds it.
 The product's own choice is timed the same way. Prints a line a point and a summary:
@@ -44,8 +45,6 @@ def main(argv=None) -> int:
     D, Q, KV, I = tuple(int(v) for v in args.sizes.split(",")) if args.sizes else SHAPES[args.shape]
     name_of_shape = args.sizes or args.shape
     rows = [int(m) for m in args.rows.split(",")]
-    if max(rows) > 64:
-        raise SystemExit("rows above 64 go to the tiled product's own plan; this sweep covers up to 64")
     lib = kernels._lib("skinny_gemm_bf16")
 
     def timed(fn, copies):
@@ -108,8 +107,8 @@ def main(argv=None) -> int:
             for s in ((1,) if gated else (1, 2, 4, 8)):
                 if s > 1 and K // s < 256:
                     continue
-                variants = [(rt, -u) for rt in (1, 2, 3, 4) for u in (2, 4, 8)]
-                if M > 16:
+                variants = [(rt, -u) for rt in (1, 2, 3, 4) for u in (2, 4, 8)] if M <= 64 else []
+                if 16 < M <= 64:
                     variants += [(3, 1), (6, 1), (8, 1)]
                 for rt, u in variants:
                     out = act if gated else (planes[s] if s > 1 else stream)
@@ -129,7 +128,10 @@ def main(argv=None) -> int:
                     except RuntimeError:
                         pass
                 if M > 32:
-                    for tile, shape in ((8, "64 x 256"), (9, "64 x 128")):
+                    tiles_tried = ((8, "64 x 256"), (9, "64 x 128")) if M <= 64 else \
+                        ((6, "128 x 256"), (7, "128 x 128"), (8, "64 x 256"), (9, "64 x 128")) if M <= 128 else \
+                        ((4, "256 x 256"), (10, "256 x 192"), (5, "256 x 128"), (6, "128 x 256"), (7, "128 x 128"))
+                    for tile, shape in tiles_tried:
                         def tiled(i, tile=tile, s=s):
                             if gated:
                                 kernels.gemm_bf16(x, weights[i], act, gated=True, tile=tile)

@@ -214,6 +214,26 @@ extern "C" int tie_scale_rows(void* rows, int dtype, int M, int width, const flo
   return tie_launch_status();
 }
 
+// ------------------------------------------------------------ a projection's bias
+// rows[m][n] += bias[n], in float32, stored in the rows' own type: a projection with a bias is its product and
+// this (the products' epilogues have no bias term; the reference's projections have none either).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ rows, const float* __restrict__ bias, size_t count, int width) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  store_from_float(rows + i, load_as_float(rows + i) + bias[i % width]);
+}
+
+extern "C" int tie_add_bias(void* rows, int dtype, int M, int width, const float* bias, hipStream_t stream) {
+  if (M <= 0 || width <= 0 || rows == nullptr || bias == nullptr) return TIE_BAD_ARGUMENT;
+  const size_t count = static_cast<size_t>(M) * width;
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+  if (dtype == TIE_F32) add_bias_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<float*>(rows), bias, count, width);
+  else if (dtype == TIE_BF16) add_bias_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(rows), bias, count, width);
+  else return TIE_BAD_ARGUMENT;
+  return tie_launch_status();
+}
+
 // ------------------------------------------------------------ tokens the host has not seen
 // tokens[i] = previous[sources[i]] where sources[i] >= 0: rows whose token an earlier step's sampling kernel left
 // on the device (the host queues this step before it has read that one); the other rows keep the host's token.

@@ -82,6 +82,7 @@ _SIGNATURES = {
         "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
         "tie_scale_rows": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_float, _c_float, _c_void],
+        "tie_add_bias": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_void],
         "tie_take_tokens": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_random_fill": [_c_void, ctypes.c_longlong, ctypes.c_ulonglong, _c_int, ctypes.c_double, _c_void],
         "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -392,6 +393,16 @@ def take_tokens(tokens: torch.Tensor, sources: torch.Tensor, previous: torch.Ten
     _i32(previous, "the earlier step's tokens")
     _call(_lib("elementwise").tie_take_tokens, "take_tokens", tokens.data_ptr(), sources.data_ptr(), previous.data_ptr(),
           T, previous.numel(), _stream())
+
+
+def add_bias(rows: torch.Tensor, bias: torch.Tensor) -> None:
+    """rows[m] += bias, in place (float32 arithmetic; rows float32 or bfloat16, bias float32 ``[width]``)."""
+    _gpu(rows, "rows")
+    if rows.dim() != 2 or not rows.is_contiguous():
+        raise InvalidArgument(f"add_bias takes contiguous rows [M, width], got {list(rows.shape)}")
+    _f32(bias, "bias", (rows.shape[1],))
+    _call(_lib("elementwise").tie_add_bias, "add_bias", rows.data_ptr(), _code(rows, "rows"), rows.shape[0],
+          rows.shape[1], bias.data_ptr(), _stream())
 
 
 def scale_rows(rows: torch.Tensor, row_scale: "RowScale") -> None:

@@ -11,7 +11,9 @@ keys with ``score = scale * q.k``, query head h reading KV head
 Parameters (all from the spec, none assumed): ``hidden``, ``num_heads``,
 ``num_kv_heads``, ``head_dim``, ``scale``, ``window`` (None = all keys),
 ``qk_norm`` (None or ``{"eps", "q_weight", "k_weight"}``), ``position`` (a
-PartSpec of the position family) and ``names`` (``q``, ``k``, ``v``, ``o``).
+PartSpec of the position family), ``names`` (``q``, ``k``, ``v``, ``o``) and, for
+architectures whose projections have one, ``bias`` (names of bias vectors under ``q``,
+``k``, ``v`` - all three or none - and/or ``o``; the reference has none).
 """
 
 from __future__ import annotations
@@ -22,6 +24,7 @@ import torch
 
 from .. import kernels
 from ..cache.spec import PagedKV
+from ..errors import InvalidArgument
 from .base import Mixer, Part, PartSpec, StepContext, TensorSpec, build_part, register_part
 from .linear import Linear
 
@@ -44,8 +47,12 @@ class PagedAttention(Mixer):
         names = params["names"]
         q_dim, kv_dim = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
         self.q_dim, self.kv_dim = q_dim, kv_dim
-        self.qkv = Linear([names["q"], names["k"], names["v"]], [q_dim, kv_dim, kv_dim], self.hidden)
-        self.out = Linear([names["o"]], [self.hidden], q_dim)
+        bias = params.get("bias") or {}
+        if any(k in bias for k in "qkv") and not all(k in bias for k in "qkv"):
+            raise InvalidArgument("the q, k and v projections run as one product: a bias for all three or for none")
+        self.qkv = Linear([names["q"], names["k"], names["v"]], [q_dim, kv_dim, kv_dim], self.hidden,
+                          bias=[bias["q"], bias["k"], bias["v"]] if "q" in bias else None)
+        self.out = Linear([names["o"]], [self.hidden], q_dim, bias=[bias["o"]] if "o" in bias else None)
         self.qk_norm = params.get("qk_norm")
         self.q_norm_weight: torch.Tensor = None
         self.k_norm_weight: torch.Tensor = None

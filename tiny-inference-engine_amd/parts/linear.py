@@ -4,12 +4,13 @@ Weights keep their stored ``[out, in]`` layout (``src/model/qwen3.cpp:81-90``).
 Listing several names concatenates them along the output dimension at load
 time (q, k, v or gate, up in one product): the arithmetic of each output
 column is unchanged, the activation is read once instead of several times.
-No bias: the reference has none.
+The reference's projections have no bias; ``bias`` names one vector per weight for architectures that have
+(added by a kernel of its own after the product, which then is neither cut into planes nor left pending).
 """
 
 from __future__ import annotations
 
-from typing import List, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -19,10 +20,15 @@ from ..weights.binder import TensorSpec
 
 
 class Linear:
-    def __init__(self, names: Sequence[str], out_features: Sequence[int], in_features: int, init_std: float = 0.02):
+    def __init__(self, names: Sequence[str], out_features: Sequence[int], in_features: int, init_std: float = 0.02,
+                 bias: Optional[Sequence[str]] = None):
         if len(names) != len(out_features) or not names:
             raise InvalidArgument("a projection needs one output size per weight name")
+        if bias is not None and len(bias) != len(names):
+            raise InvalidArgument("a projection with a bias needs one bias name per weight name")
         self.names = list(names)
+        self.bias_names = list(bias) if bias is not None else None
+        self.bias: Optional[torch.Tensor] = None          # float32 [total_out], the stored vectors side by side
         self.out_features = list(out_features)
         self.in_features = in_features
         self.init_std = init_std
@@ -35,10 +41,16 @@ class Linear:
         return sum(self.out_features)
 
     def tensors(self) -> List[TensorSpec]:
-        return [TensorSpec(n, (o, self.in_features), "matrix", ("normal", self.init_std))
-                for n, o in zip(self.names, self.out_features)]
+        specs = [TensorSpec(n, (o, self.in_features), "matrix", ("normal", self.init_std))
+                 for n, o in zip(self.names, self.out_features)]
+        if self.bias_names is not None:
+            specs += [TensorSpec(b, (o,), "vector", ("normal", self.init_std))
+                      for b, o in zip(self.bias_names, self.out_features)]
+        return specs
 
     def load(self, fetch) -> None:
+        if self.bias_names is not None:
+            self.bias = torch.cat([fetch(b, "vector").to(torch.float32) for b in self.bias_names]).contiguous()
         parts = [fetch(n, "matrix") for n in self.names]
         if len(parts) == 1:
             self.set_weight(parts[0])
@@ -62,6 +74,12 @@ class Linear:
         ``out`` (or ``ctx.settle()``) adds it. Callers that pass no context always get the sum at once. With
         ``ctx``, rows ``x`` that lack their norm's 1 / rms (``ctx.row_scale_of``) have it applied to the sums.
         """
+        if self.bias is not None:
+            if ctx is not None:
+                ctx.settle()                      # what is still owed to ``out`` lands before this adds to it
+            kernels.linear(x, self.weight, out, accumulate, row_scale=self.row_scale_for(ctx, x, self.weight))
+            kernels.add_bias(out, self.bias)
+            return out
         if ctx is not None and accumulate and out.dtype == torch.float32:
             if self.prepares_norms(x):
                 ctx.defer_product(out, self, x)
@@ -114,7 +132,7 @@ class Linear:
         """
         M, K = x.shape
         w = self.weight
-        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8:
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 8 or self.bias is not None:
             return None
         decode_product = kernels.decode_product_rows(M, w)
         if decode_product:
