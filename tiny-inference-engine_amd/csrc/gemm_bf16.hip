@@ -604,9 +604,11 @@ static bool gemm_dma_takes(const void* x, const void* w, const void* out, int N,
 // Which tile, and how many ranges of K (planes of partial sums that the caller adds), a product takes when
 // left to choose.
 //
-// Up to 64 rows over packed weights: rules measured on the projections of the 1.7B, 8B and 32B shapes; 65 to 128
-// rows: few_rows_us. Above that, for shapes the straight-to-LDS tiles take: the cheapest of (tile, ranges) by an estimate of
-// the time, whose terms were fitted to sweeps over the same shapes at 256 to 2048 rows:
+// Up to 64 rows over packed weights: a score (below); 65 to 128 rows: few_rows_us. Above that, for shapes the
+// straight-to-LDS tiles take: the cheapest of (tile, ranges) by an estimate of the time, whose constants were chosen
+// on sweeps over the projections of four shapes (widths 2048, 3072, 4096 and 5120) at 160 to 2048 rows, every
+// candidate timed with the kernel that consumes its planes, so that the choice lies as close to the best candidate
+// as it can (2.2 % above it on average, 3.6 % with the constants fitted to times of three shapes before):
 //   * a compute unit holds one workgroup (two of the 128 x 128 tile), so the workgroups run in rounds of
 //     256; a round that is nearly empty lasts as long as a full one, which is what a rule by thresholds
 //     gets wrong (768 rows of 256 x 128 tiles over 6144 columns and two ranges: 288 workgroups, two rounds);
@@ -634,16 +636,16 @@ struct DmaTile { int id, bm, bn; float start_us, full_us, slice_us; int per_cu; 
 // for the 256 x 256 and 256 x 192 tiles, whatever the length of K: 256 workgroups of the first start about 11 us
 // later than 192);
 // slice_us: one slice of 32 along K with the compute unit to itself.
-static const DmaTile kDmaTiles[] = {{4, 256, 256, 8.f, 11.f, 0.67f, 1}, {10, 256, 192, 5.f, 6.f, 0.61f, 1},
-                                    {5, 256, 128, 5.f, 0.f, 0.53f, 1}, {6, 128, 256, 5.f, 0.f, 0.50f, 1},
-                                    {7, 128, 128, 4.f, 0.f, 0.36f, 2}};
+static const DmaTile kDmaTiles[] = {{4, 256, 256, 8.8f, 7.9f, 0.67f, 1}, {10, 256, 192, 5.f, 5.4f, 0.55f, 1},
+                                    {5, 256, 128, 6.25f, 0.f, 0.53f, 1}, {6, 128, 256, 6.25f, 1.f, 0.50f, 1},
+                                    {7, 128, 128, 3.24f, 1.f, 0.324f, 2}};
 
 static float estimated_us(const DmaTile& t, int M, int N, int K, int ranges) {
   const long wgs = static_cast<long>((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * ranges;
   const int k_slices = K / GD_BK;
   const int slices = (k_slices + ranges - 1) / ranges;
   const long slots = 256L * t.per_cu;
-  const float pace = t.slice_us * (t.per_cu > 1 && wgs > 256 ? 1.6f : 1.0f);   // two workgroups share the matrix cores
+  const float pace = t.slice_us * (t.per_cu > 1 && wgs > 256 ? 1.94f : 1.0f);   // two workgroups share the matrix cores
   auto round_us = [&](float fill) {
     const float crowded = fminf(fmaxf((fill - 0.75f) * 4.0f, 0.f), 1.f);
     return t.start_us + t.full_us * crowded + slices * pace;
@@ -651,7 +653,7 @@ static float estimated_us(const DmaTile& t, int M, int N, int K, int ranges) {
   float us = static_cast<float>(wgs / slots) * round_us(1.0f);
   if (wgs % slots) us += round_us(static_cast<float>(wgs % slots) / slots);
   const float plane_mb = static_cast<float>(M) * N * 4e-6f;
-  return us + ranges * plane_mb * (1.0f / 6.0f + 1.0f / 5.0f);   // written here, read by the consumer: MB / (TB/s) = us
+  return ranges > 1 ? us + ranges * plane_mb * 0.2f : us;   // planes written here, read by the consumer: MB / (TB/s) = us
 }
 
 // 65 to 128 rows: a workgroup's pace is set by the bytes it loads a slice of 32 along K, its rows of x and its
