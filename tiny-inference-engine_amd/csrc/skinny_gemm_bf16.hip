@@ -13,8 +13,11 @@
 //
 // With splits > 1 the output is [splits, M, N] float32 partial sums, one plane per range of K, for
 // the consumer to add up in plane order (no atomics, no fences: the result is the same in every
-// run). How K is cut depends on K and splits alone, never on M or RT, so a row's sums are formed in
-// the same order whatever else is in the batch.
+// run). How K is cut depends on K, splits and the waves of a workgroup, never on RT or on which rows
+// are present; up to 16 rows the caller's splits follow from the weight's shape alone, so a row's sums
+// are formed in the same order whatever else is in the batch. From 17 rows on the plan (few_rows_plan)
+// may name other ranges for another number of rows: between steps of such sizes a row's sums differ
+// by rounding, as they do between this product and the tiled one.
 //
 // Requires K % 8 == 0 (16-byte loads); other shapes go to the generic kernel.
 //
@@ -24,7 +27,8 @@
 // row and 16-column tile, the sum of the squares of the new x; the products that read those rows multiply their
 // sums by 1 / sqrt(sum of the squares / n + eps), the factor that was left out (every workgroup adds the
 // tiles' squares in the same fixed order), which commutes with the product. Sums of squares, the factor and
-// the stream stay float32.
+// the stream stay float32. Not cut along K, a narrow output would leave such a product one workgroup of four
+// waves a compute unit; it runs in workgroups of sixteen waves over one tile, or eight over two (producer_shape).
 //
 // PACKED: w is stored as [N/16][K/32] blocks of 1 KB, block (t, b) holding rows 16 t .. 16 t + 15 over
 // k = 32 b .. 32 b + 31 in the order the matrix core takes them: lane l's 16 bytes (row l % 16, k-chunk
