@@ -37,6 +37,10 @@ SHAPES = {
     "dh256": (config(1, 64, 2, 1, 256, 96, 130), 32, [1, 50, 64, 140]),
     "dh96_dh112": (config(1, 88, 6, 3, 96, 104, 211), 8, [7, 70, 129]),
     "block_of_12": (config(1, 64, 4, 2, 32, 72, 90), 12, [5, 40, 100]),       # no power of two: generic attention
+    # five and eight query heads a KV head (the 14B and 32B models' grouping): the prefill kernel takes a group in two
+    # passes of four heads, the decode kernel's matrix columns hold five or eight of sixteen
+    "five_per_group_dh128": (config(2, 160, 10, 2, 128, 224, 300, theta=1e6), 16, [3, 40, 129, 200]),
+    "eight_per_group_dh64": (config(1, 128, 16, 2, 64, 160, 257), 16, [6, 65, 130]),
 }
 
 
