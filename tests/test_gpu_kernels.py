@@ -1123,7 +1123,8 @@ def test_random_weights_are_the_same_bits_on_the_gpu_and_on_the_host():
         assert torch.equal(on_gpu[name].cpu().float(), t.float()), name
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (3, 4096, 4096), (8, 96, 12288), (16, 1024, 160)])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (3, 4096, 4096), (8, 96, 12288), (16, 1024, 160), (16, 8192, 128),
+                                   (7, 5200, 96)])
 @pytest.mark.parametrize("packed", [True, False])
 def test_decode_product_with_the_norms_work_in_its_epilogue(M, N, K, packed):
     """The product that ends a sub-layer adds to the stream in place and leaves bf16(stream * weight) and the sums
