@@ -1192,3 +1192,59 @@ def test_decode_product_with_the_norms_work_in_its_epilogue(M, N, K, packed):
     with pytest.raises(kernels.InvalidArgument):
         kernels.skinny_gemm_bf16(rnd(17, K, dtype=torch.bfloat16).cuda(), weight, torch.empty(17, N, device="cuda"),
                                  row_scale=scale)
+
+
+@pytest.mark.parametrize("Dh,bs,planes", [(128, 16, 1), (64, 8, 2), (256, 32, 1), (32, 16, 4), (128, 4, 1)])
+@pytest.mark.parametrize("cache_dtype", [torch.bfloat16, torch.float16])
+def test_values_of_a_portion_reach_the_cache_in_pieces_of_eight_tokens(Dh, bs, planes, cache_dtype):
+    """From 32 rows on the values are stored by a kernel that takes eight consecutive rows of a dimension at once
+    where their slots are eight consecutive, aligned positions of one page, and one by one elsewhere: runs that
+    start inside a page, a sequence that ends in the middle of a group, scattered single slots. The same bits as
+    the rows written a few at a time (the kernel that writes a token a workgroup), and the plain transposition."""
+    from tie_amd import kernels
+
+    H, KVH, eps = 4, 2, 1e-6
+    NB = 40
+    rng = np.random.RandomState(5)
+    # rows of the step: a run aligned to a page, a run that starts at position 3 of a page, scattered slots, and a
+    # run that ends 5 rows into a group
+    pages = rng.permutation(NB)
+    runs = []
+    runs += [pages[0] * bs + i for i in range(min(bs, 24))] + [pages[1] * bs + i for i in range(bs)]
+    runs += [pages[2] * bs + 3 + i for i in range(bs - 3)] + [pages[3] * bs + i for i in range(bs)]
+    runs += [int(pages[4 + i] * bs + rng.randint(bs)) for i in range(9)]
+    runs += [pages[20] * bs + i for i in range(min(bs, 13))]
+    while len(runs) < 40:
+        runs.append(int(pages[21 + len(runs) % 10] * bs + len(runs) % bs))
+    assert len(set(runs)) == len(runs)
+    T = len(runs)
+    width = (H + 2 * KVH) * Dh
+    qkv = rnd(planes, T, width, seed=61).cuda()
+    summed = qkv[0].clone()
+    for p in range(1, planes):
+        summed = summed + qkv[p]
+    qw, kw = (1 + 0.1 * rnd(Dh, seed=62)).cuda(), (1 + 0.1 * rnd(Dh, seed=63)).cuda()
+    inv_freq = torch.from_numpy(plain.rope_inv_freq(1e4, Dh)).cuda()
+    positions, slots = i32(list(range(T))), i32(runs)
+    q_dtype = torch.bfloat16 if cache_dtype == torch.bfloat16 else torch.float32
+    x = qkv if q_dtype == torch.float32 else qkv        # float32 sums either way
+
+    def run(rows):
+        kc = torch.zeros(NB, KVH, bs, Dh, device="cuda", dtype=cache_dtype)
+        vc = torch.zeros(NB, KVH, Dh, bs, device="cuda", dtype=cache_dtype)
+        q = torch.empty(T, H * Dh, device="cuda", dtype=q_dtype)
+        for first in range(0, T, rows):
+            n = min(rows, T - first)
+            kernels.qk_norm_rope_kv_write(x[0, first:first + n], q[first:first + n], qw, kw, eps, inv_freq,
+                                          positions[first:first + n], slots[first:first + n], kc, vc, H, KVH, Dh, bs,
+                                          planes=planes, plane_stride=T * width)
+        return q, kc, vc
+
+    q_all, k_all, v_all = run(T)            # one call: 40 rows or more, the values by the kernel of their own
+    q_few, k_few, v_few = run(7)            # a few rows a call: the kernel that writes a token a workgroup
+    assert torch.equal(q_all, q_few) and torch.equal(k_all, k_few)
+    assert torch.equal(v_all, v_few), "the values differ between the two ways of writing them"
+    want = summed[:, (H + KVH) * Dh:].view(T, KVH, Dh).cpu()
+    for t, slot in enumerate(runs):
+        assert torch.equal(v_all[slot // bs, :, :, slot % bs].cpu(), want[t].to(cache_dtype)), f"row {t}, slot {slot}"
+    assert int((v_all != 0).sum()) <= T * KVH * Dh          # nothing written beside the rows' slots

@@ -549,6 +549,55 @@ __global__ void qk_norm_rope_kv_write_kernel(const TX* qkv, TQ* q_out, const flo
   }
 }
 
+// The values of a portion of tokens into the cache, eight tokens at a time. A page holds a value head transposed
+// (one row of block_size positions per dimension), so the kernel above, a token a workgroup, writes 2 bytes here
+// and 2 bytes there: 2048 tokens of an 8B layer took 13 us for 8 MB. Here (extra workgroups of the same launch) a thread takes one dimension of eight
+// consecutive rows of the step; where their slots are eight consecutive positions of one page, starting at a
+// multiple of eight (a portion of a prompt nearly everywhere), it stores them as one 16-byte piece, else one by
+// one. The same conversions, the same bits. Caches of 2-byte elements, pages of a multiple of 8 positions.
+#define VROWS_THREADS 256
+#define VROWS_TOKENS 8
+
+template <typename TX, typename TC>
+__device__ __forceinline__ void v_write_rows(const TX* __restrict__ qkv, const int* __restrict__ slots,
+                                             TC* __restrict__ v_cache, int T, int KVH, int Dh, int block_size,
+                                             int in_row, int v_offset, size_t plane_stride, int planes, int head,
+                                             int block_of_groups) {
+  static_assert(sizeof(TC) == 2, "eight elements are one 16-byte piece");
+  const int groups_a_workgroup = Dh >= VROWS_THREADS ? 1 : VROWS_THREADS / Dh;
+  const int group = block_of_groups * groups_a_workgroup + (Dh >= VROWS_THREADS ? 0 : threadIdx.x / Dh);
+  const int t0 = group * VROWS_TOKENS;
+  if (t0 >= T) return;
+  const int n = min(VROWS_TOKENS, T - t0);
+  int slot[VROWS_TOKENS];
+#pragma unroll
+  for (int i = 0; i < VROWS_TOKENS; ++i) slot[i] = slots[min(t0 + i, T - 1)];
+  bool together = n == VROWS_TOKENS && slot[0] % VROWS_TOKENS == 0;
+#pragma unroll
+  for (int i = 1; i < VROWS_TOKENS; ++i) together = together && slot[i] == slot[0] + i;
+  for (int d = Dh >= VROWS_THREADS ? threadIdx.x : threadIdx.x % Dh; d < Dh; d += VROWS_THREADS) {
+    const TX* in = qkv + static_cast<size_t>(t0) * in_row + v_offset + static_cast<size_t>(head) * Dh + d;
+    float v[VROWS_TOKENS];
+#pragma unroll
+    for (int i = 0; i < VROWS_TOKENS; ++i)
+      v[i] = i < n ? load_planes(in + static_cast<size_t>(i) * in_row, plane_stride, planes) : 0.f;
+    if (together) {
+      TC* dst = v_cache + (static_cast<size_t>(slot[0] / block_size) * KVH + head) * Dh * block_size +
+                static_cast<size_t>(d) * block_size + slot[0] % block_size;
+      TC piece[VROWS_TOKENS];
+#pragma unroll
+      for (int i = 0; i < VROWS_TOKENS; ++i) store_from_float(piece + i, v[i]);
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(piece);
+    } else {
+      for (int i = 0; i < n; ++i) {
+        TC* dst = v_cache + (static_cast<size_t>(slot[i] / block_size) * KVH + head) * Dh * block_size +
+                  static_cast<size_t>(d) * block_size + slot[i] % block_size;
+        store_from_float(dst, v[i]);
+      }
+    }
+  }
+}
+
 // The same for head sizes of 32, 64, 128, 256 or 512: a lane takes 4 consecutive elements of a head's
 // first half and the 4 they pair with in the second (16-byte loads and stores where the one-wave-a-head
 // kernel above moves 4 and 2 bytes), head_dim / 8 lanes share a head, four waves of heads a workgroup.
@@ -560,10 +609,22 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
     const TX* qkv, TQ* q_out, const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
     const float* __restrict__ inv_freq, const float* __restrict__ angles, const int* __restrict__ positions,
     const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache, TQ* k_dense, int H, int KVH,
-    int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads) {
+    int block_size, int in_row, int q_row, int k_row, size_t plane_stride, int planes, int heads, int tokens,
+    int blocks_a_token) {
   constexpr int Dh = LPH * 8, half = LPH * 4;
-  const int t = blockIdx.y;
-  const int slot_index = blockIdx.x * (QK4_THREADS / LPH) + threadIdx.x / LPH;
+  // Workgroups 0 .. T x blocks_a_token - 1 take the heads of a token; those behind them, where there are any, the
+  // values of groups of tokens (v_write_rows), KVH of them a block of groups.
+  const int qk_blocks = tokens * blocks_a_token;
+  if (static_cast<int>(blockIdx.x) >= qk_blocks) {
+    if constexpr (sizeof(TC) == 2) {
+      const int b = blockIdx.x - qk_blocks;
+      v_write_rows<TX, TC>(qkv, slots, v_cache, tokens, KVH, Dh, block_size, in_row, (H + KVH) * Dh, plane_stride, planes,
+                           b % KVH, b / KVH);
+    }
+    return;
+  }
+  const int t = blockIdx.x / blocks_a_token;
+  const int slot_index = (blockIdx.x % blocks_a_token) * (QK4_THREADS / LPH) + threadIdx.x / LPH;
   const int p0 = (threadIdx.x % LPH) * 4;
   if (slot_index >= heads) return;             // whole heads leave: the shuffles below stay inside a head
   const TX* in = qkv + static_cast<size_t>(t) * in_row + static_cast<size_t>(slot_index) * Dh;
@@ -671,12 +732,24 @@ extern "C" int tie_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_
                     reinterpret_cast<uintptr_t>(k_w) % 16 == 0;
   if (wide) {
     const int lph = Dh / 8;
-    const dim3 grid4((heads + QK4_THREADS / lph - 1) / (QK4_THREADS / lph), T);
+    // From 32 rows on the values go by workgroups of their own that store eight tokens of a dimension at once.
+    const bool values_apart = write_kv && T >= 32 && block_size % VROWS_TOKENS == 0 && cache_dtype != TIE_F32 &&
+                              reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+    const int heads_here = values_apart ? heads - KVH : heads;
+    const int blocks_a_token = (heads_here + QK4_THREADS / lph - 1) / (QK4_THREADS / lph);
+    long blocks = static_cast<long>(T) * blocks_a_token;
+    if (values_apart) {
+      const int groups = (T + VROWS_TOKENS - 1) / VROWS_TOKENS;
+      const int groups_a_workgroup = Dh >= VROWS_THREADS ? 1 : VROWS_THREADS / Dh;
+      blocks += static_cast<long>(KVH) * ((groups + groups_a_workgroup - 1) / groups_a_workgroup);
+    }
+    if (blocks > 0x7fffffffL) return TIE_BAD_ARGUMENT;
+    const dim3 grid4(static_cast<unsigned>(blocks));
 #define LAUNCH4_L(TX, TQ, TC, LPH)                                                                            \
   qk_norm_rope_kv_write4_kernel<TX, TQ, TC, LPH><<<grid4, QK4_THREADS, 0, stream>>>(                          \
       static_cast<const TX*>(qkv), static_cast<TQ*>(q_out), q_w, k_w, eps, inv_freq, angles, positions, slots, \
       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), static_cast<TQ*>(k_dense), H, KVH, block_size,   \
-      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads)
+      in_row, q_row, k_row, static_cast<size_t>(plane_stride), planes, heads_here, T, blocks_a_token)
 #define LAUNCH4(TX, TQ, TC)                         \
   {                                                 \
     if (lph == 4) LAUNCH4_L(TX, TQ, TC, 4);         \
