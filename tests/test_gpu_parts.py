@@ -664,3 +664,103 @@ def test_the_toy_architecture_in_bfloat16_with_recorded_decode_steps(tmp_path, k
     finally:
         unregister_architecture("ToyStateLM")
         unregister_toy_parts()
+
+
+# ------------------------------------------------------------------ a norm and an arrangement of other kinds
+@pytest.mark.parametrize("dtype,tolerance", [("float32", tolerances.FLOAT32), ("bfloat16", tolerances.BFLOAT16["toy architecture"])])
+def test_a_toy_norm_and_a_toy_arrangement_registered_from_outside(dtype, tolerance):
+    """A layer norm with a bias (mean and variance: not of the form the products' epilogues can finish) and an
+    arrangement with one norm and a parallel residual, ``x += mixer(norm(x)) + feed_forward(norm(x))``, both
+    written here with torch operations and without a word about owed sums, pending products, row scales or
+    recording: the framework's attention and SwiGLU parts run inside them, the debts are settled before the
+    foreign norm reads the stream, and every step stays eager. Against plain formulas, in every way of cutting."""
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.models import LayerCall, LayerSpec, Model, ModelSpec
+    from tie_amd.parts import PartSpec, register_part, unregister_part
+    from tie_amd.parts.base import Block, Norm, TensorSpec
+    from tie_amd.weights.random_init import random_tensors
+    from tie_amd.weights.safetensors_io import StoredTensor
+
+    @register_part("norm", "toy_layer_norm")
+    class ToyLayerNorm(Norm):
+        def __init__(self, params):
+            super().__init__(params)
+            self.dim, self.eps = int(params["dim"]), float(params["eps"])
+            self.names = (params["weight"], params["bias"])
+
+        def tensors(self):
+            return [TensorSpec(self.names[0], (self.dim,), "vector", ("one_plus_uniform", 0.1)),
+                    TensorSpec(self.names[1], (self.dim,), "vector", ("normal", 0.1))]
+
+        def load(self, fetch, mode, device):
+            self.weight, self.bias = fetch(self.names[0], "vector"), fetch(self.names[1], "vector")
+
+        def forward(self, ctx, x, rows=None, out_name="norm.out", out_dtype=None):
+            src = x if rows is None else x.index_select(0, rows.long())
+            y = torch.nn.functional.layer_norm(src.float(), (self.dim,), self.weight, self.bias, self.eps)
+            return y.to(out_dtype or ctx.act_dtype)
+
+    @register_part("block", "toy_parallel")
+    class ToyParallelBlock(Block):
+        def forward(self, ctx, x, layer, cache):
+            h = self.normed(ctx, layer.norms["only"], x, consumer=None)
+            layer.mixer.forward(ctx, h, cache, x)
+            layer.feed_forward.forward(ctx, h, x)
+
+    try:
+        D, H, KVH, Dh, I, V, eps, L = 96, 6, 2, 32, 160, 211, 1e-5, 3
+        norm = lambda w, b: PartSpec("toy_layer_norm", {"dim": D, "eps": eps, "weight": w, "bias": b})
+        layers = []
+        for l in range(L):
+            p = f"layers.{l}."
+            mixer = PartSpec("paged_attention", {
+                "hidden": D, "num_heads": H, "num_kv_heads": KVH, "head_dim": Dh, "scale": Dh ** -0.5, "window": None,
+                "qk_norm": None, "position": PartSpec("rope_neox", {"head_dim": Dh, "theta": 10000.0}),
+                "names": {"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}})
+            ffn = PartSpec("swiglu", {"hidden": D, "intermediate": I, "names": {"gate": p + "gate", "up": p + "up", "down": p + "down"}})
+            layers.append(LayerSpec(PartSpec("toy_parallel"), mixer, ffn, {"only": norm(p + "ln.w", p + "ln.b")}))
+        spec = ModelSpec("ToyParallelLM", V, D, 256, PartSpec("token_embedding", {"vocab": V, "hidden": D, "weight": "embed"}),
+                         tuple(layers), tuple(LayerCall(l) for l in range(L)),
+                         PartSpec("lm_head", {"vocab": V, "hidden": D, "norm": norm("final.w", "final.b"), "weight": "head",
+                                              "tied_to": None}))
+        model = Model(spec)
+        assert not model.capturable()                     # the toy parts declare nothing: no step is recorded
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        tensors = dict(random_tensors(model.expected_tensors(), 4, store, vector_dtype=torch.float32))
+        model.load({n: StoredTensor.from_tensor(n, t) for n, t in tensors.items()}, dtype, "cuda:0")
+        w = {n: t.to(F64) for n, t in tensors.items()}
+
+        def layer_norm(x, weight, bias):
+            mean = x.mean(-1, keepdim=True)
+            var = ((x - mean) ** 2).mean(-1, keepdim=True)
+            return (x - mean) / torch.sqrt(var + eps) * weight + bias
+
+        def forward(tokens):
+            T = len(tokens)
+            pos = list(range(T))
+            x = plain.embed(w["embed"], tokens)
+            for l in range(L):
+                p = f"layers.{l}."
+                h = layer_norm(x, w[p + "ln.w"], w[p + "ln.b"])
+                q = plain.rope_neox(plain.linear(h, w[p + "q"]).view(T, H, Dh), pos, 10000.0)
+                k = plain.rope_neox(plain.linear(h, w[p + "k"]).view(T, KVH, Dh), pos, 10000.0)
+                v = plain.linear(h, w[p + "v"]).view(T, KVH, Dh)
+                a = plain.causal_attention(q, k, v, Dh ** -0.5).reshape(T, H * Dh)
+                x = x + plain.linear(a, w[p + "o"]) + plain.swiglu(h, w[p + "gate"], w[p + "up"], w[p + "down"])
+            return plain.linear(layer_norm(x, w["final.w"], w["final.b"]), w["head"])
+
+        requests = th.make_requests(V, [45, 70, 33, 9], seed=12)
+        want = {rid: forward(toks).float() for rid, toks in requests.items()}
+        steps, peak = th.mixed(requests, max_live=3, seed=4)
+        for label, trace, room in (("whole", th.whole(requests), 256), ("prefill + decode", th.prefill_then_decode(requests), 256),
+                                   ("portions", th.portions(requests), 256), ("mixed", steps, peak)):
+            replayer = TraceReplayer(model, room, block_size=16)
+            got = th.collect(replayer, trace)
+            for rid, ref in want.items():
+                mine = torch.stack([got[rid][p] for p in range(ref.shape[0])])
+                close(mine, ref, tolerance, f"toy norm and arrangement, {label}, request {rid}")
+            assert replayer.cache.num_free() == replayer.cache.num_blocks
+            assert replayer.runner.graph_replays == 0
+    finally:
+        unregister_part("norm", "toy_layer_norm")
+        unregister_part("block", "toy_parallel")
