@@ -342,6 +342,43 @@ def test_a_projection_with_a_bias_alone():
         kernels.add_bias(torch.zeros(T, D, device="cuda"), torch.zeros(D + 1, device="cuda"))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_a_mixer_alone_and_of_a_feed_forward_alone(tmp_path, dtype):
+    """A layer may hold a mixer without a feed-forward or the other way round (an architecture that interleaves
+    them otherwise than in pairs; two mixers with caches of their own in what another framework calls one layer).
+    Qwen3's layers cut into such halves, twice as many entries in the run order, are the same model: the same
+    bits as the whole layers give, through a mixed trace with pages used again."""
+    from tie_amd.engine.replay import TraceReplayer
+    from tie_amd.models import LayerCall, LayerSpec, Model
+    from tie_amd.weights.loader import load_model_folder
+    from tie_amd.weights.random_init import write_random_model
+
+    whole, cfg = attention_model(((0, None), (1, None), (2, None)), layers=3)
+    halves = []
+    for layer in whole.spec.layers:
+        halves.append(LayerSpec(layer.block, layer.mixer, None, {"pre_mixer": layer.norms["pre_mixer"]}))
+        halves.append(LayerSpec(layer.block, None, layer.feed_forward, {"pre_feed_forward": layer.norms["pre_feed_forward"]}))
+    cut = Model(dataclasses.replace(whole.spec, layers=tuple(halves), order=tuple(LayerCall(i) for i in range(6))))
+    assert [g.num_planes for g in cut.cache_plan.groups] == [3]          # the halves without a mixer need no cache
+    with pytest.raises(Exception, match="pre_mixer"):
+        Model(dataclasses.replace(whole.spec, layers=(LayerSpec(whole.spec.layers[0].block, whole.spec.layers[0].mixer, None, {}),),
+                                  order=(LayerCall(0),)))
+    folder = write_random_model(tmp_path / "m", cfg, seed=5, dtype=dtype)
+    files = load_model_folder(folder)
+    whole.load(files.tensors, dtype, "cuda:0")
+    cut.load(files.tensors, dtype, "cuda:0")
+    requests = th.make_requests(cfg["vocab_size"], [45, 70, 33, 12], seed=10)
+    steps, peak = th.mixed(requests, max_live=3, seed=6)
+    got = {}
+    for name, model in (("whole", whole), ("cut", cut)):
+        replayer = TraceReplayer(model, peak, block_size=16)
+        got[name] = th.collect(replayer, steps)
+        assert replayer.cache.num_free() == replayer.cache.num_blocks
+    for rid in requests:
+        for p in got["whole"][rid]:
+            assert torch.equal(got["whole"][rid][p], got["cut"][rid][p]), f"request {rid}, position {p}"
+
+
 # ------------------------------------------------------------------ toy parts, defined and registered here
 def register_toy_parts():
     from tie_amd import kernels

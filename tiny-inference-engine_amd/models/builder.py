@@ -95,15 +95,19 @@ class _Launch:
 class LayerParts:
     def __init__(self, spec):
         self.block = build_part("block", spec.block)
-        self.mixer = build_part("mixer", spec.mixer)
-        self.feed_forward = build_part("feed_forward", spec.feed_forward)
+        self.mixer = build_part("mixer", spec.mixer) if spec.mixer is not None else None
+        self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
         self.norms = {name: build_part("norm", s) for name, s in spec.norms.items()}
-        check = getattr(self.block, "check", None)
+        check = getattr(self.block, "check_layer", None)
         if check is not None:
-            check(self.norms)
+            check(self)
+        else:
+            check = getattr(self.block, "check", None)
+            if check is not None:
+                check(self.norms)
 
     def parts(self):
-        return [self.block, self.mixer, self.feed_forward, *self.norms.values()]
+        return [p for p in (self.block, self.mixer, self.feed_forward, *self.norms.values()) if p is not None]
 
 
 class Model:
@@ -115,7 +119,8 @@ class Model:
         self.layers: List[LayerParts] = [LayerParts(s) for s in spec.layers]
         self.head = build_part("head", spec.head)
         self.cache_plan: CachePlan = plan_cache(
-            [self.layers[c.layer].mixer.cache_need() for c in spec.order],
+            [self.layers[c.layer].mixer.cache_need() if self.layers[c.layer].mixer is not None else None
+             for c in spec.order],
             [c.reads_cache_of for c in spec.order])
         self.mode: Optional[str] = None
         self.device = None

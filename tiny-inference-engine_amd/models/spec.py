@@ -19,11 +19,16 @@ from ..parts.base import PartSpec
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    """One layer: an arrangement (block) of a mixer, a feed-forward and their norms."""
+    """One layer: an arrangement (block) of a mixer, a feed-forward and their norms.
+
+    Either part may be None: a layer of a mixer alone or of a feed-forward alone, for architectures that
+    interleave them otherwise than in pairs, or whose layers would need two mixers with caches of their own
+    (two entries of the run order, the second without a feed-forward). The arrangement says what it needs.
+    """
 
     block: PartSpec
-    mixer: PartSpec
-    feed_forward: PartSpec
+    mixer: Optional[PartSpec]
+    feed_forward: Optional[PartSpec]
     norms: Mapping[str, PartSpec] = dataclasses.field(default_factory=dict)
 
 
