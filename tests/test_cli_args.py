@@ -23,8 +23,9 @@ def test_every_option_is_read():
                              "--seed", "9", "--max-tokens", "12", "--kv-mem", "512M", "--stop-ids", "2,3",
                              "--dtype", "float32", "--block-size", "4", "--kv-blocks", "40", "--max-seqs", "8",
                              "--max-tokens-per-step", "64", "--prefill-chunk", "13", "--policy", "fcfs",
-                             "--aging", "2", "--device", "hip", "--threads", "4", "--kv-dtype", "float16"])
+                             "--aging", "2", "--device", "hip", "--threads", "4", "--kv-dtype", "float16", "--admit-whole"])
     assert o.kv_dtype == "float16" and parse_generate_args(["-m", "m", "-p", "7"]).kv_dtype is None
+    assert o.admit_whole and not parse_generate_args(["-m", "m", "-p", "7"]).admit_whole
     assert o.sampling.temperature == 0.0 and o.sampling.top_k == 5 and o.sampling.top_p == 0.5
     assert o.sampling.seed == 9 and o.sampling.max_tokens == 12 and o.kv_bytes == 512 << 20
     assert o.stop_ids == [2, 3] and o.dtype == "float32" and o.block_size == 4 and o.kv_blocks == 40

@@ -20,8 +20,9 @@ from tie_amd.sampling.params import SamplingParams
 PLAN = plan_cache([PagedKV(1, 8)], [None])
 
 
-def config(max_tokens_per_step, max_seqs, policy=FCFS, watermark=0, aging=16, prefill_chunk=0):
-    return SchedulerConfig(ServingConfig(max_tokens_per_step, max_seqs, prefill_chunk), policy, aging, watermark)
+def config(max_tokens_per_step, max_seqs, policy=FCFS, watermark=0, aging=16, prefill_chunk=0, admit_whole=False):
+    return SchedulerConfig(ServingConfig(max_tokens_per_step, max_seqs, prefill_chunk), policy, aging, watermark,
+                           admit_whole)
 
 
 class Fixture:
@@ -107,6 +108,29 @@ def test_watermark_stays_free_and_admission_stops_at_a_head_that_does_not_fit():
     s = f.run()                                             # a's decode takes a 5th page, 3 free
     assert (s.tokens_of(a), s.tokens_of(b), s.tokens_of(c)) == (1, 0, 0)
     assert b.state == SeqState.WAITING and c.state == SeqState.WAITING
+
+
+@pytest.mark.parametrize("admit_whole", [False, True])
+def test_admission_by_the_first_portion_or_by_the_whole_pending_input(admit_whole):
+    """Not in the reference, whose admission counts the first portion (src/engine/batch_scheduler.cpp:143-146)."""
+    f = Fixture(8, config(8, 4, FCFS, watermark=0, prefill_chunk=8, admit_whole=admit_whole))
+    a = f.add(8)
+    assert f.run().tokens_of(a) == 8                        # 2 pages, 6 free
+    b = f.add(28)                                           # 7 pages in all, 2 for what the budget leaves this step
+    s = f.run()                                             # a's decode takes a 3rd page
+    assert s.tokens_of(a) == 1
+    if admit_whole:
+        assert s.tokens_of(b) == 0 and b.state == SeqState.WAITING and f.sched.num_preemptions == 0
+        f.finish(a)
+        assert f.run().tokens_of(b) == 8                    # the pool is b's alone now
+        while b.num_pending > 1:
+            f.run()
+        assert f.sched.num_preemptions == 0
+    else:
+        assert s.tokens_of(b) == 7 and b.state == SeqState.PREFILLING
+        for _ in range(8):
+            f.run()                                         # b's portions fill the pool; a's next page evicts b
+        assert f.sched.num_preemptions >= 1 and b.num_preemptions >= 1
 
 
 def test_the_head_is_admitted_past_the_watermark_when_nothing_runs():
@@ -292,7 +316,8 @@ def test_randomized_everything_finishes_and_no_page_is_shared_or_lost(seed):
     pool_tokens = blocks * 4
     budget = rng.randint(4, 32)
     cfg = config(budget, rng.randint(1, min(8, budget)), FCFS if seed % 2 else SRPT_AGING,
-                 rng.randint(-1, blocks - 1), rng.randint(0, 8), prefill_chunk=rng.choice([0, 0, 3, 7]))
+                 rng.randint(-1, blocks - 1), rng.randint(0, 8), prefill_chunk=rng.choice([0, 0, 3, 7]),
+                 admit_whole=seed % 3 == 0)
     f = Fixture(blocks, cfg)
     requests = []
     for _ in range(rng.randint(1, 20)):

@@ -25,7 +25,7 @@ DEFAULT_KV_BYTES = 4 << 30  # the reference's default KV budget (src/cli/args.h:
 
 def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, kv_blocks: Optional[int] = None,
                   block_size: int = 16, max_seqs: int = 64, max_tokens_per_step: int = 512, prefill_chunk: int = 0,
-                  policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1,
+                  policy: str = "srpt-aging", aging: int = 16, watermark_blocks: int = -1, admit_whole: bool = False,
                   stop_tokens: Sequence[int] = (), max_seq_len: Optional[int] = None,
                   device: str = "cuda:0", use_graphs: Optional[bool] = None, launch_ahead=True,
                   kv_dtype: Optional[str] = None) -> Engine:
@@ -51,7 +51,7 @@ def create_engine(model, dtype: str = "bfloat16", kv_mem: Optional[int] = None, 
                          step_tokens=prefill_chunk or max_tokens_per_step)
     serving = ServingConfig(max_tokens_per_step=max_tokens_per_step, max_seqs=max_seqs, prefill_chunk=prefill_chunk)
     scheduler = BatchScheduler(cache, SchedulerConfig(serving=serving, policy=policy, aging=aging,
-                                                      watermark_blocks=watermark_blocks))
+                                                      watermark_blocks=watermark_blocks, admit_whole=admit_whole))
     return Engine(model, cache, scheduler, serving, stop_tokens=stop_tokens, max_seq_len=max_seq_len,
                   use_graphs=use_graphs, launch_ahead=launch_ahead)
 

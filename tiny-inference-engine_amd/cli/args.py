@@ -50,9 +50,11 @@ generate options:
   --prefill-chunk C        most prompt tokens of one sequence per step, 0 = budget only (default 0)
   --policy fcfs|srpt-aging admission order (default srpt-aging)
   --aging N                srpt-aging priority gained per step waited, in tokens (default 16)
+  --admit-whole            a request enters when the cache can hold all of its pending input, not just its first
+                           portion (not in the reference: fewer evictions when the cache is scarce)
 
 bench options (and -m, --device, --dtype, --kv-dtype, --temp (default 0), --top-k, --top-p, --seed, --kv-mem, --kv-blocks,
---block-size, --max-seqs, --max-tokens-per-step, --prefill-chunk, --policy, --aging as above; --seed also seeds
+--block-size, --max-seqs, --max-tokens-per-step, --prefill-chunk, --policy, --aging, --admit-whole as above; --seed also seeds
 the synthetic workload and the arrivals):
   --prompts FILE           JSONL, one {"prompt_ids": [...], "max_tokens": N} per line
   --synthetic N            N requests of random tokens
@@ -85,6 +87,7 @@ class GenerateOptions:
     prefill_chunk: int = 0
     policy: str = "srpt-aging"
     aging: int = 16
+    admit_whole: bool = False
 
 
 def parse_int(flag: str, text: str) -> int:
@@ -193,6 +196,8 @@ def _engine_flag(flag: str, flags: _Flags, o) -> bool:
         o.aging = parse_int(flag, flags.value())
         if o.aging < 0:
             raise InvalidArgument(f"--aging must be non-negative, got {o.aging}")
+    elif flag == "--admit-whole":
+        o.admit_whole = True
     elif flag == "--threads":
         parse_int(flag, flags.value())         # CPU threads of the reference's CPU backend: nothing to set here
     else:
@@ -253,6 +258,7 @@ class BenchOptions:
     prefill_chunk: int = 0
     policy: str = "srpt-aging"
     aging: int = 16
+    admit_whole: bool = False
     json: bool = False
 
 

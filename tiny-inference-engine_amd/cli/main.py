@@ -29,7 +29,7 @@ def run_generate(argv: Sequence[str]) -> int:
     engine = create_engine(opt.model, dtype=opt.dtype, kv_dtype=opt.kv_dtype, kv_mem=opt.kv_bytes,
                            kv_blocks=opt.kv_blocks, block_size=opt.block_size, max_seqs=opt.max_seqs,
                            max_tokens_per_step=opt.max_tokens_per_step, prefill_chunk=opt.prefill_chunk,
-                           policy=opt.policy, aging=opt.aging, stop_tokens=opt.stop_ids)
+                           policy=opt.policy, aging=opt.aging, admit_whole=opt.admit_whole, stop_tokens=opt.stop_ids)
     load_seconds = time.perf_counter() - load_start
 
     gen_start = time.perf_counter()
@@ -80,7 +80,7 @@ def run_bench(argv: Sequence[str]) -> int:
     engine = create_engine(opt.model, dtype=opt.dtype, kv_dtype=opt.kv_dtype, kv_mem=opt.kv_bytes,
                            kv_blocks=opt.kv_blocks, block_size=opt.block_size, max_seqs=opt.max_seqs,
                            max_tokens_per_step=opt.max_tokens_per_step, prefill_chunk=opt.prefill_chunk,
-                           policy=opt.policy, aging=opt.aging, launch_ahead=opt.launch_ahead)
+                           policy=opt.policy, aging=opt.aging, admit_whole=opt.admit_whole, launch_ahead=opt.launch_ahead)
     vocab = engine.model.spec.vocab_size
     if opt.synthetic:
         requests = synthetic_requests(opt.synthetic, opt.prompt_len, opt.output_len, vocab, opt.sampling.seed)

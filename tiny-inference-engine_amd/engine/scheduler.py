@@ -17,7 +17,11 @@ A step is planned in rounds, each a method, each spending the same budget:
 ``_admit``             waiting sequences enter in policy order (first come first served, or least
                        remaining work first where a waiting step counts ``aging`` tokens). Admission
                        keeps ``watermark`` pages free for the running ones to grow into and stops at the
-                       first sequence that does not fit: a large request is not overtaken for ever;
+                       first sequence that does not fit: a large request is not overtaken for ever.
+                       What has to fit is the first portion, as in the reference, or with ``admit_whole``
+                       all of the sequence's pending input: a long prompt then enters only when the pool
+                       can hold it, instead of entering on its first portion and being evicted, or evicting
+                       others, on a later one;
 ``_unblock_oldest``    only if all of that produced nothing: the oldest idle running sequence takes
                        pages from newer ones until it can move, so the engine never stalls.
 
@@ -63,6 +67,7 @@ class SchedulerConfig:
     policy: str = SRPT_AGING
     aging: int = 16                # srpt-aging: tokens of priority a sequence gains per step it waits
     watermark_blocks: int = -1     # pages that admission leaves free; -1 picks max(1, 1 % of the pool)
+    admit_whole: bool = False      # admission counts pages for all of a sequence's pending input, not its first portion
 
 
 class Share:
@@ -253,7 +258,8 @@ class BatchScheduler:
             if seq.num_preemptions and seq.waiting_since_step == self._clock:
                 continue                       # evicted while this very step was planned: it waits a step
             n = self._portion(seq, budget)
-            if not self.cache.can_admit(n, self.watermark if self.running else 0):
+            counted = seq.num_pending if self.config.admit_whole else n
+            if not self.cache.can_admit(counted, self.watermark if self.running else 0):
                 break
             seq.state = SeqState.PREFILLING
             self.running.append(seq)
