@@ -188,6 +188,25 @@ def test_requests_batched_together_generate_what_each_generates_alone(model_fold
         assert alone.generate(prompt, params) == together.sequence(sid).generated, f"request {sid}"
 
 
+def test_admission_by_the_whole_pending_input_generates_the_same_tokens_with_fewer_evictions(model_folders):
+    """A scarce pool and prompts in portions of 8: by the first portion (the reference's rule) prompts enter that the
+    pool cannot hold and are evicted on a later portion; by the whole input they wait. The tokens are the same."""
+    folder, cfg = model_folders["A"]
+    reqs = mixed_requests(cfg["vocab_size"], False)
+    evictions, generated = {}, {}
+    for whole in (False, True):
+        engine = make_engine(folder, 4, kv_blocks=12, max_seqs=8, max_tokens_per_step=16, prefill_chunk=8,
+                             policy="fcfs", admit_whole=whole)
+        ids = [engine.add_request(p, s) for p, s in reqs]
+        while engine.has_work():
+            engine.step()
+        assert engine.cache.num_free() == 12
+        evictions[whole] = engine.stats().preemptions
+        generated[whole] = [engine.sequence(sid).generated for sid in ids]
+    assert generated[True] == generated[False]
+    assert evictions[True] < evictions[False]
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_a_crowded_engine_finishes_everything_twice_the_same_way(model_folders, model_folders_bf16, dtype):
     """Thirty requests of mixed lengths and sampling through a small pool: chunked prompts, decode steps
