@@ -86,12 +86,12 @@ class FakeSampler:
         return list(logits)
 
 
-def make_engine(blocks, max_tokens_per_step, max_seqs, policy, launch_ahead, prefill_chunk=0, stop=()):
+def make_engine(blocks, max_tokens_per_step, max_seqs, policy, launch_ahead, prefill_chunk=0, stop=(), admit_whole=False):
     cache = CacheManager(PLAN, block_size=4, num_blocks=blocks, max_state_slots=64)
     serving = ServingConfig(max_tokens_per_step, max_seqs, prefill_chunk)
     model = types.SimpleNamespace(spec=types.SimpleNamespace(max_positions=4096, vocab_size=VOCAB), device="cpu")
     runner = FakeRunner(max_blocks_per_seq=cache.blocks_for(4096))
-    sched = BatchScheduler(cache, SchedulerConfig(serving, policy, 16, 0))
+    sched = BatchScheduler(cache, SchedulerConfig(serving, policy, 16, 0, admit_whole))
     return Engine(model, cache, sched, serving, stop_tokens=stop, launch_ahead=launch_ahead, runner=runner,
                   sampler=FakeSampler())
 
@@ -130,7 +130,7 @@ def test_random_workloads_over_small_pools_lose_nobody(policy, launch_ahead):
         # every other workload has stop tokens: a sequence that meets one has run ahead, and what it ran is dropped
         stop = tuple(rng.sample(range(VOCAB), 6)) if seed % 2 else ()
         engine = make_engine(blocks, rng.randint(4, 12), rng.randint(2, 4), policy, launch_ahead,
-                             prefill_chunk=rng.choice([0, 3, 5]), stop=stop)
+                             prefill_chunk=rng.choice([0, 3, 5]), stop=stop, admit_whole=seed % 5 == 0)
         done = run_all(engine, requests, arrivals)
         for i, (prompt, count) in enumerate(requests):
             assert done[i].state == SeqState.FINISHED
