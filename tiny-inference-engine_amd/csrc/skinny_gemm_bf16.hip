@@ -636,7 +636,10 @@ extern "C" int tie_skinny_gemm_splits(int N, int K) {
 // would. Sixteen waves over one tile where the tiles leave every compute unit at most one workgroup; eight
 // waves over two tiles where pairs of tiles do; else the ordinary four waves. Measured in chains of a layer's
 // four products against the same chain with planes and norm kernels (us a layer, planes | this way):
-//   4096 wide (256 tiles; 2048 and 2560 wide alike): 1 row 73.6 | 67.9, 8 rows 79.9 | 74.4, 16 rows 80.9 | 80.2;
+//   4096 wide (256 tiles): 1 row 73.6 | 67.9, 8 rows 79.2 | 73.9, 10 rows 79.3 | 74.0, 12 rows 79.6 | 76.8,
+//     14 rows 80.0 | 76.9, 16 rows 80.5 | 80.4 (x comes in groups of four rows);
+//   2048 wide (128 tiles): 8 rows 34.6 | 33.3, 10 rows 35.7 | 34.1, 12 rows 35.9 | 35.8, 16 rows 36.9 | 38.0;
+//   2560 wide (160 tiles): 8 rows 53.5 | 53.1, 10 rows 55.4 | 55.2, 12 rows 55.7 | 57.0, 16 rows 58.0 | 62.0;
 //   5120 wide (320 tiles), K of 8192 and 25600: 1 row 166.7 | 159.4, 4 rows 161.9 | 163.8, 8 rows 174.4 | 178.6;
 //   5120 wide, K of 5120 and 17408: 1 row 123.3 | 113.2, 4 rows 119.6 | 117.7, 8 rows 127.8 | 128.9.
 // (One tile and sixteen waves over 320 tiles: 193 us at 8 rows; every workgroup reads all of x.)
@@ -653,7 +656,7 @@ static ProducerShape producer_shape(int N) {
 extern "C" int tie_skinny_norm_epilogue_rows(int N, int K) {
   if (N % 16 != 0 || K % 32 != 0) return 0;
   const int tiles = N / 16, cus = compute_units();
-  if (tiles <= cus) return 8;
+  if (tiles <= cus) return tiles * 4 > cus * 3 ? 14 : 10;
   if (tiles <= 2 * cus) return 4;
   return 0;
 }
