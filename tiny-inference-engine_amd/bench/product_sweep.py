@@ -3,7 +3,7 @@
 For the four projections of a layer shape (QKV, O, gate/up, down) at a list of row counts, every candidate
 the launchers can be forced to - the decode product reading x from memory (1 to 4 weight tiles a
 workgroup, 2 to 8 k-blocks a batch of loads) or sharing it through LDS (3, 6 or 8 tiles a workgroup), the tiled
-product (64-row tiles up to 64 rows, tiles of 64 and 128 rows up to 128, of 128 and 256 rows above), each in 1 to 8
+product (64-row tiles from 17 to 64 rows, tiles of 64 and 128 rows up to 128, of 128 and 256 rows above), each in 1 to 8
 ranges of K - is timed together with what its
 consumer has to do for it (planes: the kernel that adds them to the stream and norms; one plane: accumulate in
 place, then the norm kernel), in a recorded chain over several copies of the weight so that no cache holds it.
@@ -127,7 +127,7 @@ def main(argv=None) -> int:
                         results.append((timed(forced, copies), label))
                     except RuntimeError:
                         pass
-                if M > 32:
+                if M > 16:
                     tiles_tried = ((8, "64 x 256"), (9, "64 x 128")) if M <= 64 else \
                         ((6, "128 x 256"), (7, "128 x 128"), (8, "64 x 256"), (9, "64 x 128")) if M <= 128 else \
                         ((4, "256 x 256"), (10, "256 x 192"), (5, "256 x 128"), (6, "128 x 256"), (7, "128 x 128"))
