@@ -165,8 +165,10 @@ def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True):
                          max_seq_len=context, launch_ahead=launch_ahead)
 
 
-def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=None):
-    """Times ``steps`` decode steps of ``batch`` sequences whose contexts end at (just below) ``context`` tokens.
+def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=None, long_sequences=0,
+                   short_context=0):
+    """Times ``steps`` decode steps of ``batch`` sequences whose contexts end at (just below) ``context`` tokens;
+    with ``long_sequences`` > 0 only that many of them do and the others end at ``short_context``.
 
     The prompts are prefilled through the engine first (untimed). Sequences that finish their prompt
     early decode while the others still prefill, so every prompt is shortened by the number of steps
@@ -185,8 +187,10 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
     rng = random.Random(batch)
     slack = -(-batch * context // chunk) + batch + 2          # steps the prefill phase may take
     prompt_len = context - (steps + warmup) - slack - 1
-    assert prompt_len > 0, "context too short for this many steps"
-    ids = [engine.add_request([rng.randrange(cfg["vocab_size"]) for _ in range(prompt_len)],
+    lengths = [prompt_len if long_sequences <= 0 or i < long_sequences else short_context - (context - prompt_len)
+               for i in range(batch)]
+    assert min(lengths) > 0, "context too short for this many steps"
+    ids = [engine.add_request([rng.randrange(cfg["vocab_size"]) for _ in range(lengths[i])],
                               SamplingParams(max_tokens=steps + warmup + slack + 1, seed=i, **(sampling or {})))
            for i in range(batch)]
     started = time.perf_counter()
@@ -198,7 +202,7 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
             log(f"batch {batch}: prefilling, {done} of {batch} sequences done")
             last_log = time.perf_counter()
     torch.cuda.synchronize()
-    log(f"batch {batch}: prefilled {batch * prompt_len} tokens in {time.perf_counter() - started:.1f} s "
+    log(f"batch {batch}: prefilled {sum(lengths)} tokens in {time.perf_counter() - started:.1f} s "
         f"({engine.stats().steps} steps)")
     for _ in range(warmup):
         engine.step()
@@ -275,6 +279,11 @@ def main():
     parser.add_argument("--temperature", type=float, default=0.0, help="decode: sampling temperature (0 = greedy)")
     parser.add_argument("--top-k", type=int, default=0, help="decode: with a temperature, keep the k most likely (0 = all)")
     parser.add_argument("--top-p", type=float, default=1.0, help="decode: with a temperature, nucleus mass (1 = all)")
+    parser.add_argument("--long-sequences", type=int, default=0,
+                        help="decode: only this many sequences of the batch reach --context, the others --short-context")
+    parser.add_argument("--short-context", type=int, default=1024, help="decode: see --long-sequences")
+    parser.add_argument("--shares-by-sequence", action="store_true",
+                        help="decode: never plan key shares of one length for sequences of very different lengths")
     parser.add_argument("--sweep", action="store_true",
                         help="decode only, one JSON line for every (context, batch) of --sweep-contexts x --sweep-batches")
     parser.add_argument("--sweep-contexts", default="4096,16384,32768")
@@ -340,6 +349,10 @@ def main():
         return 0
 
     chunk = 8192
+    if args.shares_by_sequence:
+        from tie_amd import kernels
+
+        kernels.BALANCED_SHARES_MAX_EQUAL = 0
     sampling = None
     if args.temperature > 0:
         sampling = {"temperature": args.temperature, "top_k": args.top_k, "top_p": args.top_p}
@@ -352,7 +365,8 @@ def main():
     def decode_point(batch, context=None):
         """One decode measurement: ``--steps`` timed steps at ``batch``; the figures of its roofline."""
         seconds, mean_context, replays, median = measure_decode(model, cfg, batch, context or args.context, args.steps,
-                                                                args.warmup, chunk, sampling)
+                                                                args.warmup, chunk, sampling, args.long_sequences,
+                                                                args.short_context)
         ms = seconds / args.steps * 1e3
         step_bytes = weight_bytes_per_step(cfg, batch) + batch * mean_context * kv_bytes_per_token(cfg)
         achieved = step_bytes / (ms * 1e-3) / 1e9
@@ -390,7 +404,8 @@ def main():
             "model": f"{shape_name} shape, random weights", "layers": layers_of_shape, "layers_run": cfg["num_hidden_layers"],
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-            "global_batch": args.batch, "seq_len": args.context, "kv_block": BLOCK_SIZE, "kv_dtype": "bf16",
+            "global_batch": args.batch, "seq_len": args.context, "long_sequences": args.long_sequences,
+            "short_context": args.short_context if args.long_sequences else 0, "kv_block": BLOCK_SIZE, "kv_dtype": "bf16",
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
             "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
         },

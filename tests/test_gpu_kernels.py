@@ -639,6 +639,37 @@ def test_attention_decode_bf16_with_tiles_in_flight(H, KVH, Dh, bs, nsplit, wind
         assert torch.equal(again, first), f"{depth} tiles in flight: other bits than one"
 
 
+@pytest.mark.parametrize("H,KVH,Dh,bs", [(6, 2, 32, 16), (8, 2, 128, 16), (5, 5, 80, 64)])
+@pytest.mark.parametrize("nsplit,share_tiles,window", [(8, 4, None), (8, 7, None), (4, 1, None), (3, 100, None),
+                                                       (8, 3, 200), (2, 0, None)])
+def test_attention_decode_bf16_with_shares_of_one_length(H, KVH, Dh, bs, nsplit, share_tiles, window):
+    """Shares of one length for sequences of very different lengths: a short sequence fills one share and leaves
+    the others empty, a long one fills several; a length too short to cover a sequence (1 tile in 4 shares against
+    32 tiles) falls back to that sequence's own equal shares, one longer than any sequence leaves one share each.
+    Against the plain formula, and the same bits whatever the depth of the ring; the kernel that prepares its own
+    queries takes the same argument."""
+    from tie_amd import kernels
+
+    lens = [1, 33, 64, 129, 300, 1000, 31, 700, 257, 96]
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=[1] * len(lens), lens_ctx=lens, seed=19, dtype=torch.bfloat16,
+                             window=window)
+    length = i32([share_tiles])
+    outs = []
+    for depth in (2, 3, 4):
+        out = torch.full_like(case["q"], float("nan"))
+        part_o = torch.full((S * H * nsplit * Dh,), float("nan"), dtype=torch.float32, device="cuda")
+        part_ml = torch.full((S * H * nsplit * 2,), float("nan"), dtype=torch.float32, device="cuda")
+        kernels.attention_decode_bf16(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                      case["tables"], S, H, Dh ** -0.5, window, nsplit, part_o, part_ml, depth=depth,
+                                      share_tiles=length)
+        outs.append(out)
+    close(outs[0], case["want"], 1e-2, f"decode attention, shares of {share_tiles} tiles in a grid of {nsplit}")
+    assert torch.equal(outs[1], outs[0]) and torch.equal(outs[2], outs[0])
+    with pytest.raises(Exception, match="more than one share"):
+        kernels.attention_decode_bf16(case["q"], case["kc"], case["vc"], out, case["query_start"], case["context_lens"],
+                                      case["tables"], S, H, Dh ** -0.5, window, 1, share_tiles=length)
+
+
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
                                          (16, 1, 64, 4), (2, 1, 256, 32)])
 @pytest.mark.parametrize("nsplit", [1, 3, 8])

@@ -214,6 +214,39 @@ def test_decoding_across_context_buckets_in_bfloat16(long_models, expected, monk
         assert runner.graph_replays == 0 and not runner._recorded
 
 
+@pytest.mark.parametrize("prepares", [True, False])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_shares_of_one_length_while_sequences_of_300_and_4000_keys_decode_together(long_models, expected, monkeypatch,
+                                                                                  name, prepares):
+    """The plan for sequences of very different lengths (one length for all shares, a short sequence filling one of
+    them) is made for steps of many sequences; here the rule by the step's size is bent to two shares a sequence so
+    that four requests meet it: recorded steps and eager ones, the kernel that prepares its queries and the other,
+    while the plan changes from step to step with the lengths."""
+    import tie_amd.engine.batch as batch_module
+    import tie_amd.parts.attention as attention_part
+    from tie_amd import kernels
+    from tie_amd.engine.replay import TraceReplayer
+
+    folder, cfg, _ = long_models[name]
+    tokens, steps, pool, wanted, want = expected[name]
+    monkeypatch.setattr(kernels, "decode_splits", lambda *a, **k: 2)
+    if not prepares:
+        monkeypatch.setattr(attention_part.kernels, "decode_attention_prepares", lambda *a, **k: False)
+    plans = []
+    real = kernels.decode_share_plan
+
+    def watched(*args, **kwargs):
+        plans.append(real(*args, **kwargs))
+        return plans[-1]
+
+    monkeypatch.setattr(batch_module.kernels, "decode_share_plan", watched)
+    replayer = TraceReplayer.from_folder(folder, "bfloat16", pool, block_size=16, use_graphs=True)
+    run_and_compare(replayer, steps, wanted, want, BOUND[name], f"{name}/bfloat16/shares of one length/prepares {prepares}")
+    lengths = {length for shares, length in plans if length > 0}
+    assert len(lengths) >= 2 and all(shares == 8 for shares, length in plans if length > 0), sorted(lengths)
+    assert replayer.runner.graph_replays > 50 and (8,) in {key[3] for key in replayer.runner._recorded}
+
+
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_decoding_across_context_buckets_in_float32(long_models, expected, name):
     from tie_amd.engine.replay import TraceReplayer

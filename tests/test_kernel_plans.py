@@ -197,3 +197,32 @@ def test_the_decode_products_plan_for_17_to_64_rows():
             assert ranges in (1, 2, 4, 8) and (ranges == 1 or K // ranges >= 512)
             assert kernels.gemm_tile(M, N, K, True) == kernels.gemm_tile(M, N, K, True, ranges) in (8, 9)
     assert kernels.gemm_tile(64, 51200, 5120, True, 1) == 8 and kernels.gemm_tile(64, 151936, 4096, True, 1) == 8
+
+
+def test_shares_of_one_length_are_planned_for_sequences_of_very_different_lengths():
+    import random
+
+    from tie_amd import kernels
+
+    rng = random.Random(0)
+    assert kernels.decode_share_plan([2048] * 32, 8, 4096) == (kernels.decode_splits(32, 8, 4096), 0)
+    assert kernels.decode_share_plan([4000, 3900, 4096] * 11, 8, 4096)[1] == 0          # about one length
+    assert kernels.decode_share_plan([100, 4000], 8, 4096) == (kernels.decode_splits(2, 8, 4096), 0)   # many shares anyway
+    assert kernels.decode_share_plan([100, 4000] * 16, 8, 4096, block_size=8)[1] == 0     # the other kernel
+    planned = 0
+    for S, kvh, ctx in ((32, 8, 4096), (64, 8, 4096), (16, 8, 4096), (40, 4, 16384), (24, 8, 2048)):
+        for i in range(20):
+            lens = [rng.randint(20, ctx) for _ in range(S)] if i % 2 else [ctx] * 2 + [rng.randint(20, ctx // 6) for _ in range(S - 2)]
+            shares, length = kernels.decode_share_plan(lens, kvh, ctx)
+            equal = kernels.decode_splits(S, kvh, ctx)
+            if length == 0:
+                assert shares == equal
+                continue
+            tiles = [(n - 1) // 32 + 1 for n in lens]
+            planned += 1
+            assert shares >= equal and shares * length >= max(tiles) and length >= 4
+            assert kvh * sum(-(-t // length) for t in tiles) <= (768 if S * kvh <= 256 else 1024)
+            assert 2 * length <= -(-max(tiles) // equal) and equal <= 3
+    assert planned >= 20
+    # a window bounds what a sequence shows: sequences far longer than the window are all of one length
+    assert kernels.decode_share_plan([300, 4000] * 16, 8, 4096, window=256)[1] == 0

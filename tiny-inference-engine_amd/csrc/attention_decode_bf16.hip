@@ -287,11 +287,16 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
-    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit, QkSource src) {
+    int block_shift, int max_blocks, float scale_log2e, int window, int nsplit, const int* __restrict__ share_tiles,
+    QkSource src) {
   const int lane = threadIdx.x;
   const int col = lane & 15;
   const int quad = lane >> 4;
-  const int split = blockIdx.x;
+  // Workgroups go to the eight XCDs in turn by their number, of which the share is the fastest part: with shares
+  // of one length, where the later shares of most sequences are empty, share j is therefore given to another
+  // workgroup of the sequence's eight from pair to pair, or a few XCDs would carry all the work.
+  const int split = share_tiles != nullptr ? static_cast<int>((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x)
+                                           : static_cast<int>(blockIdx.x);
   const int kvh = blockIdx.y;
   const int s = seq_ids ? seq_ids[blockIdx.z] : blockIdx.z;
   const int G = H / KVH;
@@ -302,9 +307,23 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 
   const int first_tile = start / 32;
   const int num_tiles = pos / 32 + 1;
-  const int per_split = (num_tiles - first_tile + nsplit - 1) / nsplit;
+  // A share is the nsplit-th part of this sequence's tiles, or, where the step names a length for all shares
+  // (share_tiles, in tiles; sequences of very different lengths), that many tiles if it is more: a short sequence
+  // then fills fewer shares, the others are empty (the merge gives them no weight), and every wave that works
+  // walks about as many keys. Whatever the step names, the shares cover the sequence.
+  int per_split = (num_tiles - first_tile + nsplit - 1) / nsplit;
+  if (share_tiles != nullptr) per_split = max(per_split, *share_tiles);
   const int tile_begin = first_tile + split * per_split;
   const int tile_end = min(num_tiles, tile_begin + per_split);
+  if (share_tiles != nullptr && tile_begin >= tile_end) {
+    // An empty share leaves at once: a maximum of -inf gives it no weight, and the merge does not read the rest.
+    if (quad == 0 && col < G) {
+      const size_t slot = (static_cast<size_t>(blockIdx.z) * H + kvh * G + col) * nsplit + split;
+      part_ml[slot * 2] = -INFINITY;
+      part_ml[slot * 2 + 1] = 0.f;
+    }
+    return;
+  }
 
   const size_t page_stride = static_cast<size_t>(KVH) * block_size * DH;
   const size_t head_off = static_cast<size_t>(kvh) * block_size * DH;
@@ -518,7 +537,8 @@ constexpr bool PREPARE_HEAD_DIM = DH == 32 || DH == 64 || DH == 128 || DH == 256
 static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out,
                          float* part_o, float* part_ml, const int* query_start, const int* context_lens,
                          const int* block_tables, const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
-                         int max_blocks, float scale, int window, int nsplit, int depth, hipStream_t stream) {
+                         int max_blocks, float scale, int window, int nsplit, const int* share_tiles, int depth,
+                         hipStream_t stream) {
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
@@ -529,6 +549,7 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   // a whole sequence.
   if (depth == 0) depth = block_size < 16 ? 1 : (nsplit == 1 ? 4 : 3);
   if (src != nullptr && (depth < 2 || !PREPARE_HEAD_DIM)) return TIE_BAD_ARGUMENT;
+  if (share_tiles != nullptr && (depth < 2 || nsplit == 1)) return TIE_BAD_ARGUMENT;   // the ring kernel's, with a merge
   const dim3 grid(nsplit, KVH, num_seqs);
   const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
@@ -538,9 +559,10 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   {                                                                                                          \
     if (src == nullptr) {                                                                                    \
       attention_decode_ring_kernel<DEPTH, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS,   \
-                                                                                QkSource{});                 \
+                                                                                share_tiles, QkSource{});    \
     } else if constexpr (PREPARE_HEAD_DIM) {                                                                 \
-      attention_decode_ring_kernel<DEPTH, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS, *src); \
+      attention_decode_ring_kernel<DEPTH, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS,    \
+                                                                               share_tiles, *src);           \
     }                                                                                                        \
   }
   if (depth == 4) LAUNCH_RING(4)
@@ -558,15 +580,18 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
 
 // depth: 0 = by the rule, 1 = the kernel that looks its pages up per lane (any page size), 2 to 4 = the ring
 // kernel with that many register sets (pages of 16 positions or more); for tests and sweeps.
+// share_tiles (or null): one int on the device, the tiles of 32 keys of a share where the sequences' lengths differ
+// much (the ring kernel and more than one share only; 0 there means shares by each sequence's own length).
 extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
                                               float* part_o, float* part_ml, const int* query_start,
                                               const int* context_lens, const int* block_tables, const int* seq_ids,
                                               int num_seqs, int H, int KVH, int block_size, int max_blocks,
-                                              float scale, int window, int nsplit, int depth, hipStream_t stream) {
+                                              float scale, int window, int nsplit, const int* share_tiles, int depth,
+                                              hipStream_t stream) {
   return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
                        static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
                        query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
-                       scale, window, nsplit, depth, stream);
+                       scale, window, nsplit, share_tiles, depth, stream);
 }
 
 // The same for a step of single decoded tokens whose queries, newest keys and values still lie in the QKV
@@ -583,8 +608,8 @@ extern "C" int tie_attention_decode_prepared_bf16(const float* qkv, long plane_s
                                                   void* out, float* part_o, float* part_ml, const int* query_start,
                                                   const int* context_lens, const int* block_tables,
                                                   const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
-                                                  int max_blocks, float scale, int window, int nsplit, int depth,
-                                                  hipStream_t stream) {
+                                                  int max_blocks, float scale, int window, int nsplit,
+                                                  const int* share_tiles, int depth, hipStream_t stream) {
   if (qkv == nullptr || angles == nullptr || planes < 1 || planes > 8 || plane_stride < 0 || block_size < 16 ||
       depth == 1 || H <= 0 || KVH <= 0 || in_row < (H + 2 * KVH) * DH || in_row % 4 != 0 || plane_stride % 4 != 0 ||
       reinterpret_cast<uintptr_t>(qkv) % 16 != 0 || reinterpret_cast<uintptr_t>(angles) % 16 != 0 ||
@@ -594,7 +619,7 @@ extern "C" int tie_attention_decode_prepared_bf16(const float* qkv, long plane_s
   const QkSource src = {qkv, static_cast<size_t>(plane_stride), planes, in_row, q_weight, k_weight, eps, angles, write_kv};
   return launch_decode(nullptr, &src, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache),
                        static_cast<bf16_t*>(out), part_o, part_ml, query_start, context_lens, block_tables, seq_ids,
-                       num_seqs, H, KVH, block_size, max_blocks, scale, window, nsplit, depth, stream);
+                       num_seqs, H, KVH, block_size, max_blocks, scale, window, nsplit, share_tiles, depth, stream);
 }
 
 extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
@@ -604,5 +629,5 @@ extern "C" int tie_attention_decode_bf16(const void* q, const void* k_cache, con
                                          int window, int nsplit, hipStream_t stream) {
   return tie_attention_decode_bf16_with(q, k_cache, v_cache, out, part_o, part_ml, query_start, context_lens,
                                         block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale, window,
-                                        nsplit, 0, stream);
+                                        nsplit, nullptr, 0, stream);
 }

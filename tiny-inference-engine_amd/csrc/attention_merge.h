@@ -38,7 +38,12 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
   for (int d = threadIdx.x; d < DH; d += blockDim.x) {
     float o = 0.f;
 #pragma unroll 8
-    for (int k = 0; k < nsplit; ++k) o += part_o[(slot0 + k) * DH + d] * weight[k];   // an empty split wrote zeros
+    for (int k = 0; k < nsplit; ++k) {
+      // every load is asked for whatever the weight (they are in flight together); a split without weight is
+      // empty and may have written nothing, so what came back for it is not used
+      const float p = part_o[(slot0 + k) * DH + d];
+      o += (weight[k] != 0.f ? p : 0.f) * weight[k];
+    }
     out[(static_cast<size_t>(t) * H + h) * DH + d] = float_to_bf16(o / L);
   }
 }
@@ -87,9 +92,9 @@ __global__ __launch_bounds__(MERGE_WAVES* TIE_WAVE) void attention_merge_wave_ke
 #pragma unroll 8
     for (int k = 0; k < nsplit; ++k) {
       const float w = __shfl(wi, k, TIE_WAVE);
-      const float2 p = *reinterpret_cast<const float2*>(po + static_cast<size_t>(k) * DH + dr);   // an empty split wrote zeros
-      o0 += p.x * w;
-      o1 += p.y * w;
+      const float2 p = *reinterpret_cast<const float2*>(po + static_cast<size_t>(k) * DH + dr);
+      o0 += (w != 0.f ? p.x : 0.f) * w;   // a split without weight is empty and may have written nothing
+      o1 += (w != 0.f ? p.y : 0.f) * w;
     }
     if (d < DH) *reinterpret_cast<uint32_t*>(o + d) = pack_bf16x2(o0 / L, o1 / L);
   }

@@ -23,6 +23,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
+from .. import kernels
 from ..cache.manager import CacheManager, RequestCache
 from ..errors import CapacityError, InvalidArgument
 
@@ -44,6 +45,9 @@ class GroupStep:
         self.slot_mapping = slot_mapping     # int32 [T]
         self.block_tables = block_tables     # int32 [S, max_blocks_per_seq]
         self.extra: Dict[str, torch.Tensor] = {}
+        # a step of single tokens over sequences of very different lengths: (shares, their length in tiles of 32
+        # keys as one int32 on the device) for the decode attention kernel; None: the rule by the step's size
+        self.key_shares = None
 
 
 class StepBatch:
@@ -63,6 +67,7 @@ class StepBatch:
         self.host_state_slots: List[int] = []
         self.max_context = 0
         self.plan_context = 0      # the context length kernels size their grids for (>= max_context)
+        self.share_key = ()        # the shares planned per cache group, where a recorded step depends on them
         self.max_new_tokens = 0
         self.all_decode = False
         self.memo: Dict = {}       # per-step values kernels derive once and share between layers
@@ -247,6 +252,8 @@ class BatchBuilder:
             offset += _align(T)
             layout[("tables", g)] = (offset, S * MB)
             offset += _align(S * MB)
+            layout[("share_tiles", g)] = (offset, 1)
+            offset += _align(1)
         host_t, dev_t = self._buffers(offset)
         host = host_t.numpy()
 
@@ -259,6 +266,17 @@ class BatchBuilder:
             self._fill_decode(entries, view, batch)
         else:
             self._fill_general(entries, view, batch)
+
+        batch.max_context = max(batch.host_context_lens)
+        batch.plan_context = 1024                 # contexts are planned for in buckets: 1024, 2048, 4096, ...
+        while batch.plan_context < batch.max_context:
+            batch.plan_context *= 2
+        shares = {}
+        for g in groups:
+            need = self.cache.plan.groups[g].need
+            shares[g] = (kernels.decode_share_plan(batch.host_context_lens, need.num_kv_heads, batch.plan_context,
+                                                   self.cache.block_size, need.window) if all_single else (0, 0))
+            view(("share_tiles", g))[0] = shares[g][1]
 
         dev_t[:offset].copy_(host_t[:offset], non_blocking=True)
         if self.device.type == "cuda":
@@ -278,10 +296,9 @@ class BatchBuilder:
         batch.takes_device_tokens = any(e.token_from >= 0 for e in entries)
         for g in groups:
             batch.groups[g] = GroupStep(dev(("slots", g)), dev(("tables", g), (S, MB)))
-        batch.max_context = max(batch.host_context_lens)
-        batch.plan_context = 1024                 # contexts are planned for in buckets: 1024, 2048, 4096, ...
-        while batch.plan_context < batch.max_context:
-            batch.plan_context *= 2
+            if shares[g][1] > 0:
+                batch.groups[g].key_shares = (shares[g][0], dev(("share_tiles", g)))
+        batch.share_key = tuple(shares[g][0] if shares[g][1] > 0 else 0 for g in groups)
         batch.max_new_tokens = max(batch.host_new_tokens)
         batch.all_decode = batch.max_new_tokens == 1
         return batch

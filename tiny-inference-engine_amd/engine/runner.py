@@ -58,7 +58,7 @@ class ModelRunner:
         # bake them into the recording (see Part.capturable). ``use_graphs`` can only switch it off.
         wanted = (model.mode == BFLOAT16) if use_graphs is None else bool(use_graphs)
         self.use_graphs = wanted and self.device.type == "cuda" and model.capturable()
-        self._recorded: Dict[Tuple[int, int, int], _RecordedStep] = {}
+        self._recorded: Dict[Tuple, _RecordedStep] = {}
         self.graph_replays = 0
 
     def _forward(self, batch: StepBatch) -> Optional[torch.Tensor]:
@@ -95,7 +95,7 @@ class ModelRunner:
             return self._forward(batch)
 
         # A decode-only step: replay its recording, or run it eagerly once and record it for next time.
-        key = (batch.num_seqs, batch.num_logit_rows, batch.plan_context)
+        key = (batch.num_seqs, batch.num_logit_rows, batch.plan_context, batch.share_key)
         staging_ptr = self.builder.staging_ptr
         recorded = self._recorded.get(key)
         if recorded is not None and recorded.staging_ptr == staging_ptr and \

@@ -144,10 +144,10 @@ _SIGNATURES = {
         "tie_attention_decode_prepared_bf16": [_c_void, _c_long, _c_int, _c_int, _c_void, _c_void, _c_float, _c_void,
                                                _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                                _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                               _c_int, _c_int, _c_int, _c_void],
+                                               _c_int, _c_int, _c_void, _c_int, _c_void],
         "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                            _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                                           _c_int, _c_int, _c_void],
+                                           _c_int, _c_void, _c_int, _c_void],
     },
 }
 
@@ -1042,6 +1042,69 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int, block_size
     return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
 
 
+# Shares of one length for all sequences (``decode_share_plan``) are planned where each sequence's own shares
+# would be this few at most: with more of them the waves are many and short whatever the lengths (16 sequences of
+# 8 KV heads in 4 shares each: 38.0 us a layer, with shares of one length 40.3).
+BALANCED_SHARES_MAX_EQUAL = 3
+BALANCED_SHARES_GRID = 8          # shares a sequence may be cut into then (the grid; most of them may stay empty)
+
+
+def decode_share_plan(context_lens, num_kv_heads: int, plan_context: int, block_size: int = 16,
+                      window: Optional[int] = None) -> "tuple":
+    """``(shares, share_tiles)`` for a step of single decoded tokens over sequences of these lengths.
+
+    ``share_tiles`` = 0: every sequence's keys go into ``shares`` equal parts of its own (``decode_splits``): the
+    rule for sequences of about one length. A wave walks its share tile after tile, so the longest share sets
+    the kernel's time, and with sequences of very different lengths (the longest a quarter above the mean) that
+    is the longest sequence's, while the waves of the short ones are done early (32 sequences of 8 KV heads, 65 k
+    keys in all: 51 us a layer with 2048 each, 79 with 100 to 4000, 87 with a quarter of them 4096 long; 2 of 4096
+    beside 30 of 600: 83 for 26 k keys). Then, where the shares are few, all shares get ONE length, ``share_tiles``
+    tiles of 32 keys: the smallest for which the waves that have keys at all stay within 768 (1024 above 256
+    (sequence, KV head) pairs), with up to ``BALANCED_SHARES_GRID`` shares a sequence. A short sequence fills one
+    share, a long one several, and the others are empty (those three steps: 68, 62 and 43 us; 64 sequences, 2 of
+    them long: 94 -> 53). Taken only if the longest share gets half as long: between that and equal the merge and
+    the empty shares cost what the balance gains (56 sequences, a quarter long: 94 -> 109 us at two thirds).
+    """
+    S = len(context_lens)
+    equal = decode_splits(S, num_kv_heads, plan_context, block_size)
+    if block_size < 16 or S < 2 or equal > BALANCED_SHARES_MAX_EQUAL:
+        return equal, 0
+    tiles = []
+    for n in context_lens:
+        pos = n - 1
+        first = max(0, pos - window + 1) // 32 if window else 0
+        tiles.append(pos // 32 + 1 - first)
+    longest = max(tiles)
+    if longest * S < 1.25 * sum(tiles):
+        return equal, 0
+    pairs = S * num_kv_heads
+    target = (768 if pairs <= 256 else 1024) // num_kv_heads      # waves with keys, a KV head
+    grid = min(max(BALANCED_SHARES_GRID, equal), MAX_KEY_SPLITS)
+    if target <= S or grid < 2:
+        return equal, 0
+    lo, hi = max(4, -(-longest // grid)), longest                # a share of at least 128 keys that covers the longest
+    if lo >= hi:
+        return equal, 0
+    while lo < hi:                                               # the count of waves falls as the shares grow
+        mid = (lo + hi) // 2
+        if sum(-(-t // mid) for t in tiles) <= target:
+            hi = mid
+        else:
+            lo = mid + 1
+    if 2 * lo > -(-longest // equal):
+        return equal, 0
+    return grid, lo
+
+
+def step_key_shares(step, num_seqs: int, num_kv_heads: int, plan_context: int, block_size: int) -> "tuple":
+    """``(shares, share_tiles tensor or None)`` of a decode step: what the step's builder planned for this cache
+    group (``key_shares`` of the group's view of the step), else the rule by the step's size alone."""
+    planned = getattr(step, "key_shares", None)
+    if planned is not None:
+        return planned
+    return decode_splits(num_seqs, num_kv_heads, plan_context, block_size), None
+
+
 def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
     """Refuses, when a model is built, head geometries that no attention kernel here takes."""
     if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
@@ -1055,8 +1118,13 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                           num_seqs: int, num_heads: int, scale: float, window: Optional[int], nsplit: int,
                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
-                          seq_ids: Optional[torch.Tensor] = None, depth: int = 0) -> None:
+                          seq_ids: Optional[torch.Tensor] = None, depth: int = 0,
+                          share_tiles: Optional[torch.Tensor] = None) -> None:
     """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all).
+
+    ``share_tiles`` (one int32 on the device, or None): the length of every share in tiles of 32 keys, for steps
+    whose sequences differ much in length (``decode_share_plan``); with pages of 16 positions or more and more than
+    one share.
 
     ``depth`` picks the kernel (0: by the library's rule; 1: page lookups per lane, any page size; 2 to 4: that
     many tiles of keys in registers, pages of 16 positions or more); all give the same bits.
@@ -1090,10 +1158,14 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     lib = _lib("attention_decode_bf16", Dh)
     if not 0 <= depth <= 4 or (depth > 1 and bs < 16):
         raise InvalidArgument(f"attention_decode_bf16: depth {depth} with pages of {bs} positions")
+    if share_tiles is not None:
+        _i32(share_tiles, "the shares' length", 1)
+        if nsplit == 1 or bs < 16 or depth == 1:
+            raise InvalidArgument("a length for all shares goes with more than one share and pages of 16 positions or more")
     _call(lib.tie_attention_decode_bf16_with, "attention_decode_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
-        block_tables.shape[1], float(scale), int(window or 0), nsplit, depth, _stream())
+        block_tables.shape[1], float(scale), int(window or 0), nsplit, _ptr(share_tiles), depth, _stream())
 
 
 def decode_attention_prepares(batch, q_dtype: torch.dtype, k_cache: torch.Tensor, num_heads: int) -> bool:
@@ -1135,7 +1207,7 @@ def paged_attention_prepared(planes: torch.Tensor, q_weight: Optional[torch.Tens
     for w, name in ((q_weight, "q norm weight"), (k_weight, "k norm weight")):
         if w is not None:
             _f32(w, name, (Dh,))
-    nsplit = decode_splits(S, KVH, batch.plan_context, bs)
+    nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
     part_o = part_ml = None
     if nsplit > 1:
         part_o = scratch("attention.split_o", (S * H * nsplit * Dh,), torch.float32)
@@ -1144,7 +1216,7 @@ def paged_attention_prepared(planes: torch.Tensor, q_weight: Optional[torch.Tens
           planes.data_ptr(), rows * width, P, width, _ptr(q_weight), _ptr(k_weight), float(eps), angles.data_ptr(),
           int(bool(write_kv)), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
           batch.query_start.data_ptr(), batch.context_lens.data_ptr(), step.block_tables.data_ptr(), None, S, H, KVH,
-          bs, step.block_tables.shape[1], float(scale), int(window or 0), nsplit, 0, _stream())
+          bs, step.block_tables.shape[1], float(scale), int(window or 0), nsplit, _ptr(share_tiles), 0, _stream())
 
 
 def prefill_items(new_tokens, group_size: int) -> "list":
@@ -1252,13 +1324,13 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
-        nsplit = decode_splits(S, KVH, batch.plan_context, bs)
+        nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
         part_o = part_ml = None
         if nsplit > 1:
             part_o = scratch("attention.split_o", (S * num_heads * nsplit * Dh,), torch.float32)
             part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
         attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                              S, num_heads, scale, window, nsplit, part_o, part_ml)
+                              S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles)
         return
     if fast:
         # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
