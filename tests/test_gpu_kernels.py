@@ -670,6 +670,48 @@ def test_attention_decode_bf16_with_shares_of_one_length(H, KVH, Dh, bs, nsplit,
                                       case["tables"], S, H, Dh ** -0.5, window, 1, share_tiles=length)
 
 
+def test_single_rows_beside_a_portion_with_shares_of_one_length(monkeypatch):
+    """A step of a prompt portion and many single decoded rows of very different lengths, through the entry point
+    the attention part calls: the single rows go to the decode kernel with shares of one length (the rule by the
+    step's size bent to two shares a sequence, so that twelve sequences meet the plan), the portion to the prefill
+    kernel; every row against the plain formula."""
+    from tie_amd import kernels
+
+    H, KVH, Dh, bs = 8, 2, 128, 16
+    lens_ctx = [300, 1000, 40, 1000, 90, 33, 64, 700, 17, 130, 257, 50, 31]
+    lens_new = [70] + [1] * 12
+    case, S = attention_case(H, KVH, Dh, bs, lens_new=lens_new, lens_ctx=lens_ctx, seed=23, dtype=torch.bfloat16)
+    monkeypatch.setattr(kernels, "decode_splits", lambda *a, **k: 2)
+    monkeypatch.setattr(kernels, "SINGLE_ROWS_RIDE_ALONG", 0)
+    plans = []
+    real = kernels.decode_share_plan
+
+    def watched(*args, **kwargs):
+        plans.append(real(*args, **kwargs))
+        return plans[-1]
+
+    monkeypatch.setattr(kernels, "decode_share_plan", watched)
+
+    class Batch:
+        all_decode, num_seqs, plan_context, memo = False, S, 1024, {}
+        host_new_tokens, host_context_lens = lens_new, lens_ctx
+        query_start, context_lens, seq_of_row = case["query_start"], case["context_lens"], case["seq_of_row"]
+
+    class Step:
+        block_tables = case["tables"]
+
+    memory = {}
+
+    def scratch(name, shape, dtype):
+        return memory.setdefault((name, tuple(shape), dtype), torch.full(tuple(shape), float("nan"), dtype=dtype, device="cuda"))
+
+    out = torch.full_like(case["q"], float("nan"))
+    for _ in range(2):                                       # the second call takes the step's plan from its memo
+        kernels.paged_attention(case["q"], case["kc"], case["vc"], out, Step, Batch, H, Dh ** -0.5, None, scratch)
+    assert plans == [(8, 4)], plans
+    close(out, case["want"], 1e-2, "a portion beside single rows in shares of one length")
+
+
 @pytest.mark.parametrize("H,KVH,Dh,bs", [(4, 2, 16, 4), (6, 2, 32, 16), (3, 1, 48, 8), (5, 5, 80, 16), (8, 2, 128, 16),
                                          (16, 1, 64, 4), (2, 1, 256, 32)])
 @pytest.mark.parametrize("nsplit", [1, 3, 8])

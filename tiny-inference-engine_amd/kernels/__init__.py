@@ -1357,13 +1357,21 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 torch.tensor(merge_rows, dtype=torch.int32).to(q.device) if items else None)
         seq_ids, num_single, items, num_items, merge_rows = work
         if num_single:
-            nsplit = decode_splits(num_single, KVH, batch.plan_context, bs)
+            shares_key = ("single_row_shares", KVH, window)
+            planned = batch.memo.get(shares_key)
+            if planned is None:                # this step runs eagerly: the shares' length goes to the device by itself
+                lens = [c for c, n in zip(batch.host_context_lens, batch.host_new_tokens) if n == 1]
+                nsplit, length = decode_share_plan(lens, KVH, batch.plan_context, bs, window)
+                planned = batch.memo[shares_key] = (
+                    nsplit, torch.tensor([length], dtype=torch.int32).to(q.device) if length else None)
+            nsplit, share_tiles = planned
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = scratch("attention.split_o", (num_single * num_heads * nsplit * Dh,), torch.float32)
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                                  num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids)
+                                  num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids,
+                                  share_tiles=share_tiles)
         if items is not None and not prefill_loads_straight(Dh, bs) and not prefill_addressable(k_cache):
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
