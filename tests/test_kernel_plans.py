@@ -208,6 +208,8 @@ def test_shares_of_one_length_are_planned_for_sequences_of_very_different_length
     assert kernels.decode_share_plan([2048] * 32, 8, 4096) == (kernels.decode_splits(32, 8, 4096), 0)
     assert kernels.decode_share_plan([4000, 3900, 4096] * 11, 8, 4096)[1] == 0          # about one length
     assert kernels.decode_share_plan([100, 4000], 8, 4096) == (kernels.decode_splits(2, 8, 4096), 0)   # many shares anyway
+    assert kernels.decode_share_plan([32768] + [1024] * 7, 8, 32768) == (64, 21)          # one long sequence among short ones
+    assert kernels.decode_share_plan([32768] * 8, 8, 32768)[1] == 0
     assert kernels.decode_share_plan([100, 4000] * 16, 8, 4096, block_size=8)[1] == 0     # the other kernel
     planned = 0
     for S, kvh, ctx in ((32, 8, 4096), (64, 8, 4096), (16, 8, 4096), (40, 4, 16384), (24, 8, 2048)):
@@ -221,8 +223,9 @@ def test_shares_of_one_length_are_planned_for_sequences_of_very_different_length
             tiles = [(n - 1) // 32 + 1 for n in lens]
             planned += 1
             assert shares >= equal and shares * length >= max(tiles) and length >= 4
-            assert kvh * sum(-(-t // length) for t in tiles) <= (768 if S * kvh <= 256 else 1024)
-            assert 2 * length <= -(-max(tiles) // equal) and equal <= 3
+            assert kvh * sum(-(-t // length) for t in tiles) <= (512 if S * kvh <= 128 else 768 if S * kvh <= 256 else 1024)
+            before = -(-max(tiles) // equal)
+            assert 2 * length <= before if equal <= 3 else 4 * length < before
     assert planned >= 20
     # a window bounds what a sequence shows: sequences far longer than the window are all of one length
     assert kernels.decode_share_plan([300, 4000] * 16, 8, 4096, window=256)[1] == 0

@@ -1042,11 +1042,13 @@ def decode_splits(num_seqs: int, num_kv_heads: int, max_context: int, block_size
     return max(1, min(by_occupancy, by_length, MAX_KEY_SPLITS))
 
 
-# Shares of one length for all sequences (``decode_share_plan``) are planned where each sequence's own shares
-# would be this few at most: with more of them the waves are many and short whatever the lengths (16 sequences of
-# 8 KV heads in 4 shares each: 38.0 us a layer, with shares of one length 40.3).
+# Shares of one length for all sequences (``decode_share_plan``): the grid holds at least this many a sequence.
+BALANCED_SHARES_GRID = 8
+# Where each sequence's own shares would be this few at most, shares of one length are taken if they halve the
+# longest share; with more shares of its own a sequence's waves are short already, and only a share four times
+# shorter pays (16 sequences of 8 KV heads, 100 to 4000 keys, 4 shares each: 37.7 us a layer, shares of one
+# length 36.8 to 44.8; one sequence of 32 k keys beside 23 of 1 k: 176 -> 74).
 BALANCED_SHARES_MAX_EQUAL = 3
-BALANCED_SHARES_GRID = 8          # shares a sequence may be cut into then (the grid; most of them may stay empty)
 
 
 def decode_share_plan(context_lens, num_kv_heads: int, plan_context: int, block_size: int = 16,
@@ -1058,16 +1060,18 @@ def decode_share_plan(context_lens, num_kv_heads: int, plan_context: int, block_
     the kernel's time, and with sequences of very different lengths (the longest a quarter above the mean) that
     is the longest sequence's, while the waves of the short ones are done early (32 sequences of 8 KV heads, 65 k
     keys in all: 51 us a layer with 2048 each, 79 with 100 to 4000, 87 with a quarter of them 4096 long; 2 of 4096
-    beside 30 of 600: 83 for 26 k keys). Then, where the shares are few, all shares get ONE length, ``share_tiles``
-    tiles of 32 keys: the smallest for which the waves that have keys at all stay within 768 (1024 above 256
-    (sequence, KV head) pairs), with up to ``BALANCED_SHARES_GRID`` shares a sequence. A short sequence fills one
-    share, a long one several, and the others are empty (those three steps: 68, 62 and 43 us; 64 sequences, 2 of
-    them long: 94 -> 53). Taken only if the longest share gets half as long: between that and equal the merge and
-    the empty shares cost what the balance gains (56 sequences, a quarter long: 94 -> 109 us at two thirds).
+    beside 30 of 600: 83 for 26 k keys; one of 32 k beside 7 of 1 k: 89, as much as half of 8 of 32 k). Then all
+    shares get ONE length, ``share_tiles`` tiles of 32 keys: the smallest for which the waves that have keys at all
+    stay within 512 (768 above 128 (sequence, KV head) pairs, 1024 above 256). A short sequence fills one share, a long one many,
+    and the rest of the grid (a power of two of shares a sequence, so that a recorded step serves while the lengths
+    grow) is empty (those steps: 68, 62, 43 and 52 us; 64 sequences, 2 of them long: 94 -> 53). Taken only if the
+    longest share gets half as long, a quarter where a sequence's own shares are more than three: between that
+    and equal the merge and the empty shares cost what the balance gains (56 sequences, a quarter long: 94 -> 109
+    us at two thirds; two of 16 k beside six of 2 k: 56 -> 57 at a third).
     """
     S = len(context_lens)
     equal = decode_splits(S, num_kv_heads, plan_context, block_size)
-    if block_size < 16 or S < 2 or equal > BALANCED_SHARES_MAX_EQUAL:
+    if block_size < 16 or S < 2 or BALANCED_SHARES_MAX_EQUAL <= 0:
         return equal, 0
     tiles = []
     for n in context_lens:
@@ -1078,21 +1082,22 @@ def decode_share_plan(context_lens, num_kv_heads: int, plan_context: int, block_
     if longest * S < 1.25 * sum(tiles):
         return equal, 0
     pairs = S * num_kv_heads
-    target = (768 if pairs <= 256 else 1024) // num_kv_heads      # waves with keys, a KV head
-    grid = min(max(BALANCED_SHARES_GRID, equal), MAX_KEY_SPLITS)
-    if target <= S or grid < 2:
+    target = (512 if pairs <= 128 else 768 if pairs <= 256 else 1024) // num_kv_heads      # waves with keys, a KV head
+    if target <= S:
         return equal, 0
-    lo, hi = max(4, -(-longest // grid)), longest                # a share of at least 128 keys that covers the longest
-    if lo >= hi:
-        return equal, 0
+    lo, hi = max(4, -(-longest // MAX_KEY_SPLITS)), longest      # a share of at least 128 keys, the longest within the grid
     while lo < hi:                                               # the count of waves falls as the shares grow
         mid = (lo + hi) // 2
         if sum(-(-t // mid) for t in tiles) <= target:
             hi = mid
         else:
             lo = mid + 1
-    if 2 * lo > -(-longest // equal):
+    before = -(-longest // equal)
+    if (2 * lo > before) if equal <= BALANCED_SHARES_MAX_EQUAL else (4 * lo >= before):
         return equal, 0
+    grid = BALANCED_SHARES_GRID
+    while grid * lo < longest:
+        grid *= 2
     return grid, lo
 
 
