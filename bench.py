@@ -156,10 +156,13 @@ def measure_long_prompt(model, cfg, args):
     return best
 
 
-def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True):
+def make_engine(model, batch, context, max_tokens_per_step, launch_ahead=True, long_sequences=0, short_context=0):
     from tie_amd.api import create_engine
 
     blocks = batch * (-(-context // BLOCK_SIZE) + 1) + 8
+    if 0 < long_sequences < batch:
+        blocks = (long_sequences * (-(-context // BLOCK_SIZE) + 1) +
+                  (batch - long_sequences) * (-(-short_context // BLOCK_SIZE) + 1) + 8)
     return create_engine(model, kv_blocks=blocks, block_size=BLOCK_SIZE, max_seqs=max(batch, 1),
                          max_tokens_per_step=max(max_tokens_per_step, batch), policy="fcfs", watermark_blocks=0,
                          max_seq_len=context, launch_ahead=launch_ahead)
@@ -183,7 +186,7 @@ def measure_decode(model, cfg, batch, context, steps, warmup, chunk, sampling=No
     from tie_amd.engine.sequence import SeqState
     from tie_amd.sampling.params import SamplingParams
 
-    engine = make_engine(model, batch, context, chunk)
+    engine = make_engine(model, batch, context, chunk, long_sequences=long_sequences, short_context=short_context)
     rng = random.Random(batch)
     slack = -(-batch * context // chunk) + batch + 2          # steps the prefill phase may take
     prompt_len = context - (steps + warmup) - slack - 1
