@@ -1359,8 +1359,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             work = batch.memo[key] = (
                 torch.tensor(single, dtype=torch.int32).to(q.device) if single else None, len(single),
                 torch.tensor(items, dtype=torch.int32).to(q.device) if items else None, len(items),
-                torch.tensor(merge_rows, dtype=torch.int32).to(q.device) if items else None)
-        seq_ids, num_single, items, num_items, merge_rows = work
+                torch.tensor(merge_rows, dtype=torch.int32).to(q.device) if items else None,
+                max((batch.host_context_lens[it[0]] for it in items), default=0))
+        seq_ids, num_single, items, num_items, merge_rows, items_context = work
         if num_single:
             shares_key = ("single_row_shares", KVH, window)
             planned = batch.memo.get(shares_key)
@@ -1385,7 +1386,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             return
         if items is not None:
             rows = q.shape[0]
-            nsplit = prefill_splits(num_items, KVH, G, batch.plan_context, rows)
+            # by the longest context among the portions themselves: a single row of 32 k keys beside them says nothing
+            # about how many tiles a portion's share would hold
+            nsplit = prefill_splits(num_items, KVH, G, items_context, rows)
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = scratch("attention.prefill_split_o", (rows * num_heads * nsplit * Dh,), torch.float32)
