@@ -103,7 +103,10 @@ def measure_stress(model, cfg, args):
     engine = create_engine(model, kv_mem=args.kv_mem, block_size=BLOCK_SIZE, max_seqs=args.requests,
                            max_tokens_per_step=args.portion, prefill_chunk=args.portion, launch_ahead=args.launch_ahead,
                            admit_whole=args.admit_whole)
-    requests = synthetic_requests(args.requests, (128, 2048), (256, 256), cfg["vocab_size"], seed=0)
+    from tie_amd.bench.workload import parse_range
+
+    requests = synthetic_requests(args.requests, parse_range("--prompt-len", args.prompt_len),
+                                  parse_range("--output-len", args.output_len), cfg["vocab_size"], seed=0)
     assign_arrivals(requests, float("inf"), seed=0)
     warm = synthetic_requests(4, (600, 700), (8, 8), cfg["vocab_size"], seed=1)       # compiles nothing, but warms up
     run_workload(engine, warm)
@@ -274,6 +277,8 @@ def main():
     parser.add_argument("--portion", type=int, default=512, help="long-prompt and stress: tokens of a prompt portion (stress: also the token budget of a step)")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
     parser.add_argument("--kv-mem", type=int, default=2 << 30, help="stress: bytes of cache")
+    parser.add_argument("--prompt-len", default="128:2048", help="stress: prompt lengths A:B")
+    parser.add_argument("--output-len", default="256", help="stress: generated tokens C or C:D")
     parser.add_argument("--admit-whole", action="store_true",
                         help="stress: a request enters when the pool can hold all of its prompt, not just its first portion")
     parser.add_argument("--launch-ahead", type=int, default=1,
@@ -324,8 +329,8 @@ def main():
             "value": round(report["total_tok_per_s"], 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
             "dtype": "bf16", "data": "synthetic",
             "config": {"model": f"{shape_name} shape, random weights", "layers": layers_of_shape,
-                       "layers_run": cfg["num_hidden_layers"], "requests": args.requests, "prompt_len": "128:2048",
-                       "output_len": 256, "prefill_chunk": args.portion, "max_tokens_per_step": args.portion, "kv_bytes": args.kv_mem,
+                       "layers_run": cfg["num_hidden_layers"], "requests": args.requests, "prompt_len": args.prompt_len,
+                       "output_len": args.output_len, "prefill_chunk": args.portion, "max_tokens_per_step": args.portion, "kv_bytes": args.kv_mem,
                        "kv_block": BLOCK_SIZE, "policy": "srpt-aging", "admit_whole": int(args.admit_whole), "sampling": "greedy",
                        "launch_ahead": args.launch_ahead},
             "report": report}), flush=True)

@@ -18,6 +18,7 @@ All arrays travel to the device in one copy from one pinned staging buffer.
 from __future__ import annotations
 
 import dataclasses
+import itertools
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -194,45 +195,43 @@ class BatchBuilder:
         batch.host_state_slots = slots
 
     def _fill_general(self, entries, view, batch: StepBatch) -> None:
+        """Entries of any length: the rows of all of them are laid out as whole vectors (a step of many decoded
+        tokens beside a few prompts costs the host little more than a step of decoded tokens alone)."""
         bs, MB = self.cache.block_size, self.max_blocks_per_seq
-        groups = self.cache.plan.paged_groups
-        tokens, positions, seq_of_row = view("tokens"), view("positions"), view("seq_of_row")
-        token_sources = view("token_sources")
-        query_start, context_lens = view("query_start"), view("context_lens")
-        state_slots, logit_rows = view("state_slots"), view("logit_rows")
-        slot_views = [view(("slots", g)) for g in groups]
-        table_views = [view(("tables", g)) for g in groups]
-        row = r = 0
-        query_start[0] = 0
-        for s, e in enumerate(entries):
-            n = len(e.tokens)
-            start = e.start
-            ids = np.asarray(e.tokens, dtype=np.int64)
-            if ids.min() < 0 or ids.max() >= self.vocab_size:
-                raise self._bad_token(ids)
-            where = np.arange(start, start + n, dtype=np.int32)
-            tokens[row:row + n] = ids
-            token_sources[row:row + n] = e.token_from
-            positions[row:row + n] = where
-            seq_of_row[row:row + n] = s
-            context_lens[s] = start + n
-            state_slots[s] = max(e.cache.state_slot, 0)
-            for w in e.want:
-                logit_rows[r] = row + w
-                r += 1
-            for gi, g in enumerate(groups):
-                table = self._table_row(e.cache, g, MB)
-                pages = table[where // bs]
-                if pages.min() < 0:
-                    gone = int(where[int(np.argmin(pages))])
-                    raise InvalidArgument(f"position {gone} lies in a page that was already given back")
-                slot_views[gi][row:row + n] = pages * bs + where % bs
-                table_views[gi][s * MB:(s + 1) * MB] = np.maximum(table, 0)     # FREED (-1) -> 0: never read
-            row += n
-            query_start[s + 1] = row
-            batch.host_new_tokens.append(n)
-            batch.host_context_lens.append(start + n)
-            batch.host_state_slots.append(e.cache.state_slot)
+        S = len(entries)
+        counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=S)
+        starts = np.fromiter((e.start for e in entries), dtype=np.int32, count=S)
+        first_row = np.zeros(S + 1, dtype=np.int32)
+        np.cumsum(counts, out=first_row[1:])
+        T = int(first_row[-1])
+        ids = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int64, count=T)
+        if ids.min() < 0 or ids.max() >= self.vocab_size:
+            raise self._bad_token(ids)
+        seq = np.repeat(np.arange(S, dtype=np.int32), counts)
+        where = starts[seq] + (np.arange(T, dtype=np.int32) - first_row[seq])
+        view("tokens")[:] = ids
+        view("token_sources")[:] = np.repeat(np.fromiter((e.token_from for e in entries), dtype=np.int32, count=S), counts)
+        view("positions")[:] = where
+        view("seq_of_row")[:] = seq
+        view("query_start")[:] = first_row
+        view("context_lens")[:] = starts + counts
+        slots = [e.cache.state_slot for e in entries]
+        view("state_slots")[:] = np.maximum(np.asarray(slots, dtype=np.int32), 0)
+        view("logit_rows")[:] = [int(first_row[s]) + w for s, e in enumerate(entries) for w in e.want]
+        page_of_row = where // bs
+        for g in self.cache.plan.paged_groups:
+            tables = view(("tables", g)).reshape(S, MB)
+            for s, e in enumerate(entries):
+                tables[s] = self._table_row(e.cache, g, MB)
+            pages = tables[seq, page_of_row]
+            if pages.min() < 0:
+                gone = int(where[int(np.argmin(pages))])
+                raise InvalidArgument(f"position {gone} lies in a page that was already given back")
+            view(("slots", g))[:] = pages * bs + where % bs
+            np.maximum(tables, 0, out=tables)        # FREED (-1) -> 0: the kernels never read those entries
+        batch.host_new_tokens = counts.tolist()
+        batch.host_context_lens = (starts + counts).tolist()
+        batch.host_state_slots = slots
 
     def build(self, entries: Sequence[StepEntry]) -> StepBatch:
         if not entries:
