@@ -107,7 +107,7 @@ def measure_stress(model, cfg, args):
 
     requests = synthetic_requests(args.requests, parse_range("--prompt-len", args.prompt_len),
                                   parse_range("--output-len", args.output_len), cfg["vocab_size"], seed=0)
-    assign_arrivals(requests, float("inf"), seed=0)
+    assign_arrivals(requests, args.rate, seed=0)
     warm = synthetic_requests(4, (600, 700), (8, 8), cfg["vocab_size"], seed=1)       # compiles nothing, but warms up
     run_workload(engine, warm)
     log(f"stress: {args.requests} requests, {sum(len(r.prompt) for r in requests)} prompt tokens, "
@@ -117,6 +117,7 @@ def measure_stress(model, cfg, args):
     report = report_json(summarize(run))
     report["kv_blocks"] = engine.cache.num_blocks
     report["graph_replays"] = engine.runner.graph_replays
+    report["graphs_recorded"] = len(engine.runner._recorded)
     return report
 
 
@@ -277,6 +278,7 @@ def main():
     parser.add_argument("--portion", type=int, default=512, help="long-prompt and stress: tokens of a prompt portion (stress: also the token budget of a step)")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")
     parser.add_argument("--kv-mem", type=int, default=2 << 30, help="stress: bytes of cache")
+    parser.add_argument("--rate", type=float, default=float("inf"), help="stress: requests a second (Poisson arrivals)")
     parser.add_argument("--prompt-len", default="128:2048", help="stress: prompt lengths A:B")
     parser.add_argument("--output-len", default="256", help="stress: generated tokens C or C:D")
     parser.add_argument("--admit-whole", action="store_true",
